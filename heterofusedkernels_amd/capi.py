@@ -1,0 +1,110 @@
+"""ctypes binding of the C-ABI in include/hfk.h (libhfk_hip.so).
+
+Thin by design: arguments are raw addresses and sizes, exactly what a C caller
+passes. ``check`` turns a non-zero status into ``RuntimeError``. torch is used by
+callers for device memory and streams only; nothing here touches tensors.
+"""
+import ctypes
+import os
+
+from . import _build
+
+_lib = None
+
+KNOB_UNROLL = 0
+KNOB_NONTEMPORAL = 1
+KNOB_WORKGROUPS_PER_CU = 2
+
+ENTRY_POINTS = (
+    "hfk_version",
+    "hfk_status_string",
+    "hfk_gather_rows",
+    "hfk_multi_layer_block_transfer",
+    "hfk_fused_memcpy_multi_layer_block_transfer",
+    "hfk_swap_blocks",
+    "hfk_gather_blocks",
+    "hfk_set_tuning",
+    "hfk_get_tuning",
+)
+
+
+def library_path():
+    return _build.HFK_HIP_SO
+
+
+def load():
+    """Load libhfk_hip.so (built in-tree). Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            "libhfk_hip.so is not built (%s); run `python -m heterofusedkernels_amd._build`" % path
+        )
+    L = ctypes.CDLL(path)
+    vp, u64, u32, ci, i64 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_int, ctypes.c_int64
+    L.hfk_version.argtypes = []
+    L.hfk_version.restype = ci
+    L.hfk_status_string.argtypes = [ci]
+    L.hfk_status_string.restype = ctypes.c_char_p
+    L.hfk_gather_rows.argtypes = [vp, vp, vp, ci, u64, u64, u64, u32, vp]
+    L.hfk_gather_rows.restype = ci
+    L.hfk_multi_layer_block_transfer.argtypes = [vp, vp, u32, u32, u32, u32, u32, u32, vp]
+    L.hfk_multi_layer_block_transfer.restype = ci
+    L.hfk_fused_memcpy_multi_layer_block_transfer.argtypes = [vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
+    L.hfk_fused_memcpy_multi_layer_block_transfer.restype = ci
+    L.hfk_swap_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, u32, vp]
+    L.hfk_swap_blocks.restype = ci
+    L.hfk_gather_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u32, vp]
+    L.hfk_gather_blocks.restype = ci
+    L.hfk_set_tuning.argtypes = [ci, i64]
+    L.hfk_set_tuning.restype = ci
+    L.hfk_get_tuning.argtypes = [ci]
+    L.hfk_get_tuning.restype = i64
+    _lib = L
+    return L
+
+
+def status_string(rc):
+    return load().hfk_status_string(rc).decode()
+
+
+def check(rc, what="hfk call"):
+    if rc != 0:
+        raise RuntimeError("%s failed: %s (%d)" % (what, status_string(rc), rc))
+
+
+def gather_rows(table, dst, ids, ids_are_i64, n_ids, row_bytes, table_rows=0, workgroups=0, stream=0):
+    return load().hfk_gather_rows(table, dst, ids, int(ids_are_i64), n_ids, row_bytes, table_rows, workgroups,
+                                  stream)
+
+
+def multi_layer_block_transfer(layer_ptrs, src, T, L, H, D, elem_bytes, workgroups=0, stream=0):
+    return load().hfk_multi_layer_block_transfer(layer_ptrs, src, T, L, H, D, elem_bytes, workgroups, stream)
+
+
+def fused_memcpy_multi_layer_block_transfer(layer_ptrs, host_block, staging, T, L, H, D, elem_bytes,
+                                            workgroups=0, stream=0):
+    return load().hfk_fused_memcpy_multi_layer_block_transfer(layer_ptrs, host_block, staging, T, L, H, D,
+                                                              elem_bytes, workgroups, stream)
+
+
+def swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, src_stride, dst_stride,
+                src_blocks=0, dst_blocks=0, workgroups=0, stream=0):
+    return load().hfk_swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, src_stride,
+                                  dst_stride, src_blocks, dst_blocks, workgroups, stream)
+
+
+def gather_blocks(dst_planes, src_planes, ids, n_planes, n_ids, block_bytes, src_stride, src_blocks=0,
+                  workgroups=0, stream=0):
+    return load().hfk_gather_blocks(dst_planes, src_planes, ids, n_planes, n_ids, block_bytes, src_stride,
+                                    src_blocks, workgroups, stream)
+
+
+def set_tuning(knob, value):
+    return load().hfk_set_tuning(knob, value)
+
+
+def get_tuning(knob):
+    return load().hfk_get_tuning(knob)

@@ -1,0 +1,289 @@
+// Per-lane bodies of the three data-movement kernels.
+//
+// Each body is an ordinary function of (workgroup index, workgroup count, lane
+// index) and touches memory only through its argument struct, so the same text
+// is compiled twice: by hipcc as the body of a __global__ kernel for gfx950, and
+// by the host compiler inside the CPU index-math checker used by the unit tests
+// (which walks every (workgroup, lane) pair sequentially under a bounds checker).
+// No LDS and no barriers are used: these kernels are pure streaming copies whose
+// lanes never exchange data, so staging through LDS would only add a hop.
+//
+// Access shape: a workgroup is 256 lanes (4 wavefronts of 64). In the fast path
+// every lane moves 16-byte vectors; lane i of a wavefront touches vector i of a
+// 1 KiB contiguous span, so each wavefront instruction is one fully coalesced
+// 1 KiB request. A lane issues UNROLL independent loads before its first store
+// to keep UNROLL * 16 B in flight per lane (what hides PCIe and HBM latency).
+#pragma once
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define HFK_HD __host__ __device__ __forceinline__
+#else
+#define HFK_HD inline
+#endif
+
+// Addresses arrive as integers (plane tables, base + offset arithmetic). A plain
+// cast would give a generic pointer and flat_* instructions; every address these
+// kernels touch is global memory, so say so and get global_load/global_store.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define HFK_GLOBAL __attribute__((address_space(1)))
+#else
+#define HFK_GLOBAL
+#endif
+
+namespace hfk {
+
+constexpr uint32_t kWorkgroupLanes = 256;
+
+typedef uint32_t vec16 __attribute__((ext_vector_type(4)));
+
+// NT bit0: non-temporal loads, bit1: non-temporal stores.
+template <typename V>
+HFK_HD const HFK_GLOBAL V* global_in(uint64_t addr) {
+    return reinterpret_cast<const HFK_GLOBAL V*>(addr);
+}
+
+template <typename V>
+HFK_HD HFK_GLOBAL V* global_out(uint64_t addr) {
+    return reinterpret_cast<HFK_GLOBAL V*>(addr);
+}
+
+template <int NT, typename V>
+HFK_HD V load_unit(const HFK_GLOBAL V* p) {
+    if constexpr ((NT & 1) != 0) {
+        return __builtin_nontemporal_load(p);
+    } else {
+        return *p;
+    }
+}
+
+template <int NT, typename V>
+HFK_HD void store_unit(HFK_GLOBAL V* p, V v) {
+    if constexpr ((NT & 2) != 0) {
+        __builtin_nontemporal_store(v, p);
+    } else {
+        *p = v;
+    }
+}
+
+// Byte k of a unit, without taking the address of a register value.
+HFK_HD uint8_t unit_byte(uint8_t v, uint32_t) { return v; }
+HFK_HD uint8_t unit_byte(uint32_t v, uint32_t k) { return (uint8_t)(v >> (8u * k)); }
+HFK_HD uint8_t unit_byte(vec16 v, uint32_t k) {
+    const uint32_t word = (k < 4) ? v.x : (k < 8) ? v.y : (k < 12) ? v.z : v.w;
+    return (uint8_t)(word >> (8u * (k & 3u)));
+}
+
+// ---------------------------------------------------------------------------
+// Block copy: tiles (plane, pair) of block_bytes bytes, each cut into chunks of
+// 256 * UNROLL vectors; one workgroup iteration moves one chunk.
+// Serves the block-table swap (both directions), the multi-plane block gather
+// and the wide-row case of the row gather.
+// ---------------------------------------------------------------------------
+template <typename IdT>
+struct BlockCopyArgs {
+    const uint64_t* dst_planes;  // device array of plane base addresses, or null -> dst_base
+    const uint64_t* src_planes;  // device array of plane base addresses, or null -> src_base
+    uint64_t dst_base;
+    uint64_t src_base;
+    const IdT* src_ids;          // entry j at src_ids[j * id_stride]
+    const IdT* dst_ids;          // entry j at dst_ids[j * id_stride]; null -> dst block j
+    uint32_t id_stride;
+    uint32_t n_planes;
+    uint32_t n_pairs;
+    uint32_t chunks_per_block;
+    uint64_t block_bytes;
+    uint64_t src_stride;
+    uint64_t dst_stride;
+    uint64_t src_limit;          // block indices must be < limit (unsigned compare,
+    uint64_t dst_limit;          // so negative ids are rejected as well)
+    uint32_t n_work;             // n_planes * n_pairs * chunks_per_block
+};
+
+template <typename IdT, int UNROLL, int NT>
+HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+    constexpr uint32_t kChunkVecs = kWorkgroupLanes * UNROLL;
+    constexpr uint64_t kChunkBytes = (uint64_t)kChunkVecs * 16u;
+
+    for (uint32_t w = bid; w < a.n_work; w += nb) {
+        // Uniform over the workgroup: the compiler keeps these in scalar registers.
+        const uint32_t chunk = w % a.chunks_per_block;
+        const uint32_t tile = w / a.chunks_per_block;
+        const uint32_t pair = tile % a.n_pairs;
+        const uint32_t plane = tile / a.n_pairs;
+
+        const uint64_t sb = (uint64_t)(int64_t)a.src_ids[(uint64_t)pair * a.id_stride];
+        const uint64_t db = a.dst_ids ? (uint64_t)(int64_t)a.dst_ids[(uint64_t)pair * a.id_stride]
+                                      : (uint64_t)pair;
+        if (sb >= a.src_limit || db >= a.dst_limit) {
+            continue;
+        }
+        const uint64_t s_addr = (a.src_planes ? a.src_planes[plane] : a.src_base) + sb * a.src_stride;
+        const uint64_t d_addr = (a.dst_planes ? a.dst_planes[plane] : a.dst_base) + db * a.dst_stride;
+
+        if (((s_addr | d_addr | a.block_bytes) & 15u) == 0) {
+            const uint64_t block_vecs = a.block_bytes >> 4;
+            const uint64_t first = (uint64_t)chunk * kChunkVecs;
+            const HFK_GLOBAL vec16* sv = global_in<vec16>(s_addr) + first + tid;
+            HFK_GLOBAL vec16* dv = global_out<vec16>(d_addr) + first + tid;
+            vec16 v[UNROLL];
+            if (first + kChunkVecs <= block_vecs) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
+                }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
+                }
+            } else {
+                const uint64_t lane_first = first + tid;
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
+                        v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
+                        store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
+                    }
+                }
+            }
+        } else {
+            // Blocks that are not 16-byte aligned/sized: same chunk, narrower units.
+            const uint64_t lo = (uint64_t)chunk * kChunkBytes;
+            const uint64_t hi = (lo + kChunkBytes < a.block_bytes) ? lo + kChunkBytes : a.block_bytes;
+            if (((s_addr | d_addr | a.block_bytes) & 3u) == 0) {
+                const HFK_GLOBAL uint32_t* s4 = global_in<uint32_t>(s_addr);
+                HFK_GLOBAL uint32_t* d4 = global_out<uint32_t>(d_addr);
+                for (uint64_t o = (lo >> 2) + tid; o < (hi >> 2); o += kWorkgroupLanes) {
+                    d4[o] = s4[o];
+                }
+            } else {
+                const HFK_GLOBAL uint8_t* s1 = global_in<uint8_t>(s_addr);
+                HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(d_addr);
+                for (uint64_t o = lo + tid; o < hi; o += kWorkgroupLanes) {
+                    d1[o] = s1[o];
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Flat row gather for narrow rows (below one chunk): the destination is one
+// contiguous array of n_ids * row_units units of type V; lane g of the flat
+// index space copies unit (g % row_units) of row ids[g / row_units].
+// Consecutive lanes read consecutive units of a row, so a 1 KiB row is exactly
+// one wavefront request and shorter rows share a wavefront.
+// ---------------------------------------------------------------------------
+template <typename IdT>
+struct FlatGatherArgs {
+    uint64_t table;       // address; row r at table + r * row_units * sizeof(V)
+    uint64_t dst;
+    const IdT* ids;
+    uint64_t total_units; // n_ids * row_units
+    uint32_t row_units;
+    uint64_t row_limit;   // ids must be < limit (unsigned compare)
+    uint32_t n_work;      // ceil(total_units / (256 * UNROLL))
+};
+
+template <typename V, typename IdT, typename IndexT, int UNROLL, int NT>
+HFK_HD void flat_gather_body(const FlatGatherArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+    constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
+    const HFK_GLOBAL V* table = global_in<V>(a.table);
+    HFK_GLOBAL V* dst = global_out<V>(a.dst);
+    const IndexT total = (IndexT)a.total_units;
+    const IndexT row_units = (IndexT)a.row_units;
+
+    for (uint32_t w = bid; w < a.n_work; w += nb) {
+        const IndexT g0 = (IndexT)w * kChunkUnits + tid;
+        V v[UNROLL];
+        bool ok[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const IndexT g = g0 + (IndexT)u * kWorkgroupLanes;
+            ok[u] = false;
+            if (g < total) {
+                const IndexT row = g / row_units;
+                const IndexT col = g - row * row_units;
+                const uint64_t id = (uint64_t)(int64_t)a.ids[row];
+                if (id < a.row_limit) {
+                    ok[u] = true;
+                    v[u] = load_unit<NT>(table + id * a.row_units + col);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (ok[u]) {
+                store_unit<NT>(dst + (uint64_t)(g0 + (IndexT)u * kWorkgroupLanes), v[u]);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Layout-converting transfer of one block: source [T, L, H, row] read in memory
+// order (fully coalesced, which is what the PCIe link wants when the source is
+// host memory), every unit stored to layer l at [(h*T + t), row]. A source row
+// (D * elem_bytes bytes) stays contiguous, so stores land in row-sized runs.
+// ---------------------------------------------------------------------------
+struct TransposeArgs {
+    const uint64_t* layer_ptrs;  // device array of L destination addresses
+    uint64_t src;                // address of the [T, L, H, row] block
+    uint32_t T;
+    uint32_t L;
+    uint32_t H;
+    uint32_t row_units;          // D * elem_bytes / sizeof(V)
+    uint32_t total_units;        // T * L * H * row_units
+    uint32_t n_work;             // ceil(total_units / (256 * UNROLL))
+};
+
+template <typename V, int UNROLL, int NT>
+HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+    constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
+    const HFK_GLOBAL V* src = global_in<V>(a.src);
+    const uint32_t LH = a.L * a.H;
+
+    for (uint32_t w = bid; w < a.n_work; w += nb) {
+        const uint64_t g0 = (uint64_t)w * kChunkUnits + tid;
+        V v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint64_t g = g0 + (uint64_t)u * kWorkgroupLanes;
+            if (g < a.total_units) {
+                v[u] = load_unit<NT>(src + g);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint64_t g64 = g0 + (uint64_t)u * kWorkgroupLanes;
+            if (g64 < a.total_units) {
+                const uint32_t g = (uint32_t)g64;
+                const uint32_t r = g / a.row_units;      // source row = (t*L + l)*H + h
+                const uint32_t col = g - r * a.row_units;
+                const uint32_t t = r / LH;
+                const uint32_t lh = r - t * LH;
+                const uint32_t l = lh / a.H;
+                const uint32_t h = lh - l * a.H;
+                const uint64_t unit = ((uint64_t)h * a.T + t) * a.row_units + col;
+                const uint64_t d_addr = a.layer_ptrs[l] + unit * sizeof(V);
+                if ((d_addr & (sizeof(V) - 1)) == 0) {
+                    store_unit<NT>(global_out<V>(d_addr), v[u]);
+                } else {
+                    // Layer buffer not aligned to the unit: byte stores keep it correct.
+                    HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(d_addr);
+                    for (uint32_t k = 0; k < sizeof(V); ++k) {
+                        d1[k] = unit_byte(v[u], k);
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace hfk

@@ -1,0 +1,298 @@
+// libhfk_hip.so: gfx950 kernels and the extern "C" entry points of include/hfk.h.
+//
+// Launch shape: grids are 1-D, workgroups of 256 lanes, each workgroup walking
+// work items bid, bid + grid, ... (a grid-stride loop with a hard upper bound, so
+// every wave terminates). The grid is capped at CUs * workgroups-per-CU, which on
+// MI355X (256 CUs, 8 XCDs) both fills every XCD evenly -- workgroups are handed
+// to XCDs round-robin, and a work item's neighbours bid+-1 sit on other XCDs while
+// the item itself streams one contiguous span, so no XCD's L2 sees another's lines
+// -- and lets a caller shrink the footprint (the `workgroups` argument) when the
+// copy should overlap with compute.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdint>
+
+#include "hfk.h"
+#include "hfk_bodies.h"
+#include "hfk_plan.h"
+
+namespace {
+
+using hfk::BlockCopyArgs;
+using hfk::FlatGatherArgs;
+using hfk::TransposeArgs;
+using hfk::kWorkgroupLanes;
+using hfk::vec16;
+
+template <typename IdT, int UNROLL, int NT>
+__global__ __launch_bounds__(256) void block_copy_kernel(const BlockCopyArgs<IdT> a) {
+    hfk::block_copy_body<IdT, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+template <typename V, typename IdT, typename IndexT, int UNROLL, int NT>
+__global__ __launch_bounds__(256) void flat_gather_kernel(const FlatGatherArgs<IdT> a) {
+    hfk::flat_gather_body<V, IdT, IndexT, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+template <typename V, int UNROLL, int NT>
+__global__ __launch_bounds__(256) void transpose_kernel(const TransposeArgs a) {
+    hfk::transpose_body<V, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+// ---- tuning state ---------------------------------------------------------
+std::atomic<int> g_unroll{8};
+std::atomic<int> g_nontemporal{3};
+std::atomic<int> g_wg_per_cu{8};
+
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_cu_count[kMaxDevices];
+
+int current_cu_count(int* out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev >= 0 && dev < kMaxDevices) {
+        int c = g_cu_count[dev].load(std::memory_order_relaxed);
+        if (c > 0) {
+            *out = c;
+            return 0;
+        }
+    }
+    int cus = 0;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return (int)e;
+    if (cus <= 0) cus = 1;
+    if (dev >= 0 && dev < kMaxDevices) g_cu_count[dev].store(cus, std::memory_order_relaxed);
+    *out = cus;
+    return 0;
+}
+
+int pick_grid(uint32_t n_work, uint32_t workgroups, uint32_t* grid) {
+    uint32_t cap = workgroups;
+    if (cap == 0) {
+        int cus = 0;
+        int rc = current_cu_count(&cus);
+        if (rc != 0) return rc;
+        cap = (uint32_t)cus * (uint32_t)g_wg_per_cu.load(std::memory_order_relaxed);
+    }
+    *grid = n_work < cap ? n_work : cap;
+    return 0;
+}
+
+int finish_launch() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? HFK_OK : (int)e;
+}
+
+// ---- block copy -----------------------------------------------------------
+template <typename IdT, int UNROLL>
+void launch_block_copy_nt(const BlockCopyArgs<IdT>& a, uint32_t grid, int nt, hipStream_t s) {
+    switch (nt & 3) {
+        case 0: hipLaunchKernelGGL((block_copy_kernel<IdT, UNROLL, 0>), dim3(grid), dim3(256), 0, s, a); break;
+        case 1: hipLaunchKernelGGL((block_copy_kernel<IdT, UNROLL, 1>), dim3(grid), dim3(256), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((block_copy_kernel<IdT, UNROLL, 2>), dim3(grid), dim3(256), 0, s, a); break;
+        default: hipLaunchKernelGGL((block_copy_kernel<IdT, UNROLL, 3>), dim3(grid), dim3(256), 0, s, a); break;
+    }
+}
+
+template <typename IdT>
+int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s) {
+    int unroll = 1;
+    int rc = hfk::plan_block_copy<IdT>(a, g_unroll.load(std::memory_order_relaxed), &unroll);
+    if (rc != 0) return rc;
+    uint32_t grid = 0;
+    rc = pick_grid(a.n_work, workgroups, &grid);
+    if (rc != 0) return rc;
+    const int nt = g_nontemporal.load(std::memory_order_relaxed);
+    switch (unroll) {
+        case 1: launch_block_copy_nt<IdT, 1>(a, grid, nt, s); break;
+        case 2: launch_block_copy_nt<IdT, 2>(a, grid, nt, s); break;
+        case 4: launch_block_copy_nt<IdT, 4>(a, grid, nt, s); break;
+        case 8: launch_block_copy_nt<IdT, 8>(a, grid, nt, s); break;
+        default: launch_block_copy_nt<IdT, 16>(a, grid, nt, s); break;
+    }
+    return finish_launch();
+}
+
+// ---- flat gather ----------------------------------------------------------
+template <typename V, typename IdT, typename IndexT>
+void launch_flat_gather_v(const FlatGatherArgs<IdT>& a, uint32_t grid, int nt, hipStream_t s) {
+    if (nt & 3) {
+        hipLaunchKernelGGL((flat_gather_kernel<V, IdT, IndexT, hfk::kFlatUnroll, 3>), dim3(grid), dim3(256), 0, s, a);
+    } else {
+        hipLaunchKernelGGL((flat_gather_kernel<V, IdT, IndexT, hfk::kFlatUnroll, 0>), dim3(grid), dim3(256), 0, s, a);
+    }
+}
+
+template <typename IdT>
+int launch_flat_gather(uint64_t table, uint64_t dst, const IdT* ids, uint64_t n_ids, uint64_t row_bytes,
+                       uint64_t row_limit, uint32_t workgroups, hipStream_t s) {
+    FlatGatherArgs<IdT> a;
+    hfk::FlatGatherPlan p;
+    int rc = hfk::plan_flat_gather<IdT>(a, p, table, dst, ids, n_ids, row_bytes, row_limit);
+    if (rc != 0) return rc;
+    uint32_t grid = 0;
+    rc = pick_grid(a.n_work, workgroups, &grid);
+    if (rc != 0) return rc;
+    const int nt = g_nontemporal.load(std::memory_order_relaxed);
+    if (p.unit == 16u) {
+        if (p.index32) launch_flat_gather_v<vec16, IdT, uint32_t>(a, grid, nt, s);
+        else launch_flat_gather_v<vec16, IdT, uint64_t>(a, grid, nt, s);
+    } else if (p.unit == 4u) {
+        if (p.index32) launch_flat_gather_v<uint32_t, IdT, uint32_t>(a, grid, nt, s);
+        else launch_flat_gather_v<uint32_t, IdT, uint64_t>(a, grid, nt, s);
+    } else {
+        if (p.index32) launch_flat_gather_v<uint8_t, IdT, uint32_t>(a, grid, nt, s);
+        else launch_flat_gather_v<uint8_t, IdT, uint64_t>(a, grid, nt, s);
+    }
+    return finish_launch();
+}
+
+template <typename IdT>
+int gather_rows_typed(const void* table, void* dst, const IdT* ids, uint64_t n_ids, uint64_t row_bytes,
+                      uint64_t table_rows, uint32_t workgroups, hipStream_t s) {
+    const uint64_t limit = table_rows ? table_rows : hfk::kUnchecked;
+    if (row_bytes >= hfk::kWideRowBytes) {
+        BlockCopyArgs<IdT> a;
+        int rc = hfk::plan_wide_gather<IdT>(a, table, dst, ids, n_ids, row_bytes, limit);
+        if (rc != 0) return rc;
+        return launch_block_copy<IdT>(a, workgroups, s);
+    }
+    return launch_flat_gather<IdT>((uint64_t)(uintptr_t)table, (uint64_t)(uintptr_t)dst, ids, n_ids, row_bytes,
+                                   limit, workgroups, s);
+}
+
+// ---- transpose ------------------------------------------------------------
+template <typename V>
+void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, hipStream_t s) {
+    if (nt & 3) {
+        hipLaunchKernelGGL((transpose_kernel<V, hfk::kTransposeUnroll, 3>), dim3(grid), dim3(256), 0, s, a);
+    } else {
+        hipLaunchKernelGGL((transpose_kernel<V, hfk::kTransposeUnroll, 0>), dim3(grid), dim3(256), 0, s, a);
+    }
+}
+
+int launch_transpose(const void* dev_layer_ptrs, const void* src, uint32_t T, uint32_t L, uint32_t H,
+                     uint32_t D, uint32_t elem_bytes, uint32_t workgroups, hipStream_t s) {
+    TransposeArgs a;
+    uint32_t unit = 16;
+    int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, src, T, L, H, D, elem_bytes);
+    if (rc != 0) return rc;
+    if (a.n_work == 0) return HFK_OK;  // empty block: nothing to move
+    uint32_t grid = 0;
+    rc = pick_grid(a.n_work, workgroups, &grid);
+    if (rc != 0) return rc;
+    const int nt = g_nontemporal.load(std::memory_order_relaxed);
+    if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, s);
+    else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, s);
+    else launch_transpose_v<uint8_t>(a, grid, nt, s);
+    return finish_launch();
+}
+
+}  // namespace
+
+extern "C" {
+
+int hfk_version(void) { return HFK_VERSION_MAJOR * 1000 + HFK_VERSION_MINOR; }
+
+const char* hfk_status_string(int status) {
+    switch (status) {
+        case HFK_OK: return "ok";
+        case HFK_ERR_NULL_POINTER: return "hfk: required pointer argument is NULL";
+        case HFK_ERR_BAD_SIZE: return "hfk: size or stride is zero or inconsistent";
+        case HFK_ERR_TOO_LARGE: return "hfk: count exceeds what one launch can index";
+        case HFK_ERR_BAD_KNOB: return "hfk: unknown tuning knob or value out of range";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    return "hfk: unknown status";
+}
+
+int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i64, uint64_t n_ids,
+                    uint64_t row_bytes, uint64_t table_rows, uint32_t workgroups, hfk_stream_t stream) {
+    if (n_ids == 0) return HFK_OK;
+    if (table == nullptr || dst == nullptr || ids == nullptr) return HFK_ERR_NULL_POINTER;
+    if (row_bytes == 0) return HFK_ERR_BAD_SIZE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (ids_are_i64) {
+        return gather_rows_typed<int64_t>(table, dst, static_cast<const int64_t*>(ids), n_ids, row_bytes,
+                                          table_rows, workgroups, s);
+    }
+    return gather_rows_typed<int32_t>(table, dst, static_cast<const int32_t*>(ids), n_ids, row_bytes,
+                                      table_rows, workgroups, s);
+}
+
+int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* src_block, uint32_t T,
+                                   uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
+                                   uint32_t workgroups, hfk_stream_t stream) {
+    return launch_transpose(dev_layer_ptrs, src_block, T, L, H, D, elem_bytes, workgroups,
+                            static_cast<hipStream_t>(stream));
+}
+
+int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* host_block,
+                                                void* staging, uint32_t T, uint32_t L, uint32_t H,
+                                                uint32_t D, uint32_t elem_bytes, uint32_t workgroups,
+                                                hfk_stream_t stream) {
+    if (dev_layer_ptrs == nullptr || host_block == nullptr || staging == nullptr) return HFK_ERR_NULL_POINTER;
+    if (elem_bytes == 0) return HFK_ERR_BAD_SIZE;
+    const uint64_t bytes = (uint64_t)T * L * H * D * elem_bytes;
+    if (bytes == 0) return HFK_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = hipMemcpyAsync(staging, host_block, bytes, hipMemcpyHostToDevice, s);
+    if (e != hipSuccess) return (int)e;
+    return launch_transpose(dev_layer_ptrs, staging, T, L, H, D, elem_bytes, workgroups, s);
+}
+
+int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* block_pairs,
+                    uint32_t n_planes, uint64_t n_pairs, uint64_t block_bytes, uint64_t src_block_stride,
+                    uint64_t dst_block_stride, uint64_t src_blocks, uint64_t dst_blocks,
+                    uint32_t workgroups, hfk_stream_t stream) {
+    if (n_planes == 0 || n_pairs == 0) return HFK_OK;
+    BlockCopyArgs<int64_t> a;
+    int rc = hfk::plan_swap_blocks(a, dst_plane_ptrs, src_plane_ptrs, block_pairs, n_planes, n_pairs, block_bytes,
+                                   src_block_stride, dst_block_stride, src_blocks, dst_blocks);
+    if (rc != 0) return rc;
+    return launch_block_copy<int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
+}
+
+int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* ids,
+                      uint32_t n_planes, uint64_t n_ids, uint64_t block_bytes, uint64_t src_block_stride,
+                      uint64_t src_blocks, uint32_t workgroups, hfk_stream_t stream) {
+    if (n_planes == 0 || n_ids == 0) return HFK_OK;
+    BlockCopyArgs<int64_t> a;
+    int rc = hfk::plan_gather_blocks(a, dst_plane_ptrs, src_plane_ptrs, ids, n_planes, n_ids, block_bytes,
+                                     src_block_stride, src_blocks);
+    if (rc != 0) return rc;
+    return launch_block_copy<int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
+}
+
+int hfk_set_tuning(int knob, int64_t value) {
+    switch (knob) {
+        case HFK_KNOB_UNROLL:
+            if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return HFK_ERR_BAD_KNOB;
+            g_unroll.store((int)value);
+            return HFK_OK;
+        case HFK_KNOB_NONTEMPORAL:
+            if (value < 0 || value > 3) return HFK_ERR_BAD_KNOB;
+            g_nontemporal.store((int)value);
+            return HFK_OK;
+        case HFK_KNOB_WORKGROUPS_PER_CU:
+            if (value < 1 || value > 64) return HFK_ERR_BAD_KNOB;
+            g_wg_per_cu.store((int)value);
+            return HFK_OK;
+        default:
+            return HFK_ERR_BAD_KNOB;
+    }
+}
+
+int64_t hfk_get_tuning(int knob) {
+    switch (knob) {
+        case HFK_KNOB_UNROLL: return g_unroll.load();
+        case HFK_KNOB_NONTEMPORAL: return g_nontemporal.load();
+        case HFK_KNOB_WORKGROUPS_PER_CU: return g_wg_per_cu.load();
+        default: return HFK_ERR_BAD_KNOB;
+    }
+}
+
+}  // extern "C"

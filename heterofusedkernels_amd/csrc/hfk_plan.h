@@ -1,0 +1,172 @@
+// Launch planning: turns the C-ABI arguments into kernel argument structs and
+// picks the access width. Pure host arithmetic with no HIP calls, shared by the
+// launchers and by the CPU index-math checker, so both walk the same geometry.
+#pragma once
+
+#include <stdint.h>
+
+#include "hfk.h"
+#include "hfk_bodies.h"
+
+namespace hfk {
+
+constexpr uint64_t kUnchecked = 1ull << 63;  // "no bound": still rejects negative ids
+constexpr uint64_t kU32Max = 0xffffffffull;
+
+// Rows at least this wide go through the block-copy kernel (uniform id loads, no
+// per-lane division); narrower rows through the flat kernel.
+constexpr uint64_t kWideRowBytes = 4096;
+constexpr int kFlatUnroll = 4;
+constexpr int kTransposeUnroll = 4;
+
+// A block smaller than 256 * unroll vectors would leave lanes idle, so the unroll
+// is halved until one chunk fits inside the block (down to 1).
+inline int fit_unroll(uint64_t block_bytes, int unroll) {
+    while (unroll > 1 && (uint64_t)kWorkgroupLanes * 16u * (uint64_t)unroll > block_bytes) {
+        unroll >>= 1;
+    }
+    return unroll;
+}
+
+// Fills chunks_per_block and n_work; returns the unroll to launch with.
+template <typename IdT>
+inline int plan_block_copy(BlockCopyArgs<IdT>& a, int preferred_unroll, int* unroll_out) {
+    const int unroll = fit_unroll(a.block_bytes, preferred_unroll);
+    const uint64_t chunk_bytes = (uint64_t)kWorkgroupLanes * 16u * (uint64_t)unroll;
+    const uint64_t chunks = (a.block_bytes + chunk_bytes - 1) / chunk_bytes;
+    const uint64_t tiles = (uint64_t)a.n_planes * (uint64_t)a.n_pairs;
+    if (chunks > kU32Max || tiles > kU32Max || chunks * tiles > kU32Max) return HFK_ERR_TOO_LARGE;
+    a.chunks_per_block = (uint32_t)chunks;
+    a.n_work = (uint32_t)(chunks * tiles);
+    *unroll_out = unroll;
+    return HFK_OK;
+}
+
+inline uint32_t pick_unit(uint64_t alignment_bits) {
+    return (alignment_bits & 15u) == 0 ? 16u : (alignment_bits & 3u) == 0 ? 4u : 1u;
+}
+
+struct FlatGatherPlan {
+    uint32_t unit;       // bytes per access: 16, 4 or 1
+    bool index32;        // flat indices fit 32 bits (cheap division)
+};
+
+template <typename IdT>
+inline int plan_flat_gather(FlatGatherArgs<IdT>& a, FlatGatherPlan& p, uint64_t table, uint64_t dst,
+                            const IdT* ids, uint64_t n_ids, uint64_t row_bytes, uint64_t row_limit) {
+    p.unit = pick_unit(table | dst | row_bytes);
+    a.table = table;
+    a.dst = dst;
+    a.ids = ids;
+    a.row_units = (uint32_t)(row_bytes / p.unit);
+    a.total_units = n_ids * (uint64_t)a.row_units;
+    a.row_limit = row_limit;
+    const uint64_t chunk_units = (uint64_t)kWorkgroupLanes * kFlatUnroll;
+    const uint64_t n_work = (a.total_units + chunk_units - 1) / chunk_units;
+    if (n_work > kU32Max) return HFK_ERR_TOO_LARGE;
+    a.n_work = (uint32_t)n_work;
+    p.index32 = n_work * chunk_units <= kU32Max;
+    return HFK_OK;
+}
+
+// Returns HFK_OK with n_work == 0 for an empty block.
+inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_layer_ptrs, const void* src,
+                          uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes) {
+    a.n_work = 0;
+    if (dev_layer_ptrs == nullptr || src == nullptr) return HFK_ERR_NULL_POINTER;
+    if (elem_bytes == 0) return HFK_ERR_BAD_SIZE;
+    if (T == 0 || L == 0 || H == 0 || D == 0) return HFK_OK;
+    const uint64_t row_bytes = (uint64_t)D * elem_bytes;
+    const uint64_t rows = (uint64_t)T * L * H;
+    const uint32_t unit = pick_unit((uint64_t)(uintptr_t)src | row_bytes);
+    const uint64_t row_units = row_bytes / unit;
+    const uint64_t total = rows * row_units;
+    const uint64_t chunk_units = (uint64_t)kWorkgroupLanes * kTransposeUnroll;
+    // The kernel indexes units with 32 bits.
+    if ((uint64_t)L * H > kU32Max || row_units > kU32Max || rows > kU32Max || total + chunk_units > kU32Max) {
+        return HFK_ERR_TOO_LARGE;
+    }
+    a.layer_ptrs = static_cast<const uint64_t*>(dev_layer_ptrs);
+    a.src = (uint64_t)(uintptr_t)src;
+    a.T = T;
+    a.L = L;
+    a.H = H;
+    a.row_units = (uint32_t)row_units;
+    a.total_units = (uint32_t)total;
+    a.n_work = (uint32_t)((total + chunk_units - 1) / chunk_units);
+    *unit_out = unit;
+    return HFK_OK;
+}
+
+// Argument checks + struct fill for the public block-table entry points.
+inline int plan_swap_blocks(BlockCopyArgs<int64_t>& a, const void* dst_plane_ptrs, const void* src_plane_ptrs,
+                            const int64_t* block_pairs, uint32_t n_planes, uint64_t n_pairs,
+                            uint64_t block_bytes, uint64_t src_block_stride, uint64_t dst_block_stride,
+                            uint64_t src_blocks, uint64_t dst_blocks) {
+    if (dst_plane_ptrs == nullptr || src_plane_ptrs == nullptr || block_pairs == nullptr) {
+        return HFK_ERR_NULL_POINTER;
+    }
+    if (block_bytes == 0 || src_block_stride < block_bytes || dst_block_stride < block_bytes) {
+        return HFK_ERR_BAD_SIZE;
+    }
+    if (n_pairs > kU32Max) return HFK_ERR_TOO_LARGE;
+    a = BlockCopyArgs<int64_t>{};
+    a.dst_planes = static_cast<const uint64_t*>(dst_plane_ptrs);
+    a.src_planes = static_cast<const uint64_t*>(src_plane_ptrs);
+    a.src_ids = block_pairs;
+    a.dst_ids = block_pairs + 1;
+    a.id_stride = 2;
+    a.n_planes = n_planes;
+    a.n_pairs = (uint32_t)n_pairs;
+    a.block_bytes = block_bytes;
+    a.src_stride = src_block_stride;
+    a.dst_stride = dst_block_stride;
+    a.src_limit = src_blocks ? src_blocks : kUnchecked;
+    a.dst_limit = dst_blocks ? dst_blocks : kUnchecked;
+    return HFK_OK;
+}
+
+inline int plan_gather_blocks(BlockCopyArgs<int64_t>& a, const void* dst_plane_ptrs, const void* src_plane_ptrs,
+                              const int64_t* ids, uint32_t n_planes, uint64_t n_ids, uint64_t block_bytes,
+                              uint64_t src_block_stride, uint64_t src_blocks) {
+    if (dst_plane_ptrs == nullptr || src_plane_ptrs == nullptr || ids == nullptr) return HFK_ERR_NULL_POINTER;
+    if (block_bytes == 0 || src_block_stride < block_bytes) return HFK_ERR_BAD_SIZE;
+    if (n_ids > kU32Max) return HFK_ERR_TOO_LARGE;
+    a = BlockCopyArgs<int64_t>{};
+    a.dst_planes = static_cast<const uint64_t*>(dst_plane_ptrs);
+    a.src_planes = static_cast<const uint64_t*>(src_plane_ptrs);
+    a.src_ids = ids;
+    a.dst_ids = nullptr;
+    a.id_stride = 1;
+    a.n_planes = n_planes;
+    a.n_pairs = (uint32_t)n_ids;
+    a.block_bytes = block_bytes;
+    a.src_stride = src_block_stride;
+    a.dst_stride = block_bytes;
+    a.src_limit = src_blocks ? src_blocks : kUnchecked;
+    a.dst_limit = kUnchecked;
+    return HFK_OK;
+}
+
+// Wide-row gather expressed as a single-plane block copy with dst block i = i.
+template <typename IdT>
+inline int plan_wide_gather(BlockCopyArgs<IdT>& a, const void* table, void* dst, const IdT* ids, uint64_t n_ids,
+                            uint64_t row_bytes, uint64_t row_limit) {
+    if (n_ids > kU32Max) return HFK_ERR_TOO_LARGE;
+    a = BlockCopyArgs<IdT>{};
+    a.dst_base = (uint64_t)(uintptr_t)dst;
+    a.src_base = (uint64_t)(uintptr_t)table;
+    a.src_ids = ids;
+    a.dst_ids = nullptr;
+    a.id_stride = 1;
+    a.n_planes = 1;
+    a.n_pairs = (uint32_t)n_ids;
+    a.block_bytes = row_bytes;
+    a.src_stride = row_bytes;
+    a.dst_stride = row_bytes;
+    a.src_limit = row_limit;
+    a.dst_limit = kUnchecked;
+    return HFK_OK;
+}
+
+}  // namespace hfk

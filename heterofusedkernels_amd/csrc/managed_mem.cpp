@@ -1,0 +1,360 @@
+// libmanaged_memory.so: registry of device-visible host ranges + pinned NUMA allocator.
+#include "managed_mem.h"
+
+#include <hip/hip_runtime_api.h>
+#include <sys/syscall.h>
+#include <unistd.h>
+
+#include <cctype>
+#include <cerrno>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <mutex>
+#include <string>
+
+#include "hfk_managed_memory.h"
+
+namespace managed_memory {
+
+namespace {
+thread_local int t_last_error = 0;
+
+// Swallow the sticky error a failed HIP call leaves behind so that it is not
+// reported by an unrelated later call.
+void drop_hip_error() { (void)hipGetLastError(); }
+}  // namespace
+
+HostRegisteredMemoryManager& HostRegisteredMemoryManager::GetInstance() {
+    // Leaked on purpose: records may be released from tensor deleters that run
+    // during interpreter shutdown, after static destructors would have fired.
+    static HostRegisteredMemoryManager* instance = new HostRegisteredMemoryManager();
+    return *instance;
+}
+
+HostRegisteredMemoryManager::~HostRegisteredMemoryManager() { unregisterAll(); }
+
+int HostRegisteredMemoryManager::lastError() { return t_last_error; }
+
+const RegisteredMemoryRecord* HostRegisteredMemoryManager::findContaining(uintptr_t addr) const {
+    auto it = records_.upper_bound(addr);
+    if (it == records_.begin()) return nullptr;
+    --it;
+    const RegisteredMemoryRecord& r = it->second;
+    return (addr - r.ptr < r.buffSize) ? &r : nullptr;
+}
+
+bool HostRegisteredMemoryManager::overlapsOther(uintptr_t start, size_t size) const {
+    // Only neighbours can overlap because stored ranges are disjoint.
+    auto next = records_.lower_bound(start);
+    if (next != records_.end() && next->first - start < size) return true;
+    if (next != records_.begin()) {
+        auto prev = std::prev(next);
+        if (start - prev->second.ptr < prev->second.buffSize) return true;
+    }
+    return false;
+}
+
+const RegisteredMemoryRecord* HostRegisteredMemoryManager::adoptMapping(void* hostPtr, void* devPtr,
+                                                                        size_t bufferSize, int32_t device,
+                                                                        int32_t kind) {
+    if (hostPtr == nullptr || devPtr == nullptr || bufferSize == 0) {
+        t_last_error = HFK_MM_ERR_BAD_ARGUMENT;
+        return nullptr;
+    }
+    const uintptr_t start = reinterpret_cast<uintptr_t>(hostPtr);
+    const std::unique_lock<std::shared_mutex> guard(mux_);
+    auto hit = records_.find(start);
+    if (hit != records_.end()) return &hit->second;
+    if (overlapsOther(start, bufferSize)) {
+        t_last_error = HFK_MM_ERR_OVERLAP;
+        return nullptr;
+    }
+    auto ins = records_.emplace(
+        start, RegisteredMemoryRecord{start, reinterpret_cast<uintptr_t>(devPtr), bufferSize, device, kind});
+    return &ins.first->second;
+}
+
+const RegisteredMemoryRecord* HostRegisteredMemoryManager::registerHostPtr(void* hostPtr, size_t bufferSize) {
+    if (hostPtr == nullptr || bufferSize == 0) {
+        t_last_error = HFK_MM_ERR_BAD_ARGUMENT;
+        return nullptr;
+    }
+    const uintptr_t start = reinterpret_cast<uintptr_t>(hostPtr);
+    {
+        const std::shared_lock<std::shared_mutex> guard(mux_);
+        auto hit = records_.find(start);
+        if (hit != records_.end()) return &hit->second;  // idempotent
+        // A range inside an existing record is already device-visible.
+        const RegisteredMemoryRecord* outer = findContaining(start);
+        if (outer != nullptr && start + bufferSize <= outer->ptr + outer->buffSize) return outer;
+    }
+
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess) {
+        drop_hip_error();
+        device = -1;
+    }
+
+    // Already pinned by someone else (hipHostMalloc, torch's pinned allocator)?
+    hipPointerAttribute_t attr;
+    std::memset(&attr, 0, sizeof(attr));
+    hipError_t e = hipPointerGetAttributes(&attr, hostPtr);
+    int32_t kind = HFK_MM_KIND_ADOPTED;
+    if (e != hipSuccess) drop_hip_error();
+    if (e != hipSuccess || attr.type != hipMemoryTypeHost) {
+        e = hipHostRegister(hostPtr, bufferSize, hipHostRegisterMapped | hipHostRegisterPortable);
+        if (e != hipSuccess) {
+            drop_hip_error();
+            t_last_error = static_cast<int>(e);
+            std::fprintf(stderr, "managed_memory: hipHostRegister(%p, %zu) failed: %s\n", hostPtr, bufferSize,
+                         hipGetErrorString(e));
+            return nullptr;
+        }
+        kind = HFK_MM_KIND_REGISTERED;
+    }
+    void* devPtr = nullptr;
+    e = hipHostGetDevicePointer(&devPtr, hostPtr, 0);
+    if (e != hipSuccess || devPtr == nullptr) {
+        drop_hip_error();
+        if (kind == HFK_MM_KIND_REGISTERED) (void)hipHostUnregister(hostPtr);
+        t_last_error = e != hipSuccess ? static_cast<int>(e) : HFK_MM_ERR_BAD_ARGUMENT;
+        return nullptr;
+    }
+    const RegisteredMemoryRecord* rec = adoptMapping(hostPtr, devPtr, bufferSize, device, kind);
+    if (rec == nullptr && kind == HFK_MM_KIND_REGISTERED) (void)hipHostUnregister(hostPtr);
+    return rec;
+}
+
+int HostRegisteredMemoryManager::unregisterHostPtr(void* hostPtr) {
+    if (hostPtr == nullptr) return HFK_MM_ERR_BAD_ARGUMENT;
+    RegisteredMemoryRecord rec;
+    {
+        const std::unique_lock<std::shared_mutex> guard(mux_);
+        auto hit = records_.find(reinterpret_cast<uintptr_t>(hostPtr));
+        if (hit == records_.end()) return HFK_MM_OK;  // never registered: nothing to undo
+        rec = hit->second;
+        records_.erase(hit);
+    }
+    if (rec.kind == HFK_MM_KIND_REGISTERED) {
+        hipError_t e = hipHostUnregister(hostPtr);
+        if (e != hipSuccess) {
+            drop_hip_error();
+            return static_cast<int>(e);
+        }
+    }
+    return HFK_MM_OK;
+}
+
+void HostRegisteredMemoryManager::unregisterAll() {
+    std::map<uintptr_t, RegisteredMemoryRecord> drained;
+    {
+        const std::unique_lock<std::shared_mutex> guard(mux_);
+        drained.swap(records_);
+    }
+    for (const auto& kv : drained) {
+        if (kv.second.kind == HFK_MM_KIND_REGISTERED) {
+            if (hipHostUnregister(reinterpret_cast<void*>(kv.first)) != hipSuccess) drop_hip_error();
+        }
+    }
+}
+
+void* HostRegisteredMemoryManager::getDevicePtr(const void* hostPtr) const {
+    if (hostPtr == nullptr) return nullptr;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(hostPtr);
+    const std::shared_lock<std::shared_mutex> guard(mux_);
+    const RegisteredMemoryRecord* r = findContaining(addr);
+    return r ? reinterpret_cast<void*>(r->devptr + (addr - r->ptr)) : nullptr;
+}
+
+size_t HostRegisteredMemoryManager::getRecordSize(const void* hostPtr) const {
+    if (hostPtr == nullptr) return 0;
+    const std::shared_lock<std::shared_mutex> guard(mux_);
+    const RegisteredMemoryRecord* r = findContaining(reinterpret_cast<uintptr_t>(hostPtr));
+    return r ? r->buffSize : 0;
+}
+
+size_t HostRegisteredMemoryManager::recordCount() const {
+    const std::shared_lock<std::shared_mutex> guard(mux_);
+    return records_.size();
+}
+
+}  // namespace managed_memory
+
+using managed_memory::HostRegisteredMemoryManager;
+
+void* register_ptr(void* ptr, size_t size) {
+    const auto* rec = HostRegisteredMemoryManager::GetInstance().registerHostPtr(ptr, size);
+    if (rec == nullptr) return nullptr;
+    const uintptr_t off = reinterpret_cast<uintptr_t>(ptr) - rec->ptr;
+    return reinterpret_cast<void*>(rec->devptr + off);
+}
+
+int unregister_ptr(void* ptr) { return HostRegisteredMemoryManager::GetInstance().unregisterHostPtr(ptr); }
+
+uintptr_t get_device_ptr(uintptr_t ptr) {
+    return reinterpret_cast<uintptr_t>(
+        HostRegisteredMemoryManager::GetInstance().getDevicePtr(reinterpret_cast<const void*>(ptr)));
+}
+
+// ---------------------------------------------------------------------------
+// NUMA placement. The memory policy syscalls are used directly so the library
+// has no libnuma dependency.
+// ---------------------------------------------------------------------------
+namespace {
+
+constexpr int kMpolDefault = 0;
+constexpr int kMpolBind = 2;
+constexpr unsigned long kMaxNodes = 1024;
+constexpr size_t kMaskWords = kMaxNodes / (8 * sizeof(unsigned long));
+
+long sys_get_mempolicy(int* mode, unsigned long* mask, unsigned long maxnode) {
+    return syscall(SYS_get_mempolicy, mode, mask, maxnode, nullptr, 0ul);
+}
+
+long sys_set_mempolicy(int mode, const unsigned long* mask, unsigned long maxnode) {
+    return syscall(SYS_set_mempolicy, mode, mask, maxnode);
+}
+
+// Binds this thread's future page allocations to one node for its lifetime.
+class ScopedNodeBinding {
+public:
+    explicit ScopedNodeBinding(int node) {
+        if (node < 0 || static_cast<unsigned long>(node) >= kMaxNodes) return;
+        if (sys_get_mempolicy(&saved_mode_, saved_mask_, kMaxNodes) != 0) return;
+        unsigned long mask[kMaskWords] = {0};
+        mask[node / (8 * sizeof(unsigned long))] = 1ul << (node % (8 * sizeof(unsigned long)));
+        if (sys_set_mempolicy(kMpolBind, mask, kMaxNodes) == 0) active_ = true;
+    }
+    ~ScopedNodeBinding() {
+        if (!active_) return;
+        if (saved_mode_ == kMpolDefault) (void)sys_set_mempolicy(kMpolDefault, nullptr, 0);
+        else (void)sys_set_mempolicy(saved_mode_, saved_mask_, kMaxNodes);
+    }
+    bool active() const { return active_; }
+
+private:
+    bool active_ = false;
+    int saved_mode_ = kMpolDefault;
+    unsigned long saved_mask_[kMaskWords] = {0};
+};
+
+}  // namespace
+
+extern "C" {
+
+int hfk_mm_register(void* host_ptr, size_t bytes, void** dev_ptr_out) {
+    if (host_ptr == nullptr || bytes == 0) return HFK_MM_ERR_BAD_ARGUMENT;
+    void* dev = register_ptr(host_ptr, bytes);
+    if (dev == nullptr) {
+        const int err = HostRegisteredMemoryManager::lastError();
+        return err != 0 ? err : HFK_MM_ERR_BAD_ARGUMENT;
+    }
+    if (dev_ptr_out) *dev_ptr_out = dev;
+    return HFK_MM_OK;
+}
+
+int hfk_mm_adopt(void* host_ptr, void* dev_ptr, size_t bytes, int device) {
+    const auto* rec = HostRegisteredMemoryManager::GetInstance().adoptMapping(host_ptr, dev_ptr, bytes, device,
+                                                                              HFK_MM_KIND_ADOPTED);
+    if (rec == nullptr) return HostRegisteredMemoryManager::lastError();
+    return HFK_MM_OK;
+}
+
+int hfk_mm_unregister(void* host_ptr) { return unregister_ptr(host_ptr); }
+
+void hfk_mm_unregister_all(void) { HostRegisteredMemoryManager::GetInstance().unregisterAll(); }
+
+void* hfk_mm_get_device_ptr(const void* host_ptr) {
+    return HostRegisteredMemoryManager::GetInstance().getDevicePtr(host_ptr);
+}
+
+size_t hfk_mm_record_size(const void* host_ptr) {
+    return HostRegisteredMemoryManager::GetInstance().getRecordSize(host_ptr);
+}
+
+size_t hfk_mm_record_count(void) { return HostRegisteredMemoryManager::GetInstance().recordCount(); }
+
+int hfk_mm_device_numa_node(int device, int* node_out) {
+    if (node_out == nullptr) return HFK_MM_ERR_BAD_ARGUMENT;
+    *node_out = -1;
+    char bdf[64] = {0};
+    hipError_t e = hipDeviceGetPCIBusId(bdf, sizeof(bdf) - 1, device);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+    }
+    std::string id(bdf);
+    for (char& c : id) c = static_cast<char>(std::tolower(static_cast<unsigned char>(c)));
+    std::ifstream f("/sys/bus/pci/devices/" + id + "/numa_node");
+    if (!f.is_open()) return HFK_MM_OK;  // sysfs hidden (containers): treat as "no NUMA information"
+    int node = -1;
+    f >> node;
+    if (!f.fail()) *node_out = node;
+    return HFK_MM_OK;
+}
+
+int hfk_mm_alloc_pinned(size_t bytes, int numa_node, unsigned flags, void** host_ptr_out) {
+    if (bytes == 0 || host_ptr_out == nullptr) return HFK_MM_ERR_BAD_ARGUMENT;
+    *host_ptr_out = nullptr;
+    void* p = nullptr;
+    hipError_t e;
+    {
+        ScopedNodeBinding bind(numa_node);
+        unsigned hip_flags = hipHostMallocMapped | hipHostMallocPortable;
+        if (bind.active()) hip_flags |= hipHostMallocNumaUser;
+        if (flags & HFK_MM_ALLOC_NONCOHERENT) hip_flags |= hipHostMallocNonCoherent;
+        e = hipHostMalloc(&p, bytes, hip_flags);
+    }
+    if (e != hipSuccess || p == nullptr) {
+        (void)hipGetLastError();
+        return e != hipSuccess ? static_cast<int>(e) : HFK_MM_ERR_OS;
+    }
+    std::memset(p, 0, bytes);
+    void* dev = nullptr;
+    e = hipHostGetDevicePointer(&dev, p, 0);
+    if (e != hipSuccess || dev == nullptr) {
+        (void)hipGetLastError();
+        (void)hipHostFree(p);
+        return e != hipSuccess ? static_cast<int>(e) : HFK_MM_ERR_OS;
+    }
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess) {
+        (void)hipGetLastError();
+        device = -1;
+    }
+    const auto* rec = HostRegisteredMemoryManager::GetInstance().adoptMapping(p, dev, bytes, device,
+                                                                              HFK_MM_KIND_ALLOCATED);
+    if (rec == nullptr) {
+        (void)hipHostFree(p);
+        return HostRegisteredMemoryManager::lastError();
+    }
+    *host_ptr_out = p;
+    return HFK_MM_OK;
+}
+
+int hfk_mm_free_pinned(void* host_ptr) {
+    if (host_ptr == nullptr) return HFK_MM_ERR_BAD_ARGUMENT;
+    (void)HostRegisteredMemoryManager::GetInstance().unregisterHostPtr(host_ptr);
+    hipError_t e = hipHostFree(host_ptr);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+    }
+    return HFK_MM_OK;
+}
+
+const char* hfk_mm_status_string(int status) {
+    switch (status) {
+        case HFK_MM_OK: return "ok";
+        case HFK_MM_ERR_BAD_ARGUMENT: return "managed_memory: null pointer or zero size";
+        case HFK_MM_ERR_OVERLAP: return "managed_memory: range overlaps a different registration";
+        case HFK_MM_ERR_NOT_FOUND: return "managed_memory: pointer is not registered";
+        case HFK_MM_ERR_OS: return "managed_memory: operating-system call failed";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
+    return "managed_memory: unknown status";
+}
+
+}  // extern "C"

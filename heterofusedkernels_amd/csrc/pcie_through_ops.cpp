@@ -1,0 +1,246 @@
+// libpcie_through.so: the torch dispatcher ops of the pcie_through namespace.
+//
+// Schemas of the first three ops are those of the reference
+// (pcieThrough/csrc/host/gather_torch.cpp:60,
+//  pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:113-114);
+// swap_blocks and gather_blocks are additive. Every op unpacks its tensors into
+// raw device-visible addresses, takes the current HIP stream of the device that
+// owns the device-side tensor, and calls the C-ABI of libhfk_hip.so; nothing is
+// allocated and nothing waits.
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include <optional>
+
+#include "hfk.h"
+#include "managed_mem.h"
+
+namespace pciethrough {
+
+namespace {
+
+using managed_memory::HostRegisteredMemoryManager;
+
+// `aiv` is the reference's AI-vector-core count. It is validated exactly as there
+// (converted to uint32, zero rejected; gather_torch.cpp:32-36) and otherwise
+// unused: the grid is sized from the GPU's CU count, and results never depended on it.
+void check_aiv(const std::optional<int64_t>& aiv) {
+    if (aiv.has_value()) {
+        const uint32_t aivNum = static_cast<uint32_t>(aiv.value());
+        TORCH_CHECK(aivNum > 0, "Number of AIV blocks should be positive.");
+    }
+}
+
+// Address a kernel can use for the tensor's first element. Device tensors are
+// used as they are; host tensors must be registered (heterofusedkernels.memory)
+// or at least pinned, in which case their storage is registered on first use.
+// The reference passes an unchecked nullptr to the kernel here
+// (gather_torch.cpp:51, multi_layer_block_transfer_torch.cpp:78).
+void* device_visible(const at::Tensor& t, const char* what) {
+    if (t.is_cuda()) return t.data_ptr();
+    TORCH_CHECK(t.device().is_cpu(), what, ": unsupported device ", t.device());
+    auto& registry = HostRegisteredMemoryManager::GetInstance();
+    void* dev = registry.getDevicePtr(t.data_ptr());
+    if (dev != nullptr) return dev;
+    TORCH_CHECK(t.is_pinned(), what,
+                ": host tensor is neither registered with heterofusedkernels.memory nor pinned");
+    const auto& storage = t.storage();
+    TORCH_CHECK(registry.registerHostPtr(storage.mutable_data(), storage.nbytes()) != nullptr, what,
+                ": registering the pinned host tensor failed");
+    dev = registry.getDevicePtr(t.data_ptr());
+    TORCH_CHECK(dev != nullptr, what, ": no device-visible address for host tensor");
+    return dev;
+}
+
+hfk_stream_t current_stream() {
+    return static_cast<hfk_stream_t>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
+}
+
+void check_status(int rc, const char* entry) {
+    TORCH_CHECK(rc == 0, entry, " failed: ", hfk_status_string(rc), " (", rc, ")");
+}
+
+uint32_t workgroup_cap(const std::optional<int64_t>& workgroups) {
+    if (!workgroups.has_value()) return 0;
+    TORCH_CHECK(workgroups.value() >= 0 && workgroups.value() <= 0x7fffffff, "workgroups out of range");
+    return static_cast<uint32_t>(workgroups.value());
+}
+
+struct BlockGeometry {
+    uint32_t T, L, H, D, elem;
+};
+
+BlockGeometry block_geometry(const at::Tensor& hostBlockCache) {
+    TORCH_CHECK(hostBlockCache.dim() == 4,
+                "hostBlockCache must be [blockSize, layers, heads, headDims], got ", hostBlockCache.dim(),
+                " dims");
+    TORCH_CHECK(hostBlockCache.is_contiguous(), "hostBlockCache must be contiguous");
+    for (int i = 0; i < 4; ++i) {
+        TORCH_CHECK(hostBlockCache.size(i) <= 0xffffffffLL, "hostBlockCache dimension ", i, " too large");
+    }
+    return {static_cast<uint32_t>(hostBlockCache.size(0)), static_cast<uint32_t>(hostBlockCache.size(1)),
+            static_cast<uint32_t>(hostBlockCache.size(2)), static_cast<uint32_t>(hostBlockCache.size(3)),
+            static_cast<uint32_t>(hostBlockCache.element_size())};
+}
+
+void check_layer_ptrs(const at::Tensor& deviceBlockCachePtrs, uint32_t layers) {
+    TORCH_CHECK(deviceBlockCachePtrs.is_cuda(), "deviceBlockCachePtrs must be a device tensor");
+    TORCH_CHECK(deviceBlockCachePtrs.scalar_type() == at::kLong, "deviceBlockCachePtrs must be int64");
+    TORCH_CHECK(deviceBlockCachePtrs.is_contiguous(), "deviceBlockCachePtrs must be contiguous");
+    TORCH_CHECK(deviceBlockCachePtrs.numel() >= layers, "deviceBlockCachePtrs holds ",
+                deviceBlockCachePtrs.numel(), " pointers, hostBlockCache has ", layers, " layers");
+}
+
+void check_ptr_table(const at::Tensor& t, const char* what) {
+    TORCH_CHECK(t.scalar_type() == at::kLong, what, " must be int64");
+    TORCH_CHECK(t.is_contiguous(), what, " must be contiguous");
+}
+
+}  // namespace
+
+// dst[i, :] = table[ids[i], :]. Mirrors gather_torch.cpp:30-54. Row size is
+// element_size * size(1) for the 2-D tables the reference is used with, and the
+// product of all trailing dimensions for higher-rank (e.g. paged KV) tables.
+void gather(const at::Tensor& gmEmbed, const at::Tensor& gmEmbedDst, const at::Tensor& gmIds,
+            std::optional<int64_t> aiv) {
+    check_aiv(aiv);
+    TORCH_CHECK(gmEmbed.dim() >= 2, "gmEmbed must have at least 2 dimensions");
+    TORCH_CHECK(gmIds.dim() >= 1, "gmIds must be 1-dimensional");
+    TORCH_CHECK(gmEmbed.is_contiguous() && gmEmbedDst.is_contiguous() && gmIds.is_contiguous(),
+                "gather: tensors must be contiguous");
+    TORCH_CHECK(gmEmbedDst.is_cuda(), "gmEmbedDst must be a device tensor");
+    TORCH_CHECK(gmIds.scalar_type() == at::kLong || gmIds.scalar_type() == at::kInt, "ScalarType ",
+                c10::toString(gmIds.scalar_type()), " not supported.");
+    const uint64_t numIds = static_cast<uint64_t>(gmIds.size(0));
+    const uint64_t tableRows = static_cast<uint64_t>(gmEmbed.size(0));
+    uint64_t rowBytes = static_cast<uint64_t>(gmEmbed.element_size());
+    for (int64_t d = 1; d < gmEmbed.dim(); ++d) rowBytes *= static_cast<uint64_t>(gmEmbed.size(d));
+    if (numIds == 0) return;
+    TORCH_CHECK(rowBytes > 0, "gmEmbed rows are empty");
+    TORCH_CHECK(static_cast<uint64_t>(gmEmbedDst.nbytes()) >= numIds * rowBytes, "gmEmbedDst holds ",
+                gmEmbedDst.nbytes(), " bytes, ", numIds * rowBytes, " needed");
+
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(gmEmbedDst));
+    const void* table = device_visible(gmEmbed, "gmEmbed");
+    const void* ids = device_visible(gmIds, "gmIds");
+    check_status(hfk_gather_rows(table, gmEmbedDst.data_ptr(), ids, gmIds.scalar_type() == at::kLong, numIds,
+                                 rowBytes, tableRows, 0, current_stream()),
+                 "hfk_gather_rows");
+}
+
+// One [T,L,H,D] host block -> L device buffers [H,T,D].
+// Mirrors multi_layer_block_transfer_torch.cpp:58-80.
+void multi_layer_block_transfer(const at::Tensor& deviceBlockCachePtrs, const at::Tensor& hostBlockCache,
+                                std::optional<int64_t> aiv) {
+    check_aiv(aiv);
+    const BlockGeometry g = block_geometry(hostBlockCache);
+    check_layer_ptrs(deviceBlockCachePtrs, g.L);
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(deviceBlockCachePtrs));
+    const void* src = device_visible(hostBlockCache, "hostBlockCache");
+    check_status(hfk_multi_layer_block_transfer(deviceBlockCachePtrs.data_ptr(), src, g.T, g.L, g.H, g.D, g.elem,
+                                                0, current_stream()),
+                 "hfk_multi_layer_block_transfer");
+}
+
+// Whole-block async copy into stagingBlockCache, then the same conversion from
+// HBM. Mirrors multi_layer_block_transfer_torch.cpp:82-106.
+void fused_memcpy_multi_layer_block_transfer(const at::Tensor& deviceBlockCachePtrs,
+                                             const at::Tensor& hostBlockCache,
+                                             const at::Tensor& stagingBlockCache, std::optional<int64_t> aiv) {
+    check_aiv(aiv);
+    const BlockGeometry g = block_geometry(hostBlockCache);
+    check_layer_ptrs(deviceBlockCachePtrs, g.L);
+    TORCH_CHECK(stagingBlockCache.is_cuda(), "stagingBlockCache must be a device tensor");
+    TORCH_CHECK(stagingBlockCache.is_contiguous(), "stagingBlockCache must be contiguous");
+    TORCH_CHECK(stagingBlockCache.nbytes() >= hostBlockCache.nbytes(), "stagingBlockCache holds ",
+                stagingBlockCache.nbytes(), " bytes, ", hostBlockCache.nbytes(), " needed");
+    TORCH_CHECK(hostBlockCache.device().is_cpu(), "hostBlockCache must be a host tensor");
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(deviceBlockCachePtrs));
+    check_status(hfk_fused_memcpy_multi_layer_block_transfer(deviceBlockCachePtrs.data_ptr(),
+                                                             hostBlockCache.data_ptr(),
+                                                             stagingBlockCache.data_ptr(), g.T, g.L, g.H, g.D,
+                                                             g.elem, 0, current_stream()),
+                 "hfk_fused_memcpy_multi_layer_block_transfer");
+}
+
+// Block-table swap, every plane in one launch; see hfk_swap_blocks. The plane
+// tables hold raw addresses (device pointers, or heterofusedkernels.memory
+// .get_device_ptr() of pinned host planes), built once by the caller exactly like
+// the per-layer pointer tensor of the reference's transfer op
+// (pcieThrough/tests/test_transfer_kernel.py:42-47).
+void swap_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs, const at::Tensor& blockPairs,
+                 int64_t blockBytes, int64_t srcBlockStride, int64_t dstBlockStride, int64_t srcBlocks,
+                 int64_t dstBlocks, std::optional<int64_t> workgroups) {
+    check_ptr_table(dstPlanePtrs, "dstPlanePtrs");
+    check_ptr_table(srcPlanePtrs, "srcPlanePtrs");
+    check_ptr_table(blockPairs, "blockPairs");
+    TORCH_CHECK(dstPlanePtrs.is_cuda(), "dstPlanePtrs must be a device tensor");
+    TORCH_CHECK(dstPlanePtrs.numel() == srcPlanePtrs.numel(), "plane tables differ in length");
+    TORCH_CHECK(blockPairs.dim() == 2 && blockPairs.size(1) == 2, "blockPairs must be [n, 2]");
+    TORCH_CHECK(blockBytes > 0 && srcBlockStride >= blockBytes && dstBlockStride >= blockBytes,
+                "swap_blocks: strides must be at least blockBytes, blockBytes positive");
+    TORCH_CHECK(srcBlocks >= 0 && dstBlocks >= 0, "swap_blocks: block counts must be non-negative");
+    TORCH_CHECK(dstPlanePtrs.numel() <= 0xffffffffLL, "too many planes");
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(dstPlanePtrs));
+    check_status(
+        hfk_swap_blocks(dstPlanePtrs.data_ptr(), device_visible(srcPlanePtrs, "srcPlanePtrs"),
+                        static_cast<const int64_t*>(device_visible(blockPairs, "blockPairs")),
+                        static_cast<uint32_t>(dstPlanePtrs.numel()), static_cast<uint64_t>(blockPairs.size(0)),
+                        static_cast<uint64_t>(blockBytes), static_cast<uint64_t>(srcBlockStride),
+                        static_cast<uint64_t>(dstBlockStride), static_cast<uint64_t>(srcBlocks),
+                        static_cast<uint64_t>(dstBlocks), workgroup_cap(workgroups), current_stream()),
+        "hfk_swap_blocks");
+}
+
+// Shared-id block gather over planes; see hfk_gather_blocks.
+void gather_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs, const at::Tensor& blockIds,
+                   int64_t blockBytes, int64_t srcBlockStride, int64_t srcBlocks,
+                   std::optional<int64_t> workgroups) {
+    check_ptr_table(dstPlanePtrs, "dstPlanePtrs");
+    check_ptr_table(srcPlanePtrs, "srcPlanePtrs");
+    check_ptr_table(blockIds, "blockIds");
+    TORCH_CHECK(dstPlanePtrs.is_cuda(), "dstPlanePtrs must be a device tensor");
+    TORCH_CHECK(dstPlanePtrs.numel() == srcPlanePtrs.numel(), "plane tables differ in length");
+    TORCH_CHECK(blockIds.dim() == 1, "blockIds must be 1-dimensional");
+    TORCH_CHECK(blockBytes > 0 && srcBlockStride >= blockBytes,
+                "gather_blocks: stride must be at least blockBytes, blockBytes positive");
+    TORCH_CHECK(srcBlocks >= 0, "gather_blocks: block count must be non-negative");
+    TORCH_CHECK(dstPlanePtrs.numel() <= 0xffffffffLL, "too many planes");
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(dstPlanePtrs));
+    check_status(
+        hfk_gather_blocks(dstPlanePtrs.data_ptr(), device_visible(srcPlanePtrs, "srcPlanePtrs"),
+                          static_cast<const int64_t*>(device_visible(blockIds, "blockIds")),
+                          static_cast<uint32_t>(dstPlanePtrs.numel()), static_cast<uint64_t>(blockIds.size(0)),
+                          static_cast<uint64_t>(blockBytes), static_cast<uint64_t>(srcBlockStride),
+                          static_cast<uint64_t>(srcBlocks), workgroup_cap(workgroups), current_stream()),
+        "hfk_gather_blocks");
+}
+
+}  // namespace pciethrough
+
+TORCH_LIBRARY(pcie_through, m) {
+    m.def("gather(Tensor gmEmbed, Tensor gmEmbedDst, Tensor gmIds, int? aiv=None) -> ()");
+    m.def("multi_layer_block_transfer(Tensor deviceBlockCachePtrs, Tensor hostBlockCache, int? aiv=None) -> ()");
+    m.def(
+        "fused_memcpy_multi_layer_block_transfer(Tensor deviceBlockCachePtrs, Tensor hostBlockCache, Tensor "
+        "stagingBlockCache, int? aiv=None) -> ()");
+    m.def(
+        "swap_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockPairs, int blockBytes, int "
+        "srcBlockStride, int dstBlockStride, int srcBlocks=0, int dstBlocks=0, int? workgroups=None) -> ()");
+    m.def(
+        "gather_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockIds, int blockBytes, int "
+        "srcBlockStride, int srcBlocks=0, int? workgroups=None) -> ()");
+}
+
+// PyTorch-ROCm files HIP tensors under the CUDA dispatch key. A call whose tensors
+// are all on the CPU finds no kernel and raises, which is the intended behaviour:
+// there is no CPU implementation of these ops.
+TORCH_LIBRARY_IMPL(pcie_through, CUDA, m) {
+    m.impl("gather", TORCH_FN(pciethrough::gather));
+    m.impl("multi_layer_block_transfer", TORCH_FN(pciethrough::multi_layer_block_transfer));
+    m.impl("fused_memcpy_multi_layer_block_transfer", TORCH_FN(pciethrough::fused_memcpy_multi_layer_block_transfer));
+    m.impl("swap_blocks", TORCH_FN(pciethrough::swap_blocks));
+    m.impl("gather_blocks", TORCH_FN(pciethrough::gather_blocks));
+}

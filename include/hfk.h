@@ -1,0 +1,170 @@
+/*
+ * hfk.h - C-ABI of libhfk_hip.so: KV-cache block swap, block gather and the
+ * layout-converting multi-layer block transfer for AMD MI355X (gfx950).
+ *
+ * Every entry point
+ *   - takes plain pointers and sizes (no torch types),
+ *   - enqueues work on the HIP stream it is given and returns without waiting,
+ *   - returns 0 on success, a negative hfk_status for a rejected argument, or a
+ *     positive hipError_t reported by the HIP runtime,
+ *   - never throws, owns no memory and keeps no state between calls apart from
+ *     cached device properties and the values set through hfk_set_tuning().
+ *
+ * "Device-visible" below means an address a kernel may dereference: device
+ * memory, or pinned host memory in its mapped (hipHostGetDevicePointer) form.
+ * Host memory is read and written by the kernels directly over the PCIe link.
+ *
+ * The library moves bytes only; element types matter solely through their size.
+ */
+#ifndef HFK_H
+#define HFK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HFK_API __attribute__((visibility("default")))
+
+#define HFK_VERSION_MAJOR 0
+#define HFK_VERSION_MINOR 1
+
+/* A hipStream_t passed as an opaque pointer; NULL is the null stream. */
+typedef void* hfk_stream_t;
+
+enum hfk_status {
+    HFK_OK = 0,
+    HFK_ERR_NULL_POINTER = -1, /* a required pointer argument is NULL            */
+    HFK_ERR_BAD_SIZE = -2,     /* a size/stride is zero or inconsistent          */
+    HFK_ERR_TOO_LARGE = -3,    /* a count exceeds what one launch can index      */
+    HFK_ERR_BAD_KNOB = -4      /* unknown tuning knob or value out of range      */
+};
+
+/* HFK_VERSION_MAJOR * 1000 + HFK_VERSION_MINOR of the loaded library. */
+HFK_API int hfk_version(void);
+
+/* Static, NUL-terminated description of a value returned by any hfk_* call
+ * (negative: this library's codes, positive: hipGetErrorString). */
+HFK_API const char* hfk_status_string(int status);
+
+/*
+ * Row gather:  dst[i, :] = table[ids[i], :]   for i in [0, n_ids)
+ *
+ * Replaces the reference's gather op and kernel:
+ *   pcieThrough/csrc/host/gather_torch.cpp:30-54   (host op `pciethrough::gather`)
+ *   pcieThrough/csrc/kernel/gather.cpp:7-48        (`gather_kernel`)
+ *   pcieThrough/csrc/kernel/gather.h:85-133        (`Gather::MteCopy::LoadStoreFunc`)
+ *
+ *   table       device-visible, rows of row_bytes bytes, row r at table + r*row_bytes
+ *   dst         device-visible, n_ids contiguous rows
+ *   ids         device-visible, int64 (ids_are_i64 != 0) or int32 indices
+ *   table_rows  number of rows in table; an id outside [0, table_rows) leaves its
+ *               dst row untouched. 0 disables the check (the reference never checks).
+ *   workgroups  upper bound on workgroups launched, 0 = library default.
+ *
+ * n_ids == 0 is a successful no-op. Rows of any byte size and alignment are
+ * accepted; 16-byte aligned rows take the vectorised path.
+ */
+HFK_API int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i64,
+                    uint64_t n_ids, uint64_t row_bytes, uint64_t table_rows,
+                    uint32_t workgroups, hfk_stream_t stream);
+
+/*
+ * Layout-converting transfer of one KV block across all layers:
+ *   layer_l[(h*T + t)*D + d] = src_block[((t*L + l)*H + h)*D + d]
+ * for t<T, l<L, h<H, d<D, elements of elem_bytes bytes; layer_l is the pointer
+ * stored in dev_layer_ptrs[l].
+ *
+ * Replaces
+ *   pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:58-80
+ *       (host op `pciethrough::multi_layer_block_transfer`, incl. the tiling upload
+ *        `mvTilingToDevice` :13-39, which has no counterpart here: the geometry
+ *        travels as kernel arguments)
+ *   pcieThrough/csrc/kernel/multi_layer_block_transfer_kernel.cpp:8-29
+ *   pcieThrough/csrc/kernel/multi_layer_block_transfer_kernel.h:42-82
+ *
+ *   dev_layer_ptrs  device-visible array of L uint64 addresses, each a
+ *                   device-visible buffer of H*T*D*elem_bytes bytes ([H,T,D])
+ *   src_block       device-visible [T,L,H,D] block (pinned host memory in the
+ *                   reference's use, device memory for the staged variant)
+ */
+HFK_API int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* src_block,
+                                   uint32_t T, uint32_t L, uint32_t H, uint32_t D,
+                                   uint32_t elem_bytes, uint32_t workgroups,
+                                   hfk_stream_t stream);
+
+/*
+ * Staged variant: hipMemcpyAsync(staging <- host_block, whole block) on `stream`,
+ * then the transfer above reading `staging`. Afterwards staging == host_block.
+ *
+ * Replaces pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:82-106
+ * (`pciethrough::fused_memcpy_multi_layer_block_transfer`).
+ *
+ *   host_block  the host address of the pinned [T,L,H,D] block (not its mapped form)
+ *   staging     device buffer of T*L*H*D*elem_bytes bytes
+ */
+HFK_API int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs,
+                                                const void* host_block, void* staging,
+                                                uint32_t T, uint32_t L, uint32_t H,
+                                                uint32_t D, uint32_t elem_bytes,
+                                                uint32_t workgroups, hfk_stream_t stream);
+
+/*
+ * Block-table swap, all planes (layer x K/V) in one launch:
+ *   for p < n_planes, j < n_pairs:
+ *     copy block_bytes bytes
+ *       from src_plane_ptrs[p] + block_pairs[j][0] * src_block_stride
+ *       to   dst_plane_ptrs[p] + block_pairs[j][1] * dst_block_stride
+ * Direction-agnostic: swap-out passes device planes as src and mapped host planes
+ * as dst, swap-in the reverse; device-to-device works the same way.
+ *
+ * Replaces the caller-side per-block loop of the reference,
+ *   pcieThrough/tests/test_transfer_kernel.py:58-72
+ * (one op call, one tiling upload and two allocations per block) with a single
+ * launch. Equivalent CPU statement, per plane:
+ *   dst.index_copy_(0, pairs[:,1], src.index_select(0, pairs[:,0]))
+ *
+ *   dst_plane_ptrs, src_plane_ptrs  device-visible arrays of n_planes uint64 addresses
+ *   block_pairs   device-visible int64 [n_pairs, 2] = (src_block, dst_block)
+ *   src_blocks, dst_blocks  blocks per plane on each side; a pair with an index
+ *                 outside its range is skipped. 0 disables that side's check.
+ * Destination blocks must be distinct (as index_copy_ requires for a
+ * deterministic result); source and destination ranges must not overlap.
+ */
+HFK_API int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs,
+                    const int64_t* block_pairs, uint32_t n_planes, uint64_t n_pairs,
+                    uint64_t block_bytes, uint64_t src_block_stride,
+                    uint64_t dst_block_stride, uint64_t src_blocks, uint64_t dst_blocks,
+                    uint32_t workgroups, hfk_stream_t stream);
+
+/*
+ * Paged block gather over many planes in one launch:
+ *   for p < n_planes, i < n_ids:
+ *     dst_plane_ptrs[p][i*block_bytes ...] = src_plane_ptrs[p][ids[i]*src_block_stride ...]
+ * i.e. hfk_gather_rows applied to every plane with a shared id list
+ * (per plane: dst = src.index_select(0, ids)).
+ * Same reference anchors as hfk_gather_rows; the plane loop is additive.
+ */
+HFK_API int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs,
+                      const int64_t* ids, uint32_t n_planes, uint64_t n_ids,
+                      uint64_t block_bytes, uint64_t src_block_stride,
+                      uint64_t src_blocks, uint32_t workgroups, hfk_stream_t stream);
+
+/*
+ * Benchmark/tuning knobs (process-wide, not thread-safe against concurrent
+ * launches). Defaults are the measured best for MI355X.
+ */
+enum hfk_knob {
+    HFK_KNOB_UNROLL = 0,        /* 16-byte accesses in flight per lane: 1, 2, 4, 8, 16  */
+    HFK_KNOB_NONTEMPORAL = 1,   /* bit0: non-temporal loads, bit1: non-temporal stores */
+    HFK_KNOB_WORKGROUPS_PER_CU = 2 /* default grid bound = CUs * this, 1..64          */
+};
+HFK_API int hfk_set_tuning(int knob, int64_t value);
+HFK_API int64_t hfk_get_tuning(int knob);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HFK_H */

@@ -1,0 +1,328 @@
+// CPU index-math checker for the kernel bodies (test infrastructure).
+//
+// Compiles the exact per-lane bodies and launch planning the GPU library uses
+// (hfk_bodies.h, hfk_plan.h) for the host, walks every (workgroup, lane) pair of a
+// launch sequentially, and compares the bytes with the C oracle. Buffers are sized
+// exactly and the program is built with AddressSanitizer, so an out-of-range lane
+// access aborts the run instead of faulting a GPU later. This never runs in the
+// product; it exists so that indexing mistakes are found before a kernel is ever
+// launched on hardware.
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "hfk.h"
+#include "hfk_bodies.h"
+#include "hfk_plan.h"
+
+extern "C" {
+int oracle_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i64, uint64_t n_ids,
+                       uint64_t row_bytes, uint32_t cores);
+int oracle_multi_layer_block_transfer(void* const* layer_ptrs, const void* src, uint32_t T, uint32_t L,
+                                      uint32_t H, uint32_t D, uint32_t elem_bytes, uint32_t cores);
+int oracle_swap_blocks(void* const* dst_planes, const void* const* src_planes, const int64_t* pairs,
+                       uint32_t n_planes, uint64_t n_pairs, uint64_t block_bytes, uint64_t src_stride,
+                       uint64_t dst_stride);
+}
+
+namespace {
+
+using namespace hfk;
+
+std::mt19937_64 rng(12345);
+int g_failures = 0;
+int g_cases = 0;
+
+// Exactly-sized heap buffer (ASan red zones on both ends), optional misalignment.
+struct Buf {
+    uint8_t* raw = nullptr;
+    uint8_t* p = nullptr;
+    size_t n = 0;
+    Buf(size_t bytes, size_t misalign = 0) : n(bytes) {
+        raw = static_cast<uint8_t*>(std::aligned_alloc(64, ((bytes + misalign + 63) / 64) * 64 + 64));
+        p = raw + misalign;
+    }
+    ~Buf() { std::free(raw); }
+    void randomize() { for (size_t i = 0; i < n; ++i) p[i] = (uint8_t)rng(); }
+    void fill(uint8_t v) { std::memset(p, v, n); }
+    Buf(const Buf&) = delete;
+    Buf& operator=(const Buf&) = delete;
+};
+
+void expect_equal(const uint8_t* a, const uint8_t* b, size_t n, const char* what) {
+    ++g_cases;
+    if (std::memcmp(a, b, n) != 0) {
+        size_t i = 0;
+        while (i < n && a[i] == b[i]) ++i;
+        std::printf("FAIL %s: first difference at byte %zu of %zu\n", what, i, n);
+        ++g_failures;
+    }
+}
+
+template <typename Body, typename Args>
+void walk(const Args& a, uint32_t grid, Body body) {
+    for (uint32_t bid = 0; bid < grid; ++bid)
+        for (uint32_t tid = 0; tid < kWorkgroupLanes; ++tid) body(a, bid, grid, tid);
+}
+
+template <typename IdT, int NT>
+void run_block_copy(BlockCopyArgs<IdT> a, int preferred_unroll, uint32_t grid_cap) {
+    int unroll = 1;
+    if (plan_block_copy<IdT>(a, preferred_unroll, &unroll) != HFK_OK) { std::printf("plan failed\n"); ++g_failures; return; }
+    const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+    switch (unroll) {
+        case 1: walk(a, grid, block_copy_body<IdT, 1, NT>); break;
+        case 2: walk(a, grid, block_copy_body<IdT, 2, NT>); break;
+        case 4: walk(a, grid, block_copy_body<IdT, 4, NT>); break;
+        case 8: walk(a, grid, block_copy_body<IdT, 8, NT>); break;
+        default: walk(a, grid, block_copy_body<IdT, 16, NT>); break;
+    }
+}
+
+template <typename IdT>
+void run_flat_gather(uint64_t table, uint64_t dst, const IdT* ids, uint64_t n_ids, uint64_t row_bytes,
+                     uint64_t limit, uint32_t grid_cap, bool force64) {
+    FlatGatherArgs<IdT> a;
+    FlatGatherPlan p;
+    if (plan_flat_gather<IdT>(a, p, table, dst, ids, n_ids, row_bytes, limit) != HFK_OK) { ++g_failures; return; }
+    const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+    const bool i32 = p.index32 && !force64;
+    if (p.unit == 16u) {
+        if (i32) walk(a, grid, flat_gather_body<vec16, IdT, uint32_t, kFlatUnroll, 3>);
+        else walk(a, grid, flat_gather_body<vec16, IdT, uint64_t, kFlatUnroll, 0>);
+    } else if (p.unit == 4u) {
+        if (i32) walk(a, grid, flat_gather_body<uint32_t, IdT, uint32_t, kFlatUnroll, 0>);
+        else walk(a, grid, flat_gather_body<uint32_t, IdT, uint64_t, kFlatUnroll, 3>);
+    } else {
+        if (i32) walk(a, grid, flat_gather_body<uint8_t, IdT, uint32_t, kFlatUnroll, 0>);
+        else walk(a, grid, flat_gather_body<uint8_t, IdT, uint64_t, kFlatUnroll, 0>);
+    }
+}
+
+// ---- swap_blocks ----------------------------------------------------------
+void case_swap(uint32_t n_planes, uint32_t n_pairs, uint64_t block_bytes, uint64_t src_blocks, uint64_t dst_blocks,
+               uint64_t src_pad, uint64_t dst_pad, size_t src_mis, size_t dst_mis, int unroll, uint32_t grid_cap,
+               bool with_bad_pairs) {
+    const uint64_t ss = block_bytes + src_pad, ds = block_bytes + dst_pad;
+    std::vector<Buf*> src, dst, exp;
+    std::vector<uint64_t> sp, dp;
+    std::vector<void*> ep;
+    std::vector<const void*> spc;
+    for (uint32_t p = 0; p < n_planes; ++p) {
+        src.push_back(new Buf(src_blocks * ss - src_pad, src_mis));
+        dst.push_back(new Buf(dst_blocks * ds - dst_pad, dst_mis));
+        exp.push_back(new Buf(dst_blocks * ds - dst_pad, dst_mis));
+        src.back()->randomize();
+        dst.back()->fill(0xA5);
+        exp.back()->fill(0xA5);
+        sp.push_back((uint64_t)(uintptr_t)src.back()->p);
+        dp.push_back((uint64_t)(uintptr_t)dst.back()->p);
+        ep.push_back(exp.back()->p);
+        spc.push_back(src.back()->p);
+    }
+    // distinct destination blocks
+    std::vector<int64_t> dperm(dst_blocks);
+    for (uint64_t i = 0; i < dst_blocks; ++i) dperm[i] = (int64_t)i;
+    std::shuffle(dperm.begin(), dperm.end(), rng);
+    std::vector<int64_t> pairs, good;
+    for (uint32_t j = 0; j < n_pairs; ++j) {
+        int64_t s = (int64_t)(rng() % src_blocks), d = dperm[j % dst_blocks];
+        bool bad = false;
+        if (with_bad_pairs && j % 5 == 3) { s = (j % 2) ? -1 - (int64_t)(rng() % 7) : (int64_t)src_blocks + (int64_t)(rng() % 9); bad = true; }
+        if (with_bad_pairs && j % 7 == 5) { d = (j % 2) ? (int64_t)dst_blocks : -3; bad = true; }
+        pairs.push_back(s);
+        pairs.push_back(d);
+        if (!bad) { good.push_back(s); good.push_back(d); }
+    }
+    BlockCopyArgs<int64_t> a;
+    int rc = plan_swap_blocks(a, dp.data(), sp.data(), pairs.data(), n_planes, n_pairs, block_bytes, ss, ds,
+                              src_blocks, dst_blocks);
+    if (rc != HFK_OK) { std::printf("plan_swap_blocks rc=%d\n", rc); ++g_failures; }
+    else {
+        run_block_copy<int64_t, 3>(a, unroll, grid_cap);
+        oracle_swap_blocks(ep.data(), spc.data(), good.data(), n_planes, good.size() / 2, block_bytes, ss, ds);
+        char what[160];
+        std::snprintf(what, sizeof what, "swap planes=%u pairs=%u bytes=%llu pad=%llu/%llu mis=%zu/%zu unroll=%d grid=%u bad=%d",
+                      n_planes, n_pairs, (unsigned long long)block_bytes, (unsigned long long)src_pad,
+                      (unsigned long long)dst_pad, src_mis, dst_mis, unroll, grid_cap, (int)with_bad_pairs);
+        for (uint32_t p = 0; p < n_planes; ++p) expect_equal(dst[p]->p, exp[p]->p, dst[p]->n, what);
+    }
+    for (auto* b : src) delete b;
+    for (auto* b : dst) delete b;
+    for (auto* b : exp) delete b;
+}
+
+// ---- gather_blocks (multi-plane, shared ids) -------------------------------
+void case_gather_blocks(uint32_t n_planes, uint32_t n_ids, uint64_t block_bytes, uint64_t src_blocks, int unroll,
+                        uint32_t grid_cap) {
+    std::vector<Buf*> src, dst, exp;
+    std::vector<uint64_t> sp, dp;
+    std::vector<int64_t> ids(n_ids);
+    for (auto& i : ids) i = (int64_t)(rng() % src_blocks);
+    for (uint32_t p = 0; p < n_planes; ++p) {
+        src.push_back(new Buf(src_blocks * block_bytes));
+        dst.push_back(new Buf((uint64_t)n_ids * block_bytes));
+        exp.push_back(new Buf((uint64_t)n_ids * block_bytes));
+        src.back()->randomize();
+        dst.back()->fill(0x11);
+        sp.push_back((uint64_t)(uintptr_t)src.back()->p);
+        dp.push_back((uint64_t)(uintptr_t)dst.back()->p);
+        oracle_gather_rows(src.back()->p, exp.back()->p, ids.data(), 1, n_ids, block_bytes, 3);
+    }
+    BlockCopyArgs<int64_t> a;
+    int rc = plan_gather_blocks(a, dp.data(), sp.data(), ids.data(), n_planes, n_ids, block_bytes, block_bytes, src_blocks);
+    if (rc != HFK_OK) { ++g_failures; std::printf("plan_gather_blocks rc=%d\n", rc); }
+    else {
+        run_block_copy<int64_t, 0>(a, unroll, grid_cap);
+        char what[128];
+        std::snprintf(what, sizeof what, "gather_blocks planes=%u ids=%u bytes=%llu unroll=%d grid=%u", n_planes, n_ids,
+                      (unsigned long long)block_bytes, unroll, grid_cap);
+        for (uint32_t p = 0; p < n_planes; ++p) expect_equal(dst[p]->p, exp[p]->p, dst[p]->n, what);
+    }
+    for (auto* b : src) delete b;
+    for (auto* b : dst) delete b;
+    for (auto* b : exp) delete b;
+}
+
+// ---- gather_rows (both the wide and the flat path, as the entry point picks) --
+template <typename IdT>
+void case_gather_rows(uint64_t table_rows, uint64_t n_ids, uint64_t row_bytes, size_t t_mis, size_t d_mis, int unroll,
+                      uint32_t grid_cap, bool with_bad_ids, bool force64) {
+    Buf table(table_rows * row_bytes, t_mis), dst(n_ids * row_bytes, d_mis), exp(n_ids * row_bytes, d_mis);
+    table.randomize();
+    dst.fill(0x5A);
+    exp.fill(0x5A);
+    std::vector<IdT> ids(n_ids);
+    for (uint64_t i = 0; i < n_ids; ++i) {
+        ids[i] = (IdT)(rng() % table_rows);
+        if (with_bad_ids && i % 4 == 1) ids[i] = (i % 8 == 1) ? (IdT)-2 : (IdT)(table_rows + i);
+    }
+    for (uint64_t i = 0; i < n_ids; ++i) {  // expected: valid rows copied, invalid rows untouched
+        if (ids[i] >= 0 && (uint64_t)ids[i] < table_rows)
+            oracle_gather_rows(table.p, exp.p + i * row_bytes, &ids[i], sizeof(IdT) == 8, 1, row_bytes, 1);
+    }
+    if (row_bytes >= kWideRowBytes) {
+        BlockCopyArgs<IdT> a;
+        if (plan_wide_gather<IdT>(a, table.p, dst.p, ids.data(), n_ids, row_bytes, table_rows) != HFK_OK) { ++g_failures; return; }
+        run_block_copy<IdT, 3>(a, unroll, grid_cap);
+    } else {
+        run_flat_gather<IdT>((uint64_t)(uintptr_t)table.p, (uint64_t)(uintptr_t)dst.p, ids.data(), n_ids, row_bytes,
+                             table_rows, grid_cap, force64);
+    }
+    char what[160];
+    std::snprintf(what, sizeof what, "gather_rows<i%zu> rows=%llu ids=%llu row_bytes=%llu mis=%zu/%zu unroll=%d grid=%u bad=%d f64=%d",
+                  sizeof(IdT) * 8, (unsigned long long)table_rows, (unsigned long long)n_ids,
+                  (unsigned long long)row_bytes, t_mis, d_mis, unroll, grid_cap, (int)with_bad_ids, (int)force64);
+    expect_equal(dst.p, exp.p, dst.n, what);
+}
+
+// ---- transpose -------------------------------------------------------------
+void case_transpose(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem, size_t s_mis, size_t l_mis,
+                    uint32_t grid_cap) {
+    const uint64_t block = (uint64_t)T * L * H * D * elem, layer = (uint64_t)H * T * D * elem;
+    Buf src(block, s_mis);
+    src.randomize();
+    std::vector<Buf*> dst, exp;
+    std::vector<uint64_t> lp;
+    std::vector<void*> ep;
+    for (uint32_t l = 0; l < L; ++l) {
+        dst.push_back(new Buf(layer, l_mis));
+        exp.push_back(new Buf(layer, l_mis));
+        dst.back()->fill(0xEE);
+        exp.back()->fill(0xEE);
+        lp.push_back((uint64_t)(uintptr_t)dst.back()->p);
+        ep.push_back(exp.back()->p);
+    }
+    TransposeArgs a;
+    uint32_t unit = 0;
+    int rc = plan_transpose(a, &unit, lp.data(), src.p, T, L, H, D, elem);
+    if (rc != HFK_OK) { ++g_failures; std::printf("plan_transpose rc=%d\n", rc); }
+    else if (a.n_work > 0) {
+        const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+        if (unit == 16u) walk(a, grid, transpose_body<vec16, kTransposeUnroll, 3>);
+        else if (unit == 4u) walk(a, grid, transpose_body<uint32_t, kTransposeUnroll, 0>);
+        else walk(a, grid, transpose_body<uint8_t, kTransposeUnroll, 0>);
+    }
+    oracle_multi_layer_block_transfer(ep.data(), src.p, T, L, H, D, elem, 3);
+    char what[128];
+    std::snprintf(what, sizeof what, "transpose T=%u L=%u H=%u D=%u elem=%u mis=%zu/%zu grid=%u unit=%u", T, L, H, D, elem,
+                  s_mis, l_mis, grid_cap, unit);
+    for (uint32_t l = 0; l < L; ++l) expect_equal(dst[l]->p, exp[l]->p, layer, what);
+    for (auto* b : dst) delete b;
+    for (auto* b : exp) delete b;
+}
+
+}  // namespace
+
+int main() {
+    // swap: aligned fast path, every unroll, grid smaller and larger than the work
+    for (int unroll : {1, 2, 4, 8, 16})
+        for (uint32_t grid : {1u, 7u, 4096u}) {
+            case_swap(3, 9, 32768, 16, 12, 0, 0, 0, 0, unroll, grid, false);
+            case_swap(2, 5, 73728, 8, 8, 0, 0, 0, 0, unroll, grid, false);   // MLA block: 4.5 chunks at unroll 4
+            case_swap(2, 6, 16384, 10, 9, 0, 0, 0, 0, unroll, grid, true);   // fp8 block + out-of-range pairs
+        }
+    // swap: blocks one vector short of / past a whole number of chunks
+    for (int unroll : {1, 2, 4, 8, 16}) {
+        const uint64_t chunk = 4096ull * unroll;
+        case_swap(2, 3, chunk - 16, 5, 5, 0, 0, 0, 0, unroll, 4, false);
+        case_swap(2, 3, chunk + 16, 5, 5, 0, 0, 0, 0, unroll, 4, false);
+        case_swap(1, 3, 2 * chunk - 16, 4, 4, 0, 0, 0, 0, unroll, 100, false);
+        case_swap(1, 3, 2 * chunk + 4080, 4, 4, 16, 16, 0, 0, unroll, 100, true);
+    }
+    // swap: padded strides, tails that are not a whole chunk, tiny blocks
+    case_swap(2, 7, 4096 + 48, 9, 9, 16, 32, 0, 0, 8, 5, false);
+    case_swap(1, 4, 16, 6, 6, 0, 0, 0, 0, 8, 3, false);
+    case_swap(2, 4, 272, 6, 7, 16, 0, 0, 0, 4, 64, true);
+    // swap: 4-byte and 1-byte paths (size or base not 16-byte aligned)
+    case_swap(2, 5, 5000, 7, 7, 0, 0, 0, 0, 8, 3, false);     // size % 16 != 0, % 4 == 0... 5000 % 8 == 0
+    case_swap(2, 5, 4100, 7, 7, 0, 0, 4, 8, 4, 9, true);      // bases 4-aligned
+    case_swap(2, 5, 4099, 7, 7, 0, 0, 0, 0, 2, 9, false);     // odd size
+    case_swap(1, 3, 8192, 4, 4, 0, 0, 1, 3, 8, 2, false);     // odd bases
+    case_swap(1, 3, 40000, 4, 4, 3, 5, 2, 6, 16, 2, true);    // odd strides
+
+    for (int unroll : {1, 4, 8, 16}) {
+        case_gather_blocks(4, 11, 32768, 20, unroll, 13);
+        case_gather_blocks(3, 6, 16384, 9, unroll, 1000);
+    }
+
+    // gather_rows: wide rows (block-copy path) and narrow rows (flat path)
+    case_gather_rows<int64_t>(64, 32, 32768, 0, 0, 8, 50, false, false);   // config-1 row
+    case_gather_rows<int32_t>(64, 32, 32768, 0, 0, 8, 50, true, false);
+    case_gather_rows<int64_t>(50, 17, 4096, 0, 0, 8, 4, true, false);      // narrowest wide row
+    case_gather_rows<int64_t>(50, 17, 4112, 0, 0, 16, 4, false, false);
+    case_gather_rows<int64_t>(50, 17, 4099, 1, 2, 4, 6, true, false);      // wide, byte path
+    for (bool f64 : {false, true}) {
+        case_gather_rows<int64_t>(500, 333, 1024, 0, 0, 8, 16, false, f64);   // reference's embedding row
+        case_gather_rows<int32_t>(500, 333, 1024, 0, 0, 8, 3, true, f64);
+        case_gather_rows<int64_t>(100, 77, 16, 0, 0, 8, 2, true, f64);        // one vector per row
+        case_gather_rows<int64_t>(100, 1, 48, 0, 0, 8, 2, false, f64);
+        case_gather_rows<int64_t>(100, 77, 4080, 0, 0, 8, 9, false, f64);     // widest flat row
+        case_gather_rows<int64_t>(100, 55, 1020, 0, 0, 8, 5, true, f64);      // 4-byte units
+        case_gather_rows<int32_t>(100, 55, 1024, 4, 8, 8, 5, false, f64);     // 4-byte aligned bases
+        case_gather_rows<int64_t>(100, 55, 999, 0, 0, 8, 5, true, f64);       // byte units
+        case_gather_rows<int64_t>(100, 55, 1, 0, 0, 8, 5, false, f64);
+        case_gather_rows<int32_t>(100, 55, 1024, 1, 0, 8, 700, false, f64);   // odd table base
+    }
+
+    // transpose: the reference's test geometry scaled down, README shapes, odd shapes
+    case_transpose(64, 32, 1, 128, 1, 0, 0, 7);       // int8, H=1 (tests/test_transfer_kernel.py:15-21 with T cut)
+    case_transpose(32, 4, 8, 128, 1, 0, 0, 1000);     // H=8 (README table rows)
+    case_transpose(16, 3, 2, 128, 2, 0, 0, 3);        // bf16
+    case_transpose(5, 3, 2, 64, 4, 0, 0, 2);          // fp32
+    case_transpose(1, 1, 1, 16, 1, 0, 0, 1);
+    case_transpose(7, 1, 1, 128, 2, 0, 0, 2);         // L = H = 1: plain copy
+    case_transpose(9, 2, 3, 20, 2, 0, 0, 5);          // rows of 40 bytes -> 4-byte units
+    case_transpose(9, 2, 3, 7, 1, 0, 0, 5);           // rows of 7 bytes -> byte units
+    case_transpose(9, 2, 3, 16, 2, 0, 4, 5);          // layer buffers only 4-byte aligned: per-unit byte stores
+    case_transpose(9, 2, 3, 16, 2, 4, 0, 5);          // source 4-byte aligned
+    case_transpose(6, 2, 2, 16, 1, 1, 3, 5);          // everything odd
+    case_transpose(0, 2, 2, 16, 1, 0, 0, 5);          // empty block
+
+    std::printf("%d comparisons, %d failures\n", g_cases, g_failures);
+    return g_failures == 0 ? 0 : 1;
+}

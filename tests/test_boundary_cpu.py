@@ -1,0 +1,194 @@
+"""Drop-in boundary checks that need no GPU: the shared libraries load, export every
+symbol the public headers declare, the torch op schemas are the reference's, and the
+host-memory registry behaves like the reference's manager."""
+import ctypes
+import os
+import re
+import subprocess
+import threading
+
+import pytest
+import torch
+
+import heterofusedkernels_amd
+from heterofusedkernels_amd import _build, capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header, macro):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    return sorted(set(re.findall(macro + r"\s+[\w\s\*]+?\b(hfk_\w+)\s*\(", text)))
+
+
+def _exported(so):
+    out = subprocess.check_output(["nm", "-D", "--defined-only", so], text=True)
+    return {line.split()[-1] for line in out.splitlines() if line.strip()}
+
+
+def test_artefacts_exist():
+    for a in _build.artefacts():
+        assert os.path.exists(a), a + " missing: run python -m heterofusedkernels_amd._build"
+
+
+def test_hfk_hip_exports_every_declared_symbol():
+    names = _declared("hfk.h", "HFK_API")
+    assert sorted(names) == sorted(capi.ENTRY_POINTS)
+    assert set(names) <= _exported(_build.HFK_HIP_SO)
+
+
+def test_managed_memory_exports_every_declared_symbol():
+    names = _declared("hfk_managed_memory.h", "HFK_MM_API")
+    assert len(names) == 11
+    assert set(names) <= _exported(_build.MANAGED_MEMORY_SO)
+
+
+def test_capi_loads_and_reports():
+    L = capi.load()
+    assert L.hfk_version() == 1
+    assert capi.status_string(0) == "ok"
+    assert "NULL" in capi.status_string(-1)
+    assert capi.get_tuning(capi.KNOB_UNROLL) in (1, 2, 4, 8, 16)
+    assert capi.set_tuning(capi.KNOB_UNROLL, 3) == -4
+    assert capi.set_tuning(99, 1) == -4
+
+
+def test_argument_errors_are_reported_before_any_gpu_work():
+    # None of these reach a launch, so they are safe without a device.
+    assert capi.gather_rows(0, 0, 0, True, 0, 16) == 0                 # n_ids == 0: no-op
+    assert capi.gather_rows(0, 8, 8, True, 4, 16) == -1                # null table
+    assert capi.gather_rows(8, 8, 8, True, 4, 0) == -2                 # empty rows
+    assert capi.swap_blocks(0, 0, 0, 0, 0, 16, 16, 16) == 0            # nothing to do
+    assert capi.swap_blocks(0, 8, 8, 2, 2, 16, 16, 16) == -1
+    assert capi.swap_blocks(8, 8, 8, 2, 2, 32, 16, 32) == -2           # stride < block
+    assert capi.swap_blocks(8, 8, 8, 2, 2, 0, 16, 32) == -2
+    assert capi.swap_blocks(8, 8, 8, 2, 1 << 33, 16, 16, 16) == -3
+    assert capi.gather_blocks(8, 8, 0, 2, 2, 16, 16) == -1
+    assert capi.gather_blocks(8, 8, 8, 2, 2, 32, 16) == -2
+    assert capi.multi_layer_block_transfer(0, 8, 4, 4, 4, 4, 2) == -1
+    assert capi.multi_layer_block_transfer(8, 8, 4, 4, 4, 4, 0) == -2
+    assert capi.multi_layer_block_transfer(8, 8, 0, 4, 4, 4, 2) == 0   # empty block
+    assert capi.multi_layer_block_transfer(8, 8, 1 << 20, 1 << 10, 8, 128, 2) == -3
+    assert capi.fused_memcpy_multi_layer_block_transfer(8, 8, 0, 4, 4, 4, 4, 2) == -1
+
+
+# ---- torch ops: schemas are the reference's ---------------------------------
+def test_op_schemas_match_reference():
+    import pcie_through  # noqa: F401  (import side effect registers the ops)
+
+    want = {
+        # pcieThrough/csrc/host/gather_torch.cpp:60
+        "gather": "pcie_through::gather(Tensor gmEmbed, Tensor gmEmbedDst, Tensor gmIds, int? aiv=None) -> ()",
+        # pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:113-114
+        "multi_layer_block_transfer": "pcie_through::multi_layer_block_transfer(Tensor deviceBlockCachePtrs, "
+                                      "Tensor hostBlockCache, int? aiv=None) -> ()",
+        "fused_memcpy_multi_layer_block_transfer": "pcie_through::fused_memcpy_multi_layer_block_transfer(Tensor "
+                                                   "deviceBlockCachePtrs, Tensor hostBlockCache, Tensor "
+                                                   "stagingBlockCache, int? aiv=None) -> ()",
+    }
+    for name, schema in want.items():
+        op = getattr(torch.ops.pcie_through, name)
+        assert str(op.default._schema) == schema
+    assert hasattr(torch.ops.pcie_through, "swap_blocks") and hasattr(torch.ops.pcie_through, "gather_blocks")
+
+
+def test_ops_have_no_cpu_fallback():
+    import pcie_through  # noqa: F401
+
+    with pytest.raises(NotImplementedError):
+        torch.ops.pcie_through.gather(torch.zeros(4, 4), torch.zeros(2, 4), torch.zeros(2, dtype=torch.int64))
+    with pytest.raises(NotImplementedError):
+        torch.ops.pcie_through.multi_layer_block_transfer(torch.zeros(2, dtype=torch.int64),
+                                                          torch.zeros(2, 2, 2, 2), 4)
+
+
+def test_package_layout():
+    import pcie_through
+
+    pkg = os.path.dirname(pcie_through.__file__)
+    assert os.path.exists(os.path.join(pkg, "lib", "libpcie_through.so"))   # pcie_through/_load.py:10
+    from heterofusedkernels import memory
+
+    for name in ("alloc_numa_pinned_tensor", "host_register", "get_device_ptr"):  # common/csrc/pybind.cpp:8-10
+        assert callable(getattr(memory, name))
+    assert os.path.dirname(pkg) == heterofusedkernels_amd.DROPIN_DIR
+
+
+# ---- registry (no HIP call is made by adopt / lookup) ------------------------
+@pytest.fixture
+def mm():
+    L = ctypes.CDLL(_build.MANAGED_MEMORY_SO)
+    L.hfk_mm_adopt.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    L.hfk_mm_unregister.argtypes = [ctypes.c_void_p]
+    L.hfk_mm_get_device_ptr.argtypes = [ctypes.c_void_p]
+    L.hfk_mm_get_device_ptr.restype = ctypes.c_void_p
+    L.hfk_mm_record_size.argtypes = [ctypes.c_void_p]
+    L.hfk_mm_record_size.restype = ctypes.c_size_t
+    L.hfk_mm_record_count.restype = ctypes.c_size_t
+    L.hfk_mm_status_string.restype = ctypes.c_char_p
+    L.hfk_mm_unregister_all()
+    yield L
+    L.hfk_mm_unregister_all()
+
+
+def test_registry_range_lookup_and_offsets(mm):
+    # common/csrc/managed_memory/managed_mem.cpp:139-160: interior pointers resolve by offset
+    assert mm.hfk_mm_adopt(0x10000, 0x900000, 0x1000, 0) == 0
+    assert mm.hfk_mm_adopt(0x30000, 0xA00000, 0x2000, 0) == 0
+    assert mm.hfk_mm_get_device_ptr(0x10000) == 0x900000
+    assert mm.hfk_mm_get_device_ptr(0x10fff) == 0x900fff
+    assert mm.hfk_mm_get_device_ptr(0x11000) is None          # one past the end
+    assert mm.hfk_mm_get_device_ptr(0xffff) is None
+    assert mm.hfk_mm_get_device_ptr(0x31234) == 0xA01234
+    assert mm.hfk_mm_get_device_ptr(0) is None                 # :140-142
+    assert mm.hfk_mm_record_size(0x30010) == 0x2000            # :163-179
+    assert mm.hfk_mm_record_size(0x50000) == 0
+    assert mm.hfk_mm_record_count() == 2
+
+
+def test_registry_idempotent_overlap_and_unregister(mm):
+    assert mm.hfk_mm_adopt(0x10000, 0x900000, 0x1000, 0) == 0
+    assert mm.hfk_mm_adopt(0x10000, 0x123456, 0x1000, 0) == 0   # :49-52 same start: existing record kept
+    assert mm.hfk_mm_get_device_ptr(0x10000) == 0x900000
+    assert mm.hfk_mm_adopt(0x10800, 0x777000, 0x1000, 0) == -2  # overlaps a different record
+    assert mm.hfk_mm_adopt(0xf800, 0x777000, 0x1000, 0) == -2
+    assert mm.hfk_mm_adopt(0, 0x777000, 0x1000, 0) == -1        # :46 null / zero size rejected
+    assert mm.hfk_mm_adopt(0x70000, 0x777000, 0, 0) == -1
+    assert mm.hfk_mm_unregister(0x424242) == 0                  # :110-113 unknown pointer is not an error
+    assert mm.hfk_mm_unregister(0x10000) == 0
+    assert mm.hfk_mm_get_device_ptr(0x10000) is None
+    assert mm.hfk_mm_record_count() == 0
+    assert b"overlap" in mm.hfk_mm_status_string(-2)
+
+
+def test_registry_is_thread_safe(mm):
+    # managed_mem.h:31: writers exclude, readers share
+    errors = []
+
+    def worker(k):
+        base = 0x1000000 * (k + 1)
+        try:
+            for i in range(300):
+                host = base + i * 0x2000
+                assert mm.hfk_mm_adopt(host, host + 0x5000000000, 0x1000, k) == 0
+                assert mm.hfk_mm_get_device_ptr(host + 0x10) == host + 0x5000000000 + 0x10
+                if i % 3 == 0:
+                    assert mm.hfk_mm_unregister(host) == 0
+        except AssertionError as exc:  # pragma: no cover
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors
+    assert mm.hfk_mm_record_count() == 8 * 200
+
+
+def test_memory_module_cpu_behaviour():
+    from heterofusedkernels import memory
+
+    assert memory.get_device_ptr(0x1234) == 0                    # managed_mem.cpp:372-375
+    with pytest.raises(RuntimeError, match="Device must be CPU and tensor must be pinned"):
+        memory.host_register(torch.zeros(16))                    # managed_mem.cpp:336-340

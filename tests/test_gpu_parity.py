@@ -1,0 +1,331 @@
+"""GPU parity: the HIP kernels, called through the C-ABI (ctypes) and through the
+torch ops, against the CPU oracle and the committed golden vectors, bit for bit.
+
+Sizes here are ones the oracle finishes in seconds; the full-size configurations
+are covered by tests/test_gpu_fullsize.py through size-independent properties.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from heterofusedkernels_amd import capi
+from heterofusedkernels_amd import workloads as W
+from oracle import oracle as O
+
+from gpu_helpers import (announce, bytes_np, gather_blocks, gather_rows, host_ptr_table, ptr_table, stream_handle,
+                         swap)
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda"
+
+
+def _golden(prefix):
+    return [(os.path.basename(f), f) for f in sorted(glob.glob(os.path.join(GOLDEN, prefix + "_*.npz")))]
+
+
+@pytest.fixture(scope="module")
+def memory():
+    import heterofusedkernels_amd  # noqa: F401
+    import pcie_through  # noqa: F401
+    from heterofusedkernels import memory as m
+
+    return m
+
+
+def _pinned(memory, nbytes, fill=None):
+    t = memory.alloc_numa_pinned_tensor(nbytes)
+    assert t.is_pinned() and t.device.type == "cpu" and t.dtype == torch.int8 and t.dim() == 1
+    if fill is not None:
+        t.view(torch.uint8).fill_(fill)
+    return t
+
+
+# ---------------------------------------------------------------------------
+# golden vectors through the C-ABI
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("name,path", _golden("gather"))
+def test_golden_gather(name, path):
+    announce("golden gather " + name)
+    g = np.load(path)
+    table = torch.from_numpy(g["table"]).to(DEV)
+    ids = torch.from_numpy(g["ids"]).to(DEV)
+    dst = torch.full(g["expected"].shape, 0xEE, dtype=torch.uint8, device=DEV)
+    gather_rows(table, dst, ids, table.shape[1], table_rows=table.shape[0])
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.cpu().numpy(), g["expected"])
+
+
+@pytest.mark.parametrize("name,path", _golden("swap"))
+def test_golden_swap(name, path):
+    announce("golden swap " + name)
+    g = np.load(path)
+    planes, sblocks, bb = g["src"].shape
+    dblocks = g["dst_before"].shape[1]
+    src = [torch.from_numpy(np.ascontiguousarray(g["src"][p])).to(DEV) for p in range(planes)]
+    dst = [torch.from_numpy(g["dst_before"][p].copy()).to(DEV) for p in range(planes)]
+    pairs = torch.from_numpy(g["pairs"]).to(DEV)
+    swap(ptr_table(dst), ptr_table(src), pairs, planes, bb, src_blocks=sblocks, dst_blocks=dblocks)
+    torch.cuda.synchronize()
+    got = np.stack([d.cpu().numpy() for d in dst])
+    assert np.array_equal(got, g["expected"])
+
+
+@pytest.mark.parametrize("name,path", _golden("transfer"))
+def test_golden_transfer(name, path):
+    announce("golden transfer " + name)
+    g = np.load(path)
+    T, L, H, D, e = (int(x) for x in g["geometry"])
+    src = torch.from_numpy(g["src"]).to(DEV)
+    layers = torch.full((L, H * T * D * e), 0xEE, dtype=torch.uint8, device=DEV)
+    ptrs = ptr_table([layers[l] for l in range(L)])
+    capi.check(capi.multi_layer_block_transfer(ptrs.data_ptr(), src.data_ptr(), T, L, H, D, e, 0, stream_handle()))
+    torch.cuda.synchronize()
+    assert np.array_equal(layers.cpu().numpy(), g["expected"])
+
+
+# ---------------------------------------------------------------------------
+# configuration 1: single-layer paged KV gather, exact sizes
+# ---------------------------------------------------------------------------
+def test_config1_gather_fp16_exact():
+    cfg = W.C1_GATHER_FP16
+    announce("config 1 gather K and V [1024,16,8,128] fp16, 32 ids")
+    ids = W.gather_ids(cfg)
+    assert ids.numel() == 32 and ids.unique().numel() == 32
+    for kv in range(cfg.kv):
+        plane = W.make_plane(cfg, 0, kv, cfg.dev_blocks)
+        want = O.torch_gather_rows(plane, ids)                       # the CPU torch path
+        out = torch.zeros((32,) + cfg.block_shape, dtype=cfg.dtype, device=DEV)
+        gather_rows(plane.to(DEV), out, ids.to(DEV), cfg.block_bytes, table_rows=cfg.dev_blocks)
+        torch.cuda.synchronize()
+        assert np.array_equal(bytes_np(out), bytes_np(want))
+        assert np.array_equal(bytes_np(out), O.c_gather_rows(bytes_np(plane), ids.numpy()))
+        # same through the torch op, with the table viewed as [blocks, 16384] like an embedding table
+        out2 = torch.zeros(32, cfg.block_elems, dtype=cfg.dtype, device=DEV)
+        torch.ops.pcie_through.gather(plane.view(cfg.dev_blocks, -1).to(DEV), out2, ids.to(DEV), aiv=4)
+        torch.cuda.synchronize()
+        assert np.array_equal(bytes_np(out2), bytes_np(want))
+
+
+# ---------------------------------------------------------------------------
+# gather from host-registered memory (the reference's embedding use)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("bs", [1, 16, 256, 1024])
+@pytest.mark.parametrize("id_dtype", [torch.int64, torch.int32])
+def test_gather_from_registered_host_table(memory, bs, id_dtype):
+    rows, dim = 20000, 512                                     # fp16 rows of 1 KiB (tests/test_gather.py:35-41)
+    announce("host-table gather bs=%d ids=%s" % (bs, id_dtype))
+    embed = _pinned(memory, rows * dim * 2).view(torch.float16).view(rows, dim)
+    gen = torch.Generator().manual_seed(bs)
+    embed.copy_(torch.randn(rows, dim, generator=gen).to(torch.float16))
+    ids = torch.randint(0, rows, (bs,), generator=gen, dtype=torch.int64).to(id_dtype)
+    dst = torch.zeros(bs, dim, dtype=torch.float16, device=DEV)
+    torch.ops.pcie_through.gather(embed, dst, ids.to(DEV), aiv=4)        # keyword aiv (tests/test_gather.py:56)
+    torch.cuda.synchronize()
+    want = embed[ids.to(torch.int64)]                                    # tests/test_memcpy.py:18
+    assert np.array_equal(bytes_np(dst), bytes_np(want))
+    dst2 = torch.zeros_like(dst)
+    torch.ops.pcie_through.gather(embed, dst2, ids.to(DEV))              # default aiv (test_gather_combine.py:51-55)
+    torch.cuda.synchronize()
+    assert torch.equal(dst2.cpu().view(torch.int16), dst.cpu().view(torch.int16))
+
+
+# ---------------------------------------------------------------------------
+# configurations 2-5, scaled: block-table swap against index_select / index_copy_
+# ---------------------------------------------------------------------------
+def _host_pool(memory, cfg, blocks, fill=0x5C):
+    pool = _pinned(memory, cfg.planes * blocks * cfg.block_bytes, fill=fill)
+    return pool, list(pool.view(torch.uint8).view(cfg.planes, blocks, cfg.block_bytes).unbind(0))
+
+
+def _cpu_planes(cfg, blocks):
+    return [W.make_plane(cfg, l, kv, blocks) for l in range(cfg.layers) for kv in range(cfg.kv)]
+
+
+def test_config2_swap_out_scaled(memory):
+    cfg = W.C2_LLAMA8B_SWAP_OUT.scaled(layers=4, dev_blocks=256, host_blocks=512, n_blocks=64)
+    announce("config 2 scaled swap-out: %d planes, %d pairs, %d B blocks" % (cfg.planes, cfg.n_blocks, cfg.block_bytes))
+    cpu = _cpu_planes(cfg, cfg.dev_blocks)
+    dev = [p.to(DEV) for p in cpu]
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks)
+    src_ids, dst_ids = W.block_table(cfg, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    pairs = W.pairs_tensor(src_ids, dst_ids)
+    swap(host_ptr_table(host), ptr_table(dev), pairs.to(DEV), cfg.planes, cfg.block_bytes,
+         src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.host_blocks, cfg.block_bytes), 0x5C, dtype=torch.uint8)
+        O.torch_swap_blocks(want, W.as_bytes(cpu[p]), src_ids, dst_ids)      # index_copy_(index_select)
+        assert torch.equal(host[p], want), "plane %d" % p                     # incl. every untouched slot
+        assert torch.equal(W.as_bytes(dev[p].cpu()), W.as_bytes(cpu[p]))      # source unchanged
+    # C restatement agrees as well
+    want_c = [np.full((cfg.host_blocks, cfg.block_bytes), 0x5C, dtype=np.uint8) for _ in range(cfg.planes)]
+    O.c_swap_blocks(want_c, [bytes_np(p) for p in cpu], pairs.numpy())
+    for p in range(cfg.planes):
+        assert np.array_equal(host[p].numpy(), want_c[p])
+
+
+def test_config3_swap_in_scaled(memory):
+    cfg = W.C3_LLAMA70B_SWAP_IN.scaled(layers=5, dev_blocks=256, host_blocks=512, n_blocks=96)
+    announce("config 3 scaled swap-in: %d planes, %d pairs" % (cfg.planes, cfg.n_blocks))
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=None)
+    cpu_host = _cpu_planes(cfg, cfg.host_blocks)
+    for p in range(cfg.planes):
+        host[p].copy_(W.as_bytes(cpu_host[p]))
+    dev = [torch.full((cfg.dev_blocks, cfg.block_bytes), 0x6D, dtype=torch.uint8, device=DEV) for _ in range(cfg.planes)]
+    gen = torch.Generator().manual_seed(33)
+    perm = torch.randperm(cfg.host_blocks, generator=gen)             # block table as a permutation slice
+    src_ids = perm[:cfg.n_blocks].contiguous()
+    dst_ids = torch.randperm(cfg.dev_blocks, generator=gen)[:cfg.n_blocks].contiguous()
+    swap(ptr_table(dev), host_ptr_table(host), W.pairs_tensor(src_ids, dst_ids).to(DEV), cfg.planes, cfg.block_bytes,
+         src_blocks=cfg.host_blocks, dst_blocks=cfg.dev_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.dev_blocks, cfg.block_bytes), 0x6D, dtype=torch.uint8)
+        O.torch_swap_blocks(want, W.as_bytes(cpu_host[p]), src_ids, dst_ids)
+        assert torch.equal(dev[p].cpu(), want), "plane %d" % p
+        assert torch.equal(host[p], W.as_bytes(cpu_host[p]))
+
+
+def test_config4_mla_round_trip_scaled(memory):
+    cfg = W.C4_MLA_ROUNDTRIP.scaled(layers=7, dev_blocks=64, host_blocks=64, n_blocks=16)
+    assert cfg.block_bytes == 73728
+    announce("config 4 scaled MLA round trip: %d planes, block %d B" % (cfg.planes, cfg.block_bytes))
+    cpu = _cpu_planes(cfg, cfg.dev_blocks)
+    dev = [p.to(DEV) for p in cpu]
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0)
+    gen = torch.Generator().manual_seed(44)
+    out_src = torch.randperm(cfg.dev_blocks, generator=gen)[:cfg.n_blocks]
+    host_slots = torch.randperm(cfg.host_blocks, generator=gen)[:cfg.n_blocks]
+    free = torch.tensor([b for b in range(cfg.dev_blocks) if b not in set(out_src.tolist())])
+    in_dst = free[torch.randperm(len(free), generator=gen)[:cfg.n_blocks]]   # different slots
+    dtab, htab = ptr_table(dev), host_ptr_table(host)
+    swap(htab, dtab, W.pairs_tensor(out_src, host_slots).to(DEV), cfg.planes, cfg.block_bytes,
+         src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    swap(dtab, htab, W.pairs_tensor(host_slots, in_dst).to(DEV), cfg.planes, cfg.block_bytes,
+         src_blocks=cfg.host_blocks, dst_blocks=cfg.dev_blocks)               # same stream: ordered after swap-out
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        got = W.as_bytes(dev[p].cpu())
+        orig = W.as_bytes(cpu[p])
+        assert torch.equal(got[in_dst], orig[out_src]), "plane %d round trip" % p
+        untouched = torch.ones(cfg.dev_blocks, dtype=torch.bool)
+        untouched[in_dst] = False
+        assert torch.equal(got[untouched], orig[untouched])
+
+
+def test_config5_fp8_fragmented_scaled(memory):
+    cfg = W.C5_FP8_FRAGMENTED.scaled(layers=3, dev_blocks=512, host_blocks=512, n_blocks=256)
+    announce("config 5 scaled fp8 fragmented gather + swap-out: %d planes, %d ids" % (cfg.planes, cfg.n_blocks))
+    ids = W.fragmented_ids(cfg.dev_blocks, cfg.n_blocks)
+    cpu = _cpu_planes(cfg, cfg.dev_blocks)
+    dev = [p.to(DEV) for p in cpu]
+    prefill = [torch.zeros(cfg.n_blocks, cfg.block_bytes, dtype=torch.uint8, device=DEV) for _ in range(cfg.planes)]
+    gather_blocks(ptr_table(prefill), ptr_table(dev), ids.to(DEV), cfg.planes, cfg.block_bytes,
+                  src_blocks=cfg.dev_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = O.torch_gather_rows(W.as_bytes(cpu[p]), ids)
+        assert torch.equal(prefill[p].cpu(), want), "plane %d" % p
+    # matching swap-out of the same ids to host slots 0..n-1
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0x11)
+    pairs = W.pairs_tensor(ids, torch.arange(cfg.n_blocks))
+    swap(host_ptr_table(host), ptr_table(dev), pairs.to(DEV), cfg.planes, cfg.block_bytes,
+         src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        assert torch.equal(host[p][:cfg.n_blocks], prefill[p].cpu())
+        assert (host[p][cfg.n_blocks:] == 0x11).all()
+    # through the torch op too
+    prefill2 = [torch.zeros_like(x) for x in prefill]
+    torch.ops.pcie_through.gather_blocks(ptr_table(prefill2), ptr_table(dev), ids.to(DEV), cfg.block_bytes,
+                                         cfg.block_bytes, cfg.dev_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        assert torch.equal(prefill2[p], prefill[p])
+
+
+# ---------------------------------------------------------------------------
+# edge cases
+# ---------------------------------------------------------------------------
+def test_empty_and_out_of_range():
+    announce("edge: empty inputs and out-of-range ids")
+    table = torch.arange(64 * 32, dtype=torch.int32, device=DEV).view(64, 32)        # 128-byte rows
+    dst = torch.full((6, 32), -1, dtype=torch.int32, device=DEV)
+    ids = torch.tensor([5, -1, 63, 64, 0, 1 << 40], dtype=torch.int64, device=DEV)
+    gather_rows(table, dst, ids, 128, table_rows=64)
+    torch.cuda.synchronize()
+    got = dst.cpu()
+    assert torch.equal(got[0], table[5].cpu()) and torch.equal(got[2], table[63].cpu()) and torch.equal(got[4], table[0].cpu())
+    assert (got[1] == -1).all() and (got[3] == -1).all() and (got[5] == -1).all()
+    empty = torch.zeros(0, dtype=torch.int64, device=DEV)
+    assert capi.gather_rows(table.data_ptr(), dst.data_ptr(), empty.data_ptr(), True, 0, 128, 64, 0, stream_handle()) == 0
+    torch.ops.pcie_through.gather(table, dst, empty)
+    # swap: pairs with an out-of-range side are skipped, the rest copied
+    src = [torch.randint(0, 255, (8, 4096), dtype=torch.uint8, device=DEV)]
+    dstp = [torch.zeros(8, 4096, dtype=torch.uint8, device=DEV)]
+    pairs = torch.tensor([[1, 2], [8, 3], [2, -1], [3, 8], [4, 5]], dtype=torch.int64, device=DEV)
+    swap(ptr_table(dstp), ptr_table(src), pairs, 1, 4096, src_blocks=8, dst_blocks=8)
+    torch.cuda.synchronize()
+    d, s = dstp[0].cpu(), src[0].cpu()
+    assert torch.equal(d[2], s[1]) and torch.equal(d[5], s[4])
+    assert (d[[0, 1, 3, 4, 6, 7]] == 0).all()
+
+
+@pytest.mark.parametrize("row_bytes", [1, 7, 33, 100, 1000, 4095, 4099, 8212, 65536 + 4])
+def test_ragged_row_sizes(row_bytes):
+    announce("edge: ragged rows of %d bytes" % row_bytes)
+    rs = np.random.RandomState(row_bytes)
+    table = rs.randint(0, 256, size=(97, row_bytes)).astype(np.uint8)
+    ids = rs.randint(0, 97, size=53).astype(np.int64)
+    t_dev, i_dev = torch.from_numpy(table).to(DEV), torch.from_numpy(ids).to(DEV)
+    dst = torch.zeros(53, row_bytes, dtype=torch.uint8, device=DEV)
+    gather_rows(t_dev, dst, i_dev, row_bytes, table_rows=97)
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.cpu().numpy(), O.c_gather_rows(table, ids))
+
+
+def test_results_independent_of_tuning_and_grid():
+    announce("edge: every unroll / non-temporal / grid setting gives the same bytes")
+    cfg = W.C4_MLA_ROUNDTRIP.scaled(layers=2, dev_blocks=16, host_blocks=16, n_blocks=9)
+    cpu = _cpu_planes(cfg, cfg.dev_blocks)
+    dev = [p.to(DEV) for p in cpu]
+    src_ids, dst_ids = W.block_table(cfg, src_blocks=16, dst_blocks=16)
+    pairs = W.pairs_tensor(src_ids, dst_ids).to(DEV)
+    want = []
+    for p in range(cfg.planes):
+        w = torch.zeros(16, cfg.block_bytes, dtype=torch.uint8)
+        O.torch_swap_blocks(w, W.as_bytes(cpu[p]), src_ids, dst_ids)
+        want.append(w)
+    saved = [capi.get_tuning(k) for k in range(3)]
+    try:
+        for unroll in (1, 2, 4, 8, 16):
+            for nt in (0, 1, 2, 3):
+                for wgs in (0, 1, 5, 100000):
+                    assert capi.set_tuning(capi.KNOB_UNROLL, unroll) == 0
+                    assert capi.set_tuning(capi.KNOB_NONTEMPORAL, nt) == 0
+                    out = [torch.zeros(16, cfg.block_bytes, dtype=torch.uint8, device=DEV) for _ in range(cfg.planes)]
+                    swap(ptr_table(out), ptr_table(dev), pairs, cfg.planes, cfg.block_bytes, workgroups=wgs)
+                    torch.cuda.synchronize()
+                    for p in range(cfg.planes):
+                        assert torch.equal(out[p].cpu(), want[p]), (unroll, nt, wgs, p)
+    finally:
+        for k, v in enumerate(saved):
+            capi.set_tuning(k, v)
+
+
+def test_strided_planes():
+    announce("edge: block stride larger than block bytes on both sides")
+    src = torch.randint(0, 255, (10, 3, 2048), dtype=torch.uint8, device=DEV)    # use [:, 0, :] -> stride 6144
+    dst = torch.zeros(12, 2, 2048, dtype=torch.uint8, device=DEV)                # use [:, 1, :] -> stride 4096
+    pairs = torch.tensor([[0, 11], [9, 0], [4, 4]], dtype=torch.int64, device=DEV)
+    dst_tab = torch.tensor([dst[0, 1].data_ptr()], dtype=torch.int64, device=DEV)
+    src_tab = torch.tensor([src[0, 0].data_ptr()], dtype=torch.int64, device=DEV)
+    swap(dst_tab, src_tab, pairs, 1, 2048, src_stride=6144, dst_stride=4096, src_blocks=10, dst_blocks=12)
+    torch.cuda.synchronize()
+    d, s = dst.cpu(), src.cpu()
+    assert torch.equal(d[11, 1], s[0, 0]) and torch.equal(d[0, 1], s[9, 0]) and torch.equal(d[4, 1], s[4, 0])
+    assert (d[:, 0] == 0).all() and d[:, 1].sum() == s[[0, 9, 4], 0].sum()

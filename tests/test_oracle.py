@@ -1,0 +1,206 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Each oracle function is checked against (1) the committed golden vectors, which
+come from independent element loops, (2) the expected-value expressions of the
+reference's own tests, (3) closed forms and invariants, (4) the torch CPU
+index_select / index_copy_ statement. No GPU involved.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from heterofusedkernels_amd import workloads as W
+from oracle import oracle as O
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _load(prefix):
+    files = sorted(glob.glob(os.path.join(GOLDEN, prefix + "_*.npz")))
+    assert files, "no golden files for " + prefix
+    return [(os.path.basename(f), np.load(f)) for f in files]
+
+
+# ---- golden vectors ---------------------------------------------------------
+@pytest.mark.parametrize("name,g", _load("transfer"))
+def test_transfer_matches_golden(name, g):
+    T, L, H, D, e = (int(x) for x in g["geometry"])
+    for cores in (1, 2, 3, 4, 64):
+        out = O.c_multi_layer_block_transfer(g["src"], T, L, H, D, e, cores=cores)
+        assert np.array_equal(out, g["expected"]), (name, cores)
+    # torch statement on the same bytes (elements as e-byte groups)
+    host = torch.from_numpy(g["src"].copy()).view(T, L, H, D * e)
+    layers = O.torch_multi_layer_block_transfer(host)
+    got = np.stack([x.numpy().reshape(-1) for x in layers])
+    assert np.array_equal(got, g["expected"]), name
+
+
+@pytest.mark.parametrize("name,g", _load("gather"))
+def test_gather_matches_golden(name, g):
+    for cores in (1, 2, 5, 1000):
+        assert np.array_equal(O.c_gather_rows(g["table"], g["ids"], cores=cores), g["expected"]), (name, cores)
+    got = O.torch_gather_rows(torch.from_numpy(g["table"]), torch.from_numpy(g["ids"]))
+    assert np.array_equal(got.numpy(), g["expected"]), name
+
+
+@pytest.mark.parametrize("name,g", _load("swap"))
+def test_swap_matches_golden(name, g):
+    planes = g["src"].shape[0]
+    dst = [g["dst_before"][p].copy() for p in range(planes)]
+    src = [np.ascontiguousarray(g["src"][p]) for p in range(planes)]
+    O.c_swap_blocks(dst, src, g["pairs"])
+    assert np.array_equal(np.stack(dst), g["expected"]), name
+    pairs = torch.from_numpy(g["pairs"])
+    for p in range(planes):
+        d = torch.from_numpy(g["dst_before"][p].copy())
+        O.torch_swap_blocks(d, torch.from_numpy(src[p]), pairs[:, 0], pairs[:, 1])
+        assert np.array_equal(d.numpy(), g["expected"][p]), (name, p)
+
+
+# ---- the reference tests' own expected-value expressions --------------------
+@pytest.mark.parametrize("T,L,H,D,dtype", [
+    (64, 32, 1, 128, torch.int8),      # tests/test_transfer_kernel.py:15-21 geometry, T cut from 1024
+    (32, 4, 8, 128, torch.int8),       # H = 8 rows of tests/README.md:73,75
+    (16, 3, 2, 64, torch.bfloat16),
+    (8, 2, 2, 32, torch.float16),
+    (8, 2, 2, 32, torch.float32),
+])
+def test_transfer_satisfies_reference_permute_check(T, L, H, D, dtype):
+    """tests/test_transfer_kernel.py:77-83: device block [L,H,T,D] permuted (2,0,1,3) == host block.
+    The reference fills the host pool with a constant (:32); random bytes are used here."""
+    e = torch.empty((), dtype=dtype).element_size()
+    rs = np.random.RandomState(T * 1000 + L)
+    src = rs.randint(0, 256, size=T * L * H * D * e).astype(np.uint8)
+    out = O.c_multi_layer_block_transfer(src, T, L, H, D, e, cores=4)
+    dev_block = torch.from_numpy(out).view(L, H, T, D * e)
+    host_block = torch.from_numpy(src).view(T, L, H, D * e)
+    assert torch.equal(dev_block.permute(2, 0, 1, 3), host_block)
+
+
+def test_gather_satisfies_reference_verify_loop():
+    """tests/test_gather.py:14-29: for every i, table[ids[i]] == dst[i]."""
+    rs = np.random.RandomState(7)
+    table = rs.randint(0, 256, size=(301, 1024)).astype(np.uint8)   # 512 fp16 elements per row
+    ids = rs.randint(0, 301, size=128).astype(np.int64)
+    dst = O.c_gather_rows(table, ids, cores=4)
+    for i in range(len(ids)):
+        assert np.array_equal(table[ids[i]], dst[i])
+
+
+# ---- closed forms and invariants --------------------------------------------
+def test_gather_identity_ids_is_memcpy():
+    rs = np.random.RandomState(1)
+    table = rs.randint(0, 256, size=(40, 96)).astype(np.uint8)
+    assert np.array_equal(O.c_gather_rows(table, np.arange(40, dtype=np.int64)), table)
+    assert np.array_equal(O.c_gather_rows(table, np.arange(39, -1, -1, dtype=np.int32)), table[::-1])
+
+
+def test_gather_repeated_ids_and_empty():
+    rs = np.random.RandomState(2)
+    table = rs.randint(0, 256, size=(5, 32)).astype(np.uint8)
+    ids = np.array([3, 3, 0, 3], dtype=np.int64)
+    assert np.array_equal(O.c_gather_rows(table, ids), table[[3, 3, 0, 3]])
+    assert O.c_gather_rows(table, np.zeros(0, dtype=np.int64)).shape == (0, 32)
+
+
+def test_transfer_single_layer_single_head_is_memcpy():
+    rs = np.random.RandomState(3)
+    src = rs.randint(0, 256, size=9 * 64 * 2).astype(np.uint8)
+    out = O.c_multi_layer_block_transfer(src, 9, 1, 1, 64, 2, cores=2)
+    assert np.array_equal(out[0], src)
+
+
+def test_transfer_is_a_permutation_of_rows_and_touches_every_byte():
+    T, L, H, D, e = 6, 3, 4, 16, 2
+    # every row gets a unique tag so the multiset of rows must be preserved exactly
+    src = np.zeros((T * L * H, D * e), dtype=np.uint8)
+    src[:, 0] = np.arange(T * L * H) % 251
+    src[:, 1] = np.arange(T * L * H) // 251
+    src[:, 2:] = 0x77
+    out = O.c_multi_layer_block_transfer(src.reshape(-1), T, L, H, D, e, cores=2, fill=0xFF)
+    rows = out.reshape(-1, D * e)
+    assert sorted(map(bytes, rows)) == sorted(map(bytes, src))
+    assert not (rows[:, 2] == 0xFF).any()
+
+
+def test_swap_single_pair_is_slice_copy_and_leaves_rest_untouched():
+    rs = np.random.RandomState(4)
+    src = rs.randint(0, 256, size=(6, 48)).astype(np.uint8)
+    dst = np.full((7, 48), 0xCD, dtype=np.uint8)
+    O.c_swap_blocks([dst], [src], np.array([[2, 5]], dtype=np.int64))
+    assert np.array_equal(dst[5], src[2])
+    mask = np.ones(7, dtype=bool)
+    mask[5] = False
+    assert (dst[mask] == 0xCD).all()
+
+
+def test_swap_out_then_in_round_trip_is_identity():
+    rs = np.random.RandomState(5)
+    dev = [rs.randint(0, 256, size=(12, 64)).astype(np.uint8) for _ in range(3)]
+    original = [d.copy() for d in dev]
+    host = [np.zeros((9, 64), dtype=np.uint8) for _ in range(3)]
+    src_ids = rs.permutation(12)[:5]
+    host_ids = rs.permutation(9)[:5]
+    back_ids = rs.permutation(12)[:5]
+    O.c_swap_blocks(host, dev, np.stack([src_ids, host_ids], 1))
+    O.c_swap_blocks(dev, host, np.stack([host_ids, back_ids], 1))
+    for p in range(3):
+        assert np.array_equal(dev[p][back_ids], original[p][src_ids])
+
+
+# ---- C restatement == torch CPU path on the scaled benchmark configurations -----
+@pytest.mark.parametrize("cfg", [
+    W.C1_GATHER_FP16.scaled(dev_blocks=64, n_blocks=32),
+    W.C5_FP8_FRAGMENTED.scaled(layers=2, dev_blocks=128, n_blocks=64),
+])
+def test_c_gather_equals_torch_on_configs(cfg):
+    ids = W.fragmented_ids(cfg.dev_blocks, cfg.n_blocks) if cfg.dist == "bytes" else W.gather_ids(cfg)
+    for layer in range(cfg.layers):
+        for kv in range(cfg.kv):
+            plane = W.make_plane(cfg, layer, kv, cfg.dev_blocks)
+            table = W.as_bytes(plane)
+            want = O.torch_gather_rows(table, ids)
+            got = O.c_gather_rows(table.numpy(), ids.numpy())
+            assert np.array_equal(got, want.numpy())
+            if cfg.dtype != torch.float8_e4m3fn:   # same statement on the typed tensor
+                typed = O.torch_gather_rows(plane, ids)
+                assert torch.equal(W.as_bytes(typed), want)
+
+
+@pytest.mark.parametrize("cfg", [
+    W.C2_LLAMA8B_SWAP_OUT.scaled(layers=2, dev_blocks=48, host_blocks=96, n_blocks=16),
+    W.C3_LLAMA70B_SWAP_IN.scaled(layers=3, dev_blocks=64, host_blocks=128, n_blocks=24),
+    W.C4_MLA_ROUNDTRIP.scaled(layers=3, dev_blocks=24, host_blocks=24, n_blocks=8),
+])
+def test_c_swap_equals_torch_on_configs(cfg):
+    src_ids, dst_ids = W.block_table(cfg, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    pairs = W.pairs_tensor(src_ids, dst_ids)
+    for layer in range(cfg.layers):
+        for kv in range(cfg.kv):
+            src = W.make_plane(cfg, layer, kv, cfg.dev_blocks)
+            dst_t = torch.full((cfg.host_blocks,) + tuple(cfg.block_shape), 1.5, dtype=cfg.dtype)
+            dst_c = W.as_bytes(dst_t).numpy().copy()
+            O.torch_swap_blocks(dst_t, src, src_ids, dst_ids)
+            O.c_swap_blocks([dst_c], [W.as_bytes(src).numpy()], pairs.numpy())
+            assert np.array_equal(dst_c, W.as_bytes(dst_t).numpy())
+
+
+def test_brute_force_agrees_on_tiny_shapes():
+    rs = np.random.RandomState(9)
+    src = rs.randint(0, 256, size=3 * 2 * 2 * 4 * 2).astype(np.uint8)
+    assert np.array_equal(O.brute_multi_layer_block_transfer(src, 3, 2, 2, 4, 2),
+                          O.c_multi_layer_block_transfer(src, 3, 2, 2, 4, 2, cores=2))
+    table = rs.randint(0, 256, size=(5, 12)).astype(np.uint8)
+    ids = np.array([4, 0, 2], dtype=np.int64)
+    assert np.array_equal(O.brute_gather_rows(table, ids), O.c_gather_rows(table, ids))
+
+
+def test_fragmented_ids_shape():
+    ids = W.fragmented_ids(8192, 4096)
+    assert ids.dtype == torch.int64 and ids.numel() == 4096 and ids.unique().numel() == 4096
+    assert int(ids.min()) >= 0 and int(ids.max()) < 8192
+    runs = (ids[1:] != ids[:-1] + 1).sum().item() + 1
+    assert 500 < runs < 4096      # mixture of runs (mean length 4) and isolated blocks
