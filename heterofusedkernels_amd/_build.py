@@ -4,6 +4,7 @@ Artefacts (all in-tree, git-ignored):
 
     dropin/pcie_through/lib/libhfk_hip.so        gfx950 kernels + C-ABI (hipcc)
     dropin/pcie_through/lib/libpcie_through.so   torch dispatcher ops
+    dropin/pcie_through/lib/libhfk_bench.so      benchmark-only comparison paths
     dropin/heterofusedkernels/libmanaged_memory.so   host-memory registry + allocator
     dropin/heterofusedkernels/memory*.so         Python module heterofusedkernels.memory
     dropin/heterofusedkernels/include/*.h        headers shipped for native users
@@ -29,6 +30,7 @@ GPU_ARCH = "gfx950"
 
 HFK_HIP_SO = os.path.join(PCIE_LIB, "libhfk_hip.so")
 PCIE_THROUGH_SO = os.path.join(PCIE_LIB, "libpcie_through.so")
+HFK_BENCH_SO = os.path.join(PCIE_LIB, "libhfk_bench.so")
 MANAGED_MEMORY_SO = os.path.join(COMMON, "libmanaged_memory.so")
 MEMORY_EXT_SO = os.path.join(COMMON, "memory" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 
@@ -57,6 +59,18 @@ def build_hfk_hip():
             "-I" + INCLUDE, "-I" + CSRC, os.path.join(CSRC, "hfk_capi.hip"), "-o", HFK_HIP_SO,
         ],
         quiet_patterns=("packed-fp32-ops' is not a recognized feature",),
+    )
+
+
+def build_bench_support():
+    """Comparison paths used by bench.py only (per-block hipMemcpyAsync loop)."""
+    os.makedirs(PCIE_LIB, exist_ok=True)
+    _run(
+        [
+            "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-D__HIP_PLATFORM_AMD__=1",
+            "-I" + os.path.join(ROCM, "include"), os.path.join(CSRC, "bench_support.cpp"), "-o", HFK_BENCH_SO,
+            "-L" + os.path.join(ROCM, "lib"), "-lamdhip64",
+        ]
     )
 
 
@@ -116,13 +130,14 @@ def build_pcie_through():
 def build_all():
     """Compile everything, every time it is called."""
     build_hfk_hip()
+    build_bench_support()
     build_managed_memory()
     build_memory_ext()
     build_pcie_through()
 
 
 def artefacts():
-    return [HFK_HIP_SO, PCIE_THROUGH_SO, MANAGED_MEMORY_SO, MEMORY_EXT_SO]
+    return [HFK_HIP_SO, HFK_BENCH_SO, PCIE_THROUGH_SO, MANAGED_MEMORY_SO, MEMORY_EXT_SO]
 
 
 if __name__ == "__main__":

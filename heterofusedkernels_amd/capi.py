@@ -14,6 +14,7 @@ _lib = None
 KNOB_UNROLL = 0
 KNOB_NONTEMPORAL = 1
 KNOB_WORKGROUPS_PER_CU = 2
+KNOB_SWAP_WORKGROUPS = 3
 
 ENTRY_POINTS = (
     "hfk_version",

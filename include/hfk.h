@@ -130,6 +130,9 @@ HFK_API int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_pt
  *   block_pairs   device-visible int64 [n_pairs, 2] = (src_block, dst_block)
  *   src_blocks, dst_blocks  blocks per plane on each side; a pair with an index
  *                 outside its range is skipped. 0 disables that side's check.
+ *   workgroups    0 = library default, which is sized for the PCIe link (a small
+ *                 grid saturates it); pass a large bound (e.g. 64 per CU) when both
+ *                 sides are device memory.
  * Destination blocks must be distinct (as index_copy_ requires for a
  * deterministic result); source and destination ranges must not overlap.
  */
@@ -159,7 +162,9 @@ HFK_API int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_
 enum hfk_knob {
     HFK_KNOB_UNROLL = 0,        /* 16-byte accesses in flight per lane: 1, 2, 4, 8, 16  */
     HFK_KNOB_NONTEMPORAL = 1,   /* bit0: non-temporal loads, bit1: non-temporal stores */
-    HFK_KNOB_WORKGROUPS_PER_CU = 2 /* default grid bound = CUs * this, 1..64          */
+    HFK_KNOB_WORKGROUPS_PER_CU = 2, /* default grid bound of the gathers and the
+                                       transfer = CUs * this, 1..1024                  */
+    HFK_KNOB_SWAP_WORKGROUPS = 3    /* default grid bound of hfk_swap_blocks           */
 };
 HFK_API int hfk_set_tuning(int knob, int64_t value);
 HFK_API int64_t hfk_get_tuning(int knob);

@@ -11,6 +11,8 @@ import numpy as np
 import pytest
 import torch
 
+import heterofusedkernels_amd  # noqa: F401  (puts the drop-in packages on sys.path)
+import pcie_through  # noqa: F401  (registers torch.ops.pcie_through.*)
 from heterofusedkernels_amd import capi
 from heterofusedkernels_amd import workloads as W
 from oracle import oracle as O

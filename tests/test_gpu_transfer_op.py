@@ -6,6 +6,8 @@ import numpy as np
 import pytest
 import torch
 
+import heterofusedkernels_amd  # noqa: F401  (puts the drop-in packages on sys.path)
+import pcie_through  # noqa: F401  (registers torch.ops.pcie_through.*)
 from oracle import oracle as O
 
 from gpu_helpers import announce
