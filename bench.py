@@ -39,6 +39,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"],
                     help="c2 (default) = Llama-3-8B swap-out, the configuration the metric is quoted on")
+    ap.add_argument("--sections", default="swap_out,swap_in,gather",
+                    help="comma list of the GPU sections to run; swap_out is the timed step and always runs unless "
+                         "a profile of one other kernel alone is wanted")
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--skip-memcpy-loop", action="store_true")
     args = ap.parse_args()
@@ -62,6 +65,8 @@ def main():
     dev = torch.device("cuda:0")
     cfg = {"c2": W.C2_LLAMA8B_SWAP_OUT, "c3": W.C3_LLAMA70B_SWAP_IN, "c4": W.C4_MLA_ROUNDTRIP,
            "c5": W.C5_FP8_FRAGMENTED}[args.workload]
+    sections = set(x for x in args.sections.split(",") if x)
+    assert sections <= {"swap_out", "swap_in", "gather"}, sections
     planes, bb, n = cfg.planes, cfg.block_bytes, cfg.n_blocks
     payload = cfg.payload_bytes
     stream = torch.cuda.current_stream().cuda_stream
@@ -101,51 +106,57 @@ def main():
                                       cfg.dev_blocks, 0, stream), "hfk_gather_blocks")
 
     def timed(fn, iters, warm):
-        """(wall seconds for `iters` calls between two synchronizes, per-launch event ms list)."""
+        """Runs `warm` untimed calls, then `iters` calls back to back between two synchronizes.
+        Returns (wall seconds for the iters calls, average milliseconds per call from one HIP event
+        pair recorded on the launch stream around the whole batch, so that launch gaps of short
+        kernels are hidden by the queue exactly as in steady-state use)."""
         for _ in range(warm):
             fn()
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for s, e in evs:
-            s.record()
+        start.record()
+        for _ in range(iters):
             fn()
-            e.record()
+        end.record()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
-        return wall, [s.elapsed_time(e) for s, e in evs]
+        return wall, start.elapsed_time(end) / iters
 
     # ---- PCIe peak as one large pinned copy sees it --------------------------
     big = min(1 << 30, host_pool.numel())
     big_d = torch.empty(big, dtype=torch.int8, device=dev)
     big_h = host_pool[:big]
     _, ms = timed(lambda: big_h.copy_(big_d, non_blocking=True), 5, 2)
-    d2h_peak = big / (sorted(ms)[len(ms) // 2] * 1e6)
+    d2h_peak = big / (ms * 1e6)
     _, ms = timed(lambda: big_d.copy_(big_h, non_blocking=True), 5, 2)
-    h2d_peak = big / (sorted(ms)[len(ms) // 2] * 1e6)
+    h2d_peak = big / (ms * 1e6)
     host_pool[:big].zero_()
     del big_d
     log("hipMemcpyAsync %d MiB pinned: D2H %.2f GB/s, H2D %.2f GB/s (link %.1f GB/s theoretical)" %
         (big >> 20, d2h_peak, h2d_peak, PCIE5_X16_GBPS))
 
     # ---- the timed steps: swap-out -------------------------------------------
-    wall, ms_out = timed(swap_out, args.steps, args.warmup)
-    value = args.steps * payload / wall / 1e9
-    ms_per_step = wall * 1e3 / args.steps
-    kernel_ms_out = sum(ms_out) / len(ms_out)
-    log("swap-out: %.2f GB/s whole-job (%.3f ms/step wall, %.3f ms/launch by events)" %
-        (value, ms_per_step, kernel_ms_out))
-
-    # verify: host slots == device source blocks read back by an independent path (torch index + D2H copy)
-    t0 = time.time()
-    for p in range(planes):
-        want = dev_bytes[p].index_select(0, ids_dev).cpu()
-        assert torch.equal(host_planes[p].index_select(0, dst_ids), want), "swap-out mismatch in plane %d" % p
-    untouched = torch.ones(cfg.host_blocks, dtype=torch.bool)
-    untouched[dst_ids] = False
-    for p in (0, planes // 2, planes - 1):
-        assert int(host_planes[p][untouched].max()) == 0, "swap-out wrote outside its slots (plane %d)" % p
-    log("swap-out verified bit-exact on all %d planes (%.1fs)" % (planes, time.time() - t0))
+    value = ms_per_step = kernel_ms_out = None
+    if "swap_out" in sections:
+        wall, kernel_ms_out = timed(swap_out, args.steps, args.warmup)
+        value = args.steps * payload / wall / 1e9
+        ms_per_step = wall * 1e3 / args.steps
+        log("swap-out: %.2f GB/s whole-job (%.3f ms/step wall, %.3f ms/launch by events)" %
+            (value, ms_per_step, kernel_ms_out))
+        # verify: host slots == device source blocks read back by an independent path (torch index + D2H copy)
+        t0 = time.time()
+        for p in range(planes):
+            want = dev_bytes[p].index_select(0, ids_dev).cpu()
+            assert torch.equal(host_planes[p].index_select(0, dst_ids), want), "swap-out mismatch in plane %d" % p
+        untouched = torch.ones(cfg.host_blocks, dtype=torch.bool)
+        untouched[dst_ids] = False
+        for p in (0, planes // 2, planes - 1):
+            assert int(host_planes[p][untouched].max()) == 0, "swap-out wrote outside its slots (plane %d)" % p
+        log("swap-out verified bit-exact on all %d planes (%.1fs)" % (planes, time.time() - t0))
+    else:   # later sections still need the host slots filled: do it with plain torch copies
+        for p in range(planes):
+            host_planes[p][dst_ids] = dev_bytes[p].index_select(0, ids_dev).cpu()
 
     # ---- swap-in (host slots -> other device slots) -----------------------------
     pairs_in = W.pairs_tensor(dst_ids, back_ids).to(dev)
@@ -154,28 +165,30 @@ def main():
         capi.check(capi.swap_blocks(dev_tab.data_ptr(), host_tab.data_ptr(), pairs_in.data_ptr(), planes, n, bb, bb, bb,
                                     cfg.host_blocks, cfg.dev_blocks, 0, stream), "hfk_swap_blocks(in)")
 
-    expect_in = {p: host_planes[p].index_select(0, dst_ids).clone() for p in range(planes)}
-    wall_in, ms_in = timed(swap_in, args.steps, args.warmup)
-    for p in range(planes):
-        got = dev_bytes[p].index_select(0, back_ids.to(dev)).cpu()
-        assert torch.equal(got, expect_in[p]), "swap-in mismatch in plane %d" % p
-    del expect_in
-    swap_in_gbps = args.steps * payload / wall_in / 1e9
-    kernel_ms_in = sum(ms_in) / len(ms_in)
-    log("swap-in: %.2f GB/s (%.3f ms/launch), verified" % (swap_in_gbps, kernel_ms_in))
+    swap_in_gbps = kernel_ms_in = None
+    if "swap_in" in sections:
+        expect_in = {p: host_planes[p].index_select(0, dst_ids).clone() for p in range(planes)}
+        wall_in, kernel_ms_in = timed(swap_in, args.steps, args.warmup)
+        for p in range(planes):
+            got = dev_bytes[p].index_select(0, back_ids.to(dev)).cpu()
+            assert torch.equal(got, expect_in[p]), "swap-in mismatch in plane %d" % p
+        del expect_in
+        swap_in_gbps = args.steps * payload / wall_in / 1e9
+        log("swap-in: %.2f GB/s (%.3f ms/launch), verified" % (swap_in_gbps, kernel_ms_in))
 
     # ---- block gather, HBM -> HBM ------------------------------------------------
-    wall_g, ms_g = timed(gather, args.steps, args.warmup)
-    for p in range(planes):
-        assert torch.equal(prefill[p], dev_bytes[p].index_select(0, ids_dev)), "gather mismatch %d" % p
     gather_alg_bytes = 2 * payload + 8 * n             # read + write + the id list
-    kernel_ms_g = sum(ms_g) / len(ms_g)
-    gather_traffic_gbps = gather_alg_bytes / (kernel_ms_g * 1e6)
-    gather_payload_gbps = payload / (kernel_ms_g * 1e6)
-    _, ms_t = timed(lambda: torch.index_select(dev_bytes[0], 0, ids_dev), args.steps, args.warmup)
-    torch_gather_gbps = 2 * n * bb / (sum(ms_t) / len(ms_t) * 1e6)
-    log("gather: %.1f GB/s of HBM traffic (%.1f payload GB/s, %.3f ms/launch), verified; torch.index_select on one "
-        "plane: %.1f GB/s" % (gather_traffic_gbps, gather_payload_gbps, kernel_ms_g, torch_gather_gbps))
+    kernel_ms_g = gather_traffic_gbps = gather_payload_gbps = torch_gather_gbps = None
+    if "gather" in sections:
+        wall_g, kernel_ms_g = timed(gather, args.steps, args.warmup)
+        for p in range(planes):
+            assert torch.equal(prefill[p], dev_bytes[p].index_select(0, ids_dev)), "gather mismatch %d" % p
+        gather_traffic_gbps = gather_alg_bytes / (kernel_ms_g * 1e6)
+        gather_payload_gbps = payload / (kernel_ms_g * 1e6)
+        _, ms_t = timed(lambda: torch.index_select(dev_bytes[0], 0, ids_dev), args.steps, args.warmup)
+        torch_gather_gbps = 2 * n * bb / (ms_t * 1e6)
+        log("gather: %.1f GB/s of HBM traffic (%.1f payload GB/s, %.3f ms/launch), verified; torch.index_select on one "
+            "plane: %.1f GB/s" % (gather_traffic_gbps, gather_payload_gbps, kernel_ms_g, torch_gather_gbps))
 
     # ---- plain device copy of known size: yardstick for reachable HBM bandwidth, and the
     # calibration row for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters -----------------
@@ -183,7 +196,7 @@ def main():
     cal_a = torch.empty(cal_bytes, dtype=torch.uint8, device=dev)
     cal_b = torch.full((cal_bytes,), 7, dtype=torch.uint8, device=dev)
     _, ms_c = timed(lambda: cal_a.copy_(cal_b), args.steps, args.warmup)
-    d2d_copy_gbps = 2 * cal_bytes / (sum(ms_c) / len(ms_c) * 1e6)
+    d2d_copy_gbps = 2 * cal_bytes / (ms_c * 1e6)
     del cal_a, cal_b
     log("torch device copy of %d MiB: %.1f GB/s of HBM traffic" % (cal_bytes >> 20, d2d_copy_gbps))
 
@@ -274,7 +287,14 @@ def main():
     except (OSError, ValueError):
         pass
 
-    out_kernel_gbps = payload / (kernel_ms_out * 1e6)
+    def rate(nbytes, ms):
+        return None if ms is None else nbytes / (ms * 1e6)
+
+    def frac(x, peak):
+        return None if x is None else x / peak
+
+    out_kernel_gbps = rate(payload, kernel_ms_out)
+    in_kernel_gbps = rate(payload, kernel_ms_in)
     result = {
         "metric": "KV swap GB/s (% of PCIe5 x16 peak); block gather GB/s (% of HBM peak)",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -283,31 +303,37 @@ def main():
         "config": {"workload": cfg.name, "planes": planes, "layers": cfg.layers, "block_bytes": bb,
                    "blocks_per_launch": n, "device_blocks": cfg.dev_blocks, "host_blocks": cfg.host_blocks,
                    "payload_bytes_per_step": payload, "cache_dtype": str(cfg.dtype).replace("torch.", "")},
+        # Dominant kernel of the step. A swap never touches HBM twice; the resource it saturates is the
+        # PCIe Gen5 x16 link, so that is the roofline it is priced against (theoretical link rate as
+        # `peak`, the rate one large pinned hipMemcpyAsync reaches in this run as `peak_measured`).
         "roofline": {
-            "kernel": "block_copy_kernel via hfk_swap_blocks (swap-out, HBM -> pinned host)", "bound": "pcie",
-            "achieved": out_kernel_gbps, "peak": PCIE5_X16_GBPS, "unit": "GB/s", "frac": out_kernel_gbps / PCIE5_X16_GBPS,
+            "kernel": "swap_blocks_kernel<8, 3> via hfk_swap_blocks (swap-out, HBM -> pinned host)", "bound": "pcie",
+            "achieved": out_kernel_gbps, "peak": PCIE5_X16_GBPS, "unit": "GB/s",
+            "frac": frac(out_kernel_gbps, PCIE5_X16_GBPS),
             "traffic": traffic.get("swap_out_hbm_bytes_per_launch"),
-            "peak_measured": d2h_peak, "frac_of_measured": out_kernel_gbps / d2h_peak,
+            "peak_measured": d2h_peak, "frac_of_measured": frac(out_kernel_gbps, d2h_peak),
             "algorithmic_bytes_per_launch": payload, "avg_launch_ms": kernel_ms_out,
         },
+        # The HBM-bound kernel of the path: the multi-plane block gather on the same cache.
         "roofline_gather": {
-            "kernel": "block_copy_kernel via hfk_gather_blocks (HBM -> HBM)", "bound": "hbm",
+            "kernel": "gather_blocks_kernel<8, 3> via hfk_gather_blocks (HBM -> HBM)", "bound": "hbm",
             "achieved": gather_traffic_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": gather_traffic_gbps / HBM_PEAK_GBPS, "traffic": traffic.get("gather_hbm_bytes_per_launch"),
+            "frac": frac(gather_traffic_gbps, HBM_PEAK_GBPS), "traffic": traffic.get("gather_hbm_bytes_per_launch"),
             "algorithmic_bytes_per_launch": gather_alg_bytes, "avg_launch_ms": kernel_ms_g,
             "payload_GBps": gather_payload_gbps, "torch_index_select_GBps": torch_gather_gbps,
             "torch_device_copy_GBps": d2d_copy_gbps,
         },
-        "swap_out": {"GBps": value, "kernel_GBps": out_kernel_gbps, "pct_of_measured_d2h": 100 * out_kernel_gbps / d2h_peak,
-                     "pct_of_pcie5_x16": 100 * out_kernel_gbps / PCIE5_X16_GBPS},
-        "swap_in": {"GBps": swap_in_gbps, "kernel_GBps": payload / (kernel_ms_in * 1e6),
-                    "pct_of_measured_h2d": 100 * payload / (kernel_ms_in * 1e6) / h2d_peak,
-                    "pct_of_pcie5_x16": 100 * payload / (kernel_ms_in * 1e6) / PCIE5_X16_GBPS},
+        "swap_out": {"GBps": value, "kernel_GBps": out_kernel_gbps,
+                     "pct_of_measured_d2h": None if out_kernel_gbps is None else 100 * out_kernel_gbps / d2h_peak,
+                     "pct_of_pcie5_x16": None if out_kernel_gbps is None else 100 * out_kernel_gbps / PCIE5_X16_GBPS},
+        "swap_in": {"GBps": swap_in_gbps, "kernel_GBps": in_kernel_gbps,
+                    "pct_of_measured_h2d": None if in_kernel_gbps is None else 100 * in_kernel_gbps / h2d_peak,
+                    "pct_of_pcie5_x16": None if in_kernel_gbps is None else 100 * in_kernel_gbps / PCIE5_X16_GBPS},
         "pcie_peak_measured": {"d2h_GBps": d2h_peak, "h2d_GBps": h2d_peak, "theoretical_GBps": PCIE5_X16_GBPS,
-                               "how": "median of 5 hipMemcpyAsync of %d MiB pinned" % (big >> 20)},
+                               "how": "mean of 5 back-to-back hipMemcpyAsync of %d MiB pinned" % (big >> 20)},
         "memcpy_block_loop": memcpy_loop,
         "cpu_baseline": cpu_baseline,
-        "verified": "bit-exact on every plane: swap-out, swap-in, gather",
+        "verified": "bit-exact on every plane: " + ", ".join(sorted(sections)),
     }
     print(json.dumps(result), flush=True)
 

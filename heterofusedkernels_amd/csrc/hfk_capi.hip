@@ -25,8 +25,22 @@ using hfk::TransposeArgs;
 using hfk::kWorkgroupLanes;
 using hfk::vec16;
 
+// One body, three kernel names: the block-copy body serves the swap, the multi-plane
+// block gather and wide-row gathers, and a profile should say which one ran.
+enum class Role { kSwapBlocks, kGatherBlocks, kGatherRows };
+
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void swap_blocks_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void gather_blocks_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
 template <typename IdT, int UNROLL, int NT>
-__global__ __launch_bounds__(256) void block_copy_kernel(const BlockCopyArgs<IdT> a) {
+__global__ __launch_bounds__(256) void gather_rows_wide_kernel(const BlockCopyArgs<IdT> a) {
     hfk::block_copy_body<IdT, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
@@ -95,17 +109,28 @@ int finish_launch() {
 }
 
 // ---- block copy -----------------------------------------------------------
-template <typename IdT, int UNROLL>
-void launch_block_copy_nt(const BlockCopyArgs<IdT>& a, uint32_t grid, int nt, hipStream_t s) {
-    switch (nt & 3) {
-        case 0: hipLaunchKernelGGL((block_copy_kernel<IdT, UNROLL, 0>), dim3(grid), dim3(256), 0, s, a); break;
-        case 1: hipLaunchKernelGGL((block_copy_kernel<IdT, UNROLL, 1>), dim3(grid), dim3(256), 0, s, a); break;
-        case 2: hipLaunchKernelGGL((block_copy_kernel<IdT, UNROLL, 2>), dim3(grid), dim3(256), 0, s, a); break;
-        default: hipLaunchKernelGGL((block_copy_kernel<IdT, UNROLL, 3>), dim3(grid), dim3(256), 0, s, a); break;
+template <Role ROLE, typename IdT, int UNROLL, int NT>
+void launch_block_copy_one(const BlockCopyArgs<IdT>& a, uint32_t grid, hipStream_t s) {
+    if constexpr (ROLE == Role::kSwapBlocks) {
+        hipLaunchKernelGGL((swap_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
+    } else if constexpr (ROLE == Role::kGatherBlocks) {
+        hipLaunchKernelGGL((gather_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
+    } else {
+        hipLaunchKernelGGL((gather_rows_wide_kernel<IdT, UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
     }
 }
 
-template <typename IdT>
+template <Role ROLE, typename IdT, int UNROLL>
+void launch_block_copy_nt(const BlockCopyArgs<IdT>& a, uint32_t grid, int nt, hipStream_t s) {
+    switch (nt & 3) {
+        case 0: launch_block_copy_one<ROLE, IdT, UNROLL, 0>(a, grid, s); break;
+        case 1: launch_block_copy_one<ROLE, IdT, UNROLL, 1>(a, grid, s); break;
+        case 2: launch_block_copy_one<ROLE, IdT, UNROLL, 2>(a, grid, s); break;
+        default: launch_block_copy_one<ROLE, IdT, UNROLL, 3>(a, grid, s); break;
+    }
+}
+
+template <Role ROLE, typename IdT>
 int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s) {
     int unroll = 1;
     int rc = hfk::plan_block_copy<IdT>(a, g_unroll.load(std::memory_order_relaxed), &unroll);
@@ -115,11 +140,11 @@ int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s) 
     if (rc != 0) return rc;
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
     switch (unroll) {
-        case 1: launch_block_copy_nt<IdT, 1>(a, grid, nt, s); break;
-        case 2: launch_block_copy_nt<IdT, 2>(a, grid, nt, s); break;
-        case 4: launch_block_copy_nt<IdT, 4>(a, grid, nt, s); break;
-        case 8: launch_block_copy_nt<IdT, 8>(a, grid, nt, s); break;
-        default: launch_block_copy_nt<IdT, 16>(a, grid, nt, s); break;
+        case 1: launch_block_copy_nt<ROLE, IdT, 1>(a, grid, nt, s); break;
+        case 2: launch_block_copy_nt<ROLE, IdT, 2>(a, grid, nt, s); break;
+        case 4: launch_block_copy_nt<ROLE, IdT, 4>(a, grid, nt, s); break;
+        case 8: launch_block_copy_nt<ROLE, IdT, 8>(a, grid, nt, s); break;
+        default: launch_block_copy_nt<ROLE, IdT, 16>(a, grid, nt, s); break;
     }
     return finish_launch();
 }
@@ -166,7 +191,7 @@ int gather_rows_typed(const void* table, void* dst, const IdT* ids, uint64_t n_i
         BlockCopyArgs<IdT> a;
         int rc = hfk::plan_wide_gather<IdT>(a, table, dst, ids, n_ids, row_bytes, limit);
         if (rc != 0) return rc;
-        return launch_block_copy<IdT>(a, workgroups, s);
+        return launch_block_copy<Role::kGatherRows, IdT>(a, workgroups, s);
     }
     return launch_flat_gather<IdT>((uint64_t)(uintptr_t)table, (uint64_t)(uintptr_t)dst, ids, n_ids, row_bytes,
                                    limit, workgroups, s);
@@ -265,7 +290,7 @@ int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, cons
     // A swap is bound by the PCIe link, which a fraction of the CUs saturates; a
     // small grid leaves the rest of the chip to whatever runs beside the swap.
     if (workgroups == 0) workgroups = (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
-    return launch_block_copy<int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
+    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
 }
 
 int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* ids,
@@ -276,7 +301,7 @@ int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, co
     int rc = hfk::plan_gather_blocks(a, dst_plane_ptrs, src_plane_ptrs, ids, n_planes, n_ids, block_bytes,
                                      src_block_stride, src_blocks);
     if (rc != 0) return rc;
-    return launch_block_copy<int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
+    return launch_block_copy<Role::kGatherBlocks, int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
 }
 
 int hfk_set_tuning(int knob, int64_t value) {

@@ -1,0 +1,163 @@
+"""The benchmark configurations at their full sizes, checked through size-independent
+properties: every destination block equals its source block as read back through an
+independent path (torch indexing on the device + a plain device-to-host copy), every
+byte outside the destination blocks keeps its sentinel, swap-out followed by swap-in
+is the identity, and the gather equals index_select. The CPU oracle covers the same
+code paths at small sizes in test_gpu_parity.py; here the multi-GiB caches are
+generated on the device so that nothing has to be mirrored on the host.
+"""
+import time
+
+import pytest
+import torch
+
+import heterofusedkernels_amd  # noqa: F401
+import pcie_through  # noqa: F401
+from heterofusedkernels import memory
+from heterofusedkernels_amd import workloads as W
+
+from gpu_helpers import announce, gather_blocks, host_ptr_table, ptr_table, swap
+
+pytestmark = [pytest.mark.gpu, pytest.mark.timeout(600)]
+DEV = "cuda"
+
+
+def _mem_available_gib():
+    with open("/proc/meminfo") as f:
+        for line in f:
+            if line.startswith("MemAvailable"):
+                return int(line.split()[1]) / 2**20
+    return 0.0
+
+
+def _need(host_gib, dev_gib):
+    if _mem_available_gib() < host_gib * 1.5 + 8:
+        pytest.skip("needs %.0f GiB of pinned host memory" % host_gib)
+    free, _ = torch.cuda.mem_get_info()
+    if free / 2**30 < dev_gib + 4:
+        pytest.skip("needs %.0f GiB of device memory" % dev_gib)
+
+
+def _device_cache(cfg, blocks):
+    t0 = time.time()
+    planes = [W.make_plane(cfg, l, kv, blocks, device=DEV) for l in range(cfg.layers) for kv in range(cfg.kv)]
+    torch.cuda.synchronize()
+    announce("  device cache %d planes x %d blocks: %.1f GiB in %.1fs" %
+             (len(planes), blocks, len(planes) * blocks * cfg.block_bytes / 2**30, time.time() - t0))
+    return planes, [W.as_bytes(p) for p in planes]
+
+
+def _host_cache(cfg, blocks, max_alloc_gib=8):
+    """Pinned host planes, allocated in groups of at most max_alloc_gib (one hipHostMalloc of
+    80 GiB is refused on the test machines; the registry handles any number of ranges)."""
+    t0 = time.time()
+    plane_bytes = blocks * cfg.block_bytes
+    per_alloc = max(1, int(max_alloc_gib * 2**30) // plane_bytes)
+    pools, planes = [], []
+    for first in range(0, cfg.planes, per_alloc):
+        count = min(per_alloc, cfg.planes - first)
+        try:
+            pool = memory.alloc_numa_pinned_tensor(count * plane_bytes)
+        except RuntimeError as exc:
+            del pools, planes
+            pytest.skip("could not pin %.0f GiB of host memory: %s" % (cfg.planes * plane_bytes / 2**30, exc))
+        pools.append(pool)
+        planes.extend(pool.view(torch.uint8).view(count, blocks, cfg.block_bytes).unbind(0))
+    announce("  pinned host cache %d planes x %d blocks: %.1f GiB in %d allocations, %.1fs" %
+             (cfg.planes, blocks, cfg.planes * plane_bytes / 2**30, len(pools), time.time() - t0))
+    return pools, planes
+
+
+def test_config2_llama8b_swap_out_full():
+    cfg = W.C2_LLAMA8B_SWAP_OUT
+    _need(16, 9)
+    announce("config 2 full: 32 layers x {K,V} [4096,16,8,128] bf16 -> pinned [8192,...], 256 pairs, one launch")
+    planes, dev_bytes = _device_cache(cfg, cfg.dev_blocks)
+    pool, host = _host_cache(cfg, cfg.host_blocks)                       # zero-filled by the allocator
+    src_ids, dst_ids = W.block_table(cfg, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    assert src_ids.unique().numel() == 256 and dst_ids.unique().numel() == 256
+    swap(host_ptr_table(host), ptr_table(planes), W.pairs_tensor(src_ids, dst_ids).to(DEV), cfg.planes,
+         cfg.block_bytes, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    torch.cuda.synchronize()
+    untouched = torch.ones(cfg.host_blocks, dtype=torch.bool)
+    untouched[dst_ids] = False
+    ids_dev = src_ids.to(DEV)
+    for p in range(cfg.planes):
+        want = dev_bytes[p].index_select(0, ids_dev).cpu()               # independent read-back path
+        assert torch.equal(host[p].index_select(0, dst_ids), want), "plane %d" % p
+        assert not host[p][untouched].any(), "plane %d: bytes outside the destination slots changed" % p
+    # nonzero payload really arrived (N(0,1) bf16 blocks are never all zero)
+    assert host[0].index_select(0, dst_ids).any(dim=1).all()
+
+
+def test_config3_llama70b_swap_in_full():
+    cfg = W.C3_LLAMA70B_SWAP_IN
+    _need(80, 41)
+    announce("config 3 full: 80 layers x {K,V}, pinned [16384,16,8,128] bf16 -> device [8192,...], 1024 blocks")
+    pool, host = _host_cache(cfg, cfg.host_blocks)
+    t0 = time.time()
+    for p in range(cfg.planes):                                          # U(-1,1) generated on the device, copied by hipMemcpy
+        layer, kv = divmod(p, cfg.kv)
+        host[p].copy_(W.as_bytes(W.make_plane(cfg, layer, kv, cfg.host_blocks, device=DEV)))
+    announce("  host cache filled in %.1fs" % (time.time() - t0))
+    dev = [torch.full((cfg.dev_blocks, cfg.block_bytes), 0x7E, dtype=torch.uint8, device=DEV) for _ in range(cfg.planes)]
+    gen = torch.Generator().manual_seed(cfg.base_seed)
+    perm = torch.randperm(cfg.host_blocks, generator=gen)
+    src_ids = perm[:cfg.n_blocks].contiguous()                           # block table = slice of a random permutation
+    dst_ids = torch.randperm(cfg.dev_blocks, generator=gen)[:cfg.n_blocks].contiguous()
+    swap(ptr_table(dev), host_ptr_table(host), W.pairs_tensor(src_ids, dst_ids).to(DEV), cfg.planes, cfg.block_bytes,
+         src_blocks=cfg.host_blocks, dst_blocks=cfg.dev_blocks)
+    torch.cuda.synchronize()
+    announce("  swap-in done, verifying")
+    untouched = torch.ones(cfg.dev_blocks, dtype=torch.bool, device=DEV)
+    untouched[dst_ids.to(DEV)] = False
+    dst_dev = dst_ids.to(DEV)
+    for p in range(cfg.planes):
+        got = dev[p].index_select(0, dst_dev).cpu()
+        assert torch.equal(got, host[p].index_select(0, src_ids)), "plane %d" % p
+        assert bool((dev[p][untouched] == 0x7E).all()), "plane %d: untouched device blocks changed" % p
+
+
+def test_config4_mla_round_trip_full():
+    cfg = W.C4_MLA_ROUNDTRIP
+    _need(9, 10)
+    announce("config 4 full: 61 layers [2048,64,576] bf16, swap-out 128 blocks then swap-in to other slots")
+    planes, dev_bytes = _device_cache(cfg, cfg.dev_blocks)
+    pool, host = _host_cache(cfg, cfg.host_blocks)
+    gen = torch.Generator().manual_seed(cfg.base_seed)
+    perm = torch.randperm(cfg.dev_blocks, generator=gen)
+    out_src, in_dst = perm[:128].contiguous(), perm[128:256].contiguous()        # disjoint device slots
+    host_slots = torch.randperm(cfg.host_blocks, generator=gen)[:128].contiguous()
+    original = [dev_bytes[p].index_select(0, out_src.to(DEV)).clone() for p in range(cfg.planes)]
+    dtab, htab = ptr_table(planes), host_ptr_table(host)
+    swap(htab, dtab, W.pairs_tensor(out_src, host_slots).to(DEV), cfg.planes, cfg.block_bytes,
+         src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    swap(dtab, htab, W.pairs_tensor(host_slots, in_dst).to(DEV), cfg.planes, cfg.block_bytes,
+         src_blocks=cfg.host_blocks, dst_blocks=cfg.dev_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        assert torch.equal(dev_bytes[p].index_select(0, in_dst.to(DEV)), original[p]), "plane %d round trip" % p
+        assert torch.equal(dev_bytes[p].index_select(0, out_src.to(DEV)), original[p]), "plane %d source changed" % p
+        assert torch.equal(host[p].index_select(0, host_slots), original[p].cpu()), "plane %d host copy" % p
+
+
+def test_config5_fp8_fragmented_full():
+    cfg = W.C5_FP8_FRAGMENTED
+    host_blocks = 4096
+    _need(4, 13)
+    announce("config 5 full: 32 layers x {K,V} [8192,16,8,128] fp8, 4096 fragmented ids: gather + swap-out")
+    planes, dev_bytes = _device_cache(cfg, cfg.dev_blocks)
+    ids = W.fragmented_ids(cfg.dev_blocks, cfg.n_blocks)
+    ids_dev = ids.to(DEV)
+    prefill = torch.zeros(cfg.planes, cfg.n_blocks, cfg.block_bytes, dtype=torch.uint8, device=DEV)
+    gather_blocks(ptr_table(list(prefill.unbind(0))), ptr_table(planes), ids_dev, cfg.planes, cfg.block_bytes,
+                  src_blocks=cfg.dev_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        assert torch.equal(prefill[p], dev_bytes[p].index_select(0, ids_dev)), "plane %d gather" % p
+    pool, host = _host_cache(cfg, host_blocks)
+    swap(host_ptr_table(host), ptr_table(planes), W.pairs_tensor(ids, torch.arange(cfg.n_blocks)).to(DEV), cfg.planes,
+         cfg.block_bytes, src_blocks=cfg.dev_blocks, dst_blocks=host_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        assert torch.equal(host[p], prefill[p].cpu()), "plane %d swap-out" % p
