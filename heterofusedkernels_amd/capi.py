@@ -22,6 +22,7 @@ ENTRY_POINTS = (
     "hfk_gather_rows",
     "hfk_multi_layer_block_transfer",
     "hfk_fused_memcpy_multi_layer_block_transfer",
+    "hfk_multi_layer_block_table_transfer",
     "hfk_swap_blocks",
     "hfk_gather_blocks",
     "hfk_set_tuning",
@@ -55,6 +56,9 @@ def load():
     L.hfk_multi_layer_block_transfer.restype = ci
     L.hfk_fused_memcpy_multi_layer_block_transfer.argtypes = [vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
     L.hfk_fused_memcpy_multi_layer_block_transfer.restype = ci
+    L.hfk_multi_layer_block_table_transfer.argtypes = [vp, u64, vp, u64, vp, u64, u64, u64, u32, u32, u32, u32, u32, ci,
+                                                       u32, vp]
+    L.hfk_multi_layer_block_table_transfer.restype = ci
     L.hfk_swap_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, u32, vp]
     L.hfk_swap_blocks.restype = ci
     L.hfk_gather_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u32, vp]
@@ -89,6 +93,15 @@ def fused_memcpy_multi_layer_block_transfer(layer_ptrs, host_block, staging, T, 
                                             workgroups=0, stream=0):
     return load().hfk_fused_memcpy_multi_layer_block_transfer(layer_ptrs, host_block, staging, T, L, H, D,
                                                               elem_bytes, workgroups, stream)
+
+
+def multi_layer_block_table_transfer(layer_ptrs, dev_block_stride, packed_blocks, packed_block_stride, pairs, n_pairs,
+                                     n_packed_blocks, n_dev_blocks, T, L, H, D, elem_bytes, to_packed, workgroups=0,
+                                     stream=0):
+    return load().hfk_multi_layer_block_table_transfer(layer_ptrs, dev_block_stride, packed_blocks,
+                                                       packed_block_stride, pairs, n_pairs, n_packed_blocks,
+                                                       n_dev_blocks, T, L, H, D, elem_bytes, int(bool(to_packed)),
+                                                       workgroups, stream)
 
 
 def swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, src_stride, dst_stride,

@@ -227,56 +227,106 @@ HFK_HD void flat_gather_body(const FlatGatherArgs<IdT>& a, uint32_t bid, uint32_
 }
 
 // ---------------------------------------------------------------------------
-// Layout-converting transfer of one block: source [T, L, H, row] read in memory
-// order (fully coalesced, which is what the PCIe link wants when the source is
-// host memory), every unit stored to layer l at [(h*T + t), row]. A source row
-// (D * elem_bytes bytes) stays contiguous, so stores land in row-sized runs.
+// Layout-converting transfer. The "packed" side holds whole blocks [T, L, H, row]
+// (pinned host memory in normal use), the "layered" side holds, per layer l, a
+// cache of blocks [H, T, row] reached through layer_ptrs[l]:
+//   layered[l][db][(h*T + t), row]  <->  packed[pb][((t*L + l)*H + h), row]
+// Lanes walk the packed side in memory order, so the side that crosses the PCIe
+// link is always fully coalesced; a row (D * elem_bytes bytes) stays contiguous
+// on the layered side, so HBM sees row-sized runs. TO_PACKED picks the direction.
+// One block with no table is the reference's multi_layer_block_transfer.
 // ---------------------------------------------------------------------------
 struct TransposeArgs {
-    const uint64_t* layer_ptrs;  // device array of L destination addresses
-    uint64_t src;                // address of the [T, L, H, row] block
+    const uint64_t* layer_ptrs;  // device array of L addresses (block 0 of each layer's cache)
+    uint64_t packed;             // address of packed block 0
+    const int64_t* pairs;        // [n_pairs, 2] = (packed_block, layered_block); null -> (0, 0)
+    uint64_t packed_stride;      // bytes between packed blocks
+    uint64_t layered_stride;     // bytes between blocks inside one layer's cache
+    uint64_t packed_limit;       // block indices must be < limit (unsigned compare)
+    uint64_t layered_limit;
+    uint32_t n_pairs;
+    uint32_t chunks_per_block;   // ceil(total_units / (256 * UNROLL))
     uint32_t T;
     uint32_t L;
     uint32_t H;
     uint32_t row_units;          // D * elem_bytes / sizeof(V)
-    uint32_t total_units;        // T * L * H * row_units
-    uint32_t n_work;             // ceil(total_units / (256 * UNROLL))
+    uint32_t total_units;        // T * L * H * row_units, per block
+    uint32_t n_work;             // n_pairs * chunks_per_block
 };
 
-template <typename V, int UNROLL, int NT>
+HFK_HD void unit_from_bytes(const HFK_GLOBAL uint8_t* p, uint8_t& v) { v = p[0]; }
+HFK_HD void unit_from_bytes(const HFK_GLOBAL uint8_t* p, uint32_t& v) {
+    v = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+HFK_HD void unit_from_bytes(const HFK_GLOBAL uint8_t* p, vec16& v) {
+    uint32_t w[4];
+    for (int i = 0; i < 4; ++i) unit_from_bytes(p + 4 * i, w[i]);
+    v.x = w[0];
+    v.y = w[1];
+    v.z = w[2];
+    v.w = w[3];
+}
+
+template <typename V, int UNROLL, int NT, bool TO_PACKED>
 HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid) {
     constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
-    const HFK_GLOBAL V* src = global_in<V>(a.src);
     const uint32_t LH = a.L * a.H;
 
     for (uint32_t w = bid; w < a.n_work; w += nb) {
-        const uint64_t g0 = (uint64_t)w * kChunkUnits + tid;
-        V v[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const uint64_t g = g0 + (uint64_t)u * kWorkgroupLanes;
-            if (g < a.total_units) {
-                v[u] = load_unit<NT>(src + g);
-            }
+        const uint32_t chunk = w % a.chunks_per_block;
+        const uint32_t pair = w / a.chunks_per_block;
+        const uint64_t pb = a.pairs ? (uint64_t)a.pairs[2 * (uint64_t)pair] : 0;
+        const uint64_t db = a.pairs ? (uint64_t)a.pairs[2 * (uint64_t)pair + 1] : 0;
+        if (pb >= a.packed_limit || db >= a.layered_limit) {
+            continue;
         }
+        const uint64_t packed_addr = a.packed + pb * a.packed_stride;
+        const uint64_t layered_off = db * a.layered_stride;
+        const uint64_t g0 = (uint64_t)chunk * kChunkUnits + tid;
+
+        V v[UNROLL];
+        uint64_t layered_addr[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const uint64_t g64 = g0 + (uint64_t)u * kWorkgroupLanes;
+            layered_addr[u] = 0;
             if (g64 < a.total_units) {
                 const uint32_t g = (uint32_t)g64;
-                const uint32_t r = g / a.row_units;      // source row = (t*L + l)*H + h
+                const uint32_t r = g / a.row_units;      // packed row = (t*L + l)*H + h
                 const uint32_t col = g - r * a.row_units;
                 const uint32_t t = r / LH;
                 const uint32_t lh = r - t * LH;
                 const uint32_t l = lh / a.H;
                 const uint32_t h = lh - l * a.H;
                 const uint64_t unit = ((uint64_t)h * a.T + t) * a.row_units + col;
-                const uint64_t d_addr = a.layer_ptrs[l] + unit * sizeof(V);
-                if ((d_addr & (sizeof(V) - 1)) == 0) {
-                    store_unit<NT>(global_out<V>(d_addr), v[u]);
+                layered_addr[u] = a.layer_ptrs[l] + layered_off + unit * sizeof(V);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint64_t g64 = g0 + (uint64_t)u * kWorkgroupLanes;
+            if (g64 < a.total_units) {
+                if constexpr (TO_PACKED) {
+                    if ((layered_addr[u] & (sizeof(V) - 1)) == 0) {
+                        v[u] = load_unit<NT>(global_in<V>(layered_addr[u]));
+                    } else {  // layer cache not aligned to the unit: byte loads keep it correct
+                        unit_from_bytes(global_in<uint8_t>(layered_addr[u]), v[u]);
+                    }
                 } else {
-                    // Layer buffer not aligned to the unit: byte stores keep it correct.
-                    HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(d_addr);
+                    v[u] = load_unit<NT>(global_in<V>(packed_addr) + g64);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint64_t g64 = g0 + (uint64_t)u * kWorkgroupLanes;
+            if (g64 < a.total_units) {
+                if constexpr (TO_PACKED) {
+                    store_unit<NT>(global_out<V>(packed_addr) + g64, v[u]);
+                } else if ((layered_addr[u] & (sizeof(V) - 1)) == 0) {
+                    store_unit<NT>(global_out<V>(layered_addr[u]), v[u]);
+                } else {  // byte stores for a misaligned layer cache
+                    HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(layered_addr[u]);
                     for (uint32_t k = 0; k < sizeof(V); ++k) {
                         d1[k] = unit_byte(v[u], k);
                     }

@@ -49,9 +49,16 @@ __global__ __launch_bounds__(256) void flat_gather_kernel(const FlatGatherArgs<I
     hfk::flat_gather_body<V, IdT, IndexT, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
+// Packed [T,L,H,D] blocks -> per-layer [H,T,D] caches (the reference's direction) ...
 template <typename V, int UNROLL, int NT>
 __global__ __launch_bounds__(256) void transpose_kernel(const TransposeArgs a) {
-    hfk::transpose_body<V, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    hfk::transpose_body<V, UNROLL, NT, false>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+// ... and back: per-layer caches -> packed blocks.
+template <typename V, int UNROLL, int NT>
+__global__ __launch_bounds__(256) void transpose_to_packed_kernel(const TransposeArgs a) {
+    hfk::transpose_body<V, UNROLL, NT, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
 // ---- tuning state ---------------------------------------------------------
@@ -199,28 +206,34 @@ int gather_rows_typed(const void* table, void* dst, const IdT* ids, uint64_t n_i
 
 // ---- transpose ------------------------------------------------------------
 template <typename V>
-void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, hipStream_t s) {
-    if (nt & 3) {
-        hipLaunchKernelGGL((transpose_kernel<V, hfk::kTransposeUnroll, 3>), dim3(grid), dim3(256), 0, s, a);
+void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, bool to_packed, hipStream_t s) {
+    constexpr int U = hfk::kTransposeUnroll;
+    if (to_packed) {
+        if (nt & 3) hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, 3>), dim3(grid), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, 0>), dim3(grid), dim3(256), 0, s, a);
     } else {
-        hipLaunchKernelGGL((transpose_kernel<V, hfk::kTransposeUnroll, 0>), dim3(grid), dim3(256), 0, s, a);
+        if (nt & 3) hipLaunchKernelGGL((transpose_kernel<V, U, 3>), dim3(grid), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((transpose_kernel<V, U, 0>), dim3(grid), dim3(256), 0, s, a);
     }
 }
 
-int launch_transpose(const void* dev_layer_ptrs, const void* src, uint32_t T, uint32_t L, uint32_t H,
-                     uint32_t D, uint32_t elem_bytes, uint32_t workgroups, hipStream_t s) {
+int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64_t* pairs, uint64_t n_pairs,
+                     uint64_t packed_stride, uint64_t layered_stride, uint64_t packed_blocks,
+                     uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
+                     bool to_packed, uint32_t workgroups, hipStream_t s) {
     TransposeArgs a;
     uint32_t unit = 16;
-    int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, src, T, L, H, D, elem_bytes);
+    int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, packed, pairs, n_pairs, packed_stride, layered_stride,
+                                 packed_blocks, layered_blocks, T, L, H, D, elem_bytes);
     if (rc != 0) return rc;
-    if (a.n_work == 0) return HFK_OK;  // empty block: nothing to move
+    if (a.n_work == 0) return HFK_OK;  // nothing to move
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
-    if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, s);
-    else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, s);
-    else launch_transpose_v<uint8_t>(a, grid, nt, s);
+    if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, to_packed, s);
+    else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, to_packed, s);
+    else launch_transpose_v<uint8_t>(a, grid, nt, to_packed, s);
     return finish_launch();
 }
 
@@ -260,7 +273,7 @@ int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i
 int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* src_block, uint32_t T,
                                    uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
                                    uint32_t workgroups, hfk_stream_t stream) {
-    return launch_transpose(dev_layer_ptrs, src_block, T, L, H, D, elem_bytes, workgroups,
+    return launch_transpose(dev_layer_ptrs, src_block, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, workgroups,
                             static_cast<hipStream_t>(stream));
 }
 
@@ -275,7 +288,20 @@ int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs, cons
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipMemcpyAsync(staging, host_block, bytes, hipMemcpyHostToDevice, s);
     if (e != hipSuccess) return (int)e;
-    return launch_transpose(dev_layer_ptrs, staging, T, L, H, D, elem_bytes, workgroups, s);
+    return launch_transpose(dev_layer_ptrs, staging, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, workgroups, s);
+}
+
+int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t dev_block_stride,
+                                         void* packed_blocks, uint64_t packed_block_stride,
+                                         const int64_t* block_pairs, uint64_t n_pairs, uint64_t n_packed_blocks,
+                                         uint64_t n_dev_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D,
+                                         uint32_t elem_bytes, int to_packed, uint32_t workgroups,
+                                         hfk_stream_t stream) {
+    if (n_pairs == 0) return HFK_OK;
+    if (block_pairs == nullptr) return HFK_ERR_NULL_POINTER;
+    return launch_transpose(dev_layer_ptrs, packed_blocks, block_pairs, n_pairs, packed_block_stride,
+                            dev_block_stride, n_packed_blocks, n_dev_blocks, T, L, H, D, elem_bytes, to_packed != 0,
+                            workgroups, static_cast<hipStream_t>(stream));
 }
 
 int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* block_pairs,

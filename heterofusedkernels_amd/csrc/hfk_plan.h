@@ -69,31 +69,49 @@ inline int plan_flat_gather(FlatGatherArgs<IdT>& a, FlatGatherPlan& p, uint64_t 
     return HFK_OK;
 }
 
-// Returns HFK_OK with n_work == 0 for an empty block.
-inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_layer_ptrs, const void* src,
-                          uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes) {
-    a.n_work = 0;
-    if (dev_layer_ptrs == nullptr || src == nullptr) return HFK_ERR_NULL_POINTER;
+// Geometry of the layout-converting transfer over a block table (pairs == nullptr:
+// the single block at the two base addresses). Returns HFK_OK with n_work == 0
+// when there is nothing to move.
+inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_layer_ptrs, const void* packed,
+                          const int64_t* pairs, uint64_t n_pairs, uint64_t packed_stride, uint64_t layered_stride,
+                          uint64_t packed_blocks, uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H,
+                          uint32_t D, uint32_t elem_bytes) {
+    a = TransposeArgs{};
+    if (dev_layer_ptrs == nullptr || packed == nullptr) return HFK_ERR_NULL_POINTER;
     if (elem_bytes == 0) return HFK_ERR_BAD_SIZE;
-    if (T == 0 || L == 0 || H == 0 || D == 0) return HFK_OK;
+    if (T == 0 || L == 0 || H == 0 || D == 0 || n_pairs == 0) return HFK_OK;
     const uint64_t row_bytes = (uint64_t)D * elem_bytes;
     const uint64_t rows = (uint64_t)T * L * H;
-    const uint32_t unit = pick_unit((uint64_t)(uintptr_t)src | row_bytes);
+    // The kernel indexes the units of one block with 32 bits.
+    if ((uint64_t)L * H > kU32Max || rows > kU32Max || rows * row_bytes > kU32Max) return HFK_ERR_TOO_LARGE;
+    const uint64_t block_bytes = rows * row_bytes;
+    const uint64_t layer_block_bytes = (uint64_t)H * T * row_bytes;
+    if (pairs != nullptr && (packed_stride < block_bytes || layered_stride < layer_block_bytes)) {
+        return HFK_ERR_BAD_SIZE;
+    }
+    uint64_t align = (uint64_t)(uintptr_t)packed | row_bytes;
+    if (pairs != nullptr) align |= packed_stride | layered_stride;
+    const uint32_t unit = pick_unit(align);
     const uint64_t row_units = row_bytes / unit;
     const uint64_t total = rows * row_units;
     const uint64_t chunk_units = (uint64_t)kWorkgroupLanes * kTransposeUnroll;
-    // The kernel indexes units with 32 bits.
-    if ((uint64_t)L * H > kU32Max || row_units > kU32Max || rows > kU32Max || total + chunk_units > kU32Max) {
-        return HFK_ERR_TOO_LARGE;
-    }
+    const uint64_t chunks = (total + chunk_units - 1) / chunk_units;
+    if (n_pairs > kU32Max || chunks * n_pairs > kU32Max) return HFK_ERR_TOO_LARGE;
     a.layer_ptrs = static_cast<const uint64_t*>(dev_layer_ptrs);
-    a.src = (uint64_t)(uintptr_t)src;
+    a.packed = (uint64_t)(uintptr_t)packed;
+    a.pairs = pairs;
+    a.packed_stride = packed_stride;
+    a.layered_stride = layered_stride;
+    a.packed_limit = packed_blocks ? packed_blocks : kUnchecked;
+    a.layered_limit = layered_blocks ? layered_blocks : kUnchecked;
+    a.n_pairs = (uint32_t)n_pairs;
+    a.chunks_per_block = (uint32_t)chunks;
     a.T = T;
     a.L = L;
     a.H = H;
     a.row_units = (uint32_t)row_units;
     a.total_units = (uint32_t)total;
-    a.n_work = (uint32_t)((total + chunk_units - 1) / chunk_units);
+    a.n_work = (uint32_t)(chunks * n_pairs);
     *unit_out = unit;
     return HFK_OK;
 }

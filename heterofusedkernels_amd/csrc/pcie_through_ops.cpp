@@ -3,7 +3,7 @@
 // Schemas of the first three ops are those of the reference
 // (pcieThrough/csrc/host/gather_torch.cpp:60,
 //  pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:113-114);
-// swap_blocks and gather_blocks are additive. Every op unpacks its tensors into
+// multi_layer_block_table_transfer, swap_blocks and gather_blocks are additive. Every op unpacks its tensors into
 // raw device-visible addresses, takes the current HIP stream of the device that
 // owns the device-side tensor, and calls the C-ABI of libhfk_hip.so; nothing is
 // allocated and nothing waits.
@@ -165,6 +165,41 @@ void fused_memcpy_multi_layer_block_transfer(const at::Tensor& deviceBlockCacheP
                  "hfk_fused_memcpy_multi_layer_block_transfer");
 }
 
+// The transfer op over a block table, either direction, one launch; see
+// hfk_multi_layer_block_table_transfer. hostBlockPool is [blocks, T, L, H, D];
+// deviceLayerCachePtrs[l] points at block 0 of layer l's cache [deviceBlocks][H, T, D].
+void multi_layer_block_table_transfer(const at::Tensor& deviceLayerCachePtrs, const at::Tensor& hostBlockPool,
+                                      const at::Tensor& blockPairs, int64_t deviceBlockStride, int64_t deviceBlocks,
+                                      bool toHost, std::optional<int64_t> workgroups) {
+    TORCH_CHECK(hostBlockPool.dim() == 5,
+                "hostBlockPool must be [blocks, blockSize, layers, heads, headDims], got ", hostBlockPool.dim(),
+                " dims");
+    TORCH_CHECK(hostBlockPool.is_contiguous(), "hostBlockPool must be contiguous");
+    for (int i = 1; i < 5; ++i) {
+        TORCH_CHECK(hostBlockPool.size(i) <= 0xffffffffLL, "hostBlockPool dimension ", i, " too large");
+    }
+    const uint32_t T = static_cast<uint32_t>(hostBlockPool.size(1)), L = static_cast<uint32_t>(hostBlockPool.size(2));
+    const uint32_t H = static_cast<uint32_t>(hostBlockPool.size(3)), D = static_cast<uint32_t>(hostBlockPool.size(4));
+    const uint32_t elem = static_cast<uint32_t>(hostBlockPool.element_size());
+    check_layer_ptrs(deviceLayerCachePtrs, L);
+    check_ptr_table(blockPairs, "blockPairs");
+    TORCH_CHECK(blockPairs.dim() == 2 && blockPairs.size(1) == 2, "blockPairs must be [n, 2]");
+    const uint64_t blockBytes = static_cast<uint64_t>(T) * L * H * D * elem;
+    TORCH_CHECK(deviceBlockStride >= 0 && static_cast<uint64_t>(deviceBlockStride) >= blockBytes / (L ? L : 1),
+                "deviceBlockStride is smaller than one [heads, blockSize, headDims] block");
+    TORCH_CHECK(deviceBlocks >= 0, "deviceBlocks must be non-negative");
+    if (blockPairs.size(0) == 0 || blockBytes == 0) return;
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(deviceLayerCachePtrs));
+    check_status(hfk_multi_layer_block_table_transfer(
+                     deviceLayerCachePtrs.data_ptr(), static_cast<uint64_t>(deviceBlockStride),
+                     device_visible(hostBlockPool, "hostBlockPool"), blockBytes,
+                     static_cast<const int64_t*>(device_visible(blockPairs, "blockPairs")),
+                     static_cast<uint64_t>(blockPairs.size(0)), static_cast<uint64_t>(hostBlockPool.size(0)),
+                     static_cast<uint64_t>(deviceBlocks), T, L, H, D, elem, toHost ? 1 : 0,
+                     workgroup_cap(workgroups), current_stream()),
+                 "hfk_multi_layer_block_table_transfer");
+}
+
 // Block-table swap, every plane in one launch; see hfk_swap_blocks. The plane
 // tables hold raw addresses (device pointers, or heterofusedkernels.memory
 // .get_device_ptr() of pinned host planes), built once by the caller exactly like
@@ -227,6 +262,9 @@ TORCH_LIBRARY(pcie_through, m) {
         "fused_memcpy_multi_layer_block_transfer(Tensor deviceBlockCachePtrs, Tensor hostBlockCache, Tensor "
         "stagingBlockCache, int? aiv=None) -> ()");
     m.def(
+        "multi_layer_block_table_transfer(Tensor deviceLayerCachePtrs, Tensor hostBlockPool, Tensor blockPairs, int "
+        "deviceBlockStride, int deviceBlocks=0, bool toHost=False, int? workgroups=None) -> ()");
+    m.def(
         "swap_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockPairs, int blockBytes, int "
         "srcBlockStride, int dstBlockStride, int srcBlocks=0, int dstBlocks=0, int? workgroups=None) -> ()");
     m.def(
@@ -241,6 +279,7 @@ TORCH_LIBRARY_IMPL(pcie_through, CUDA, m) {
     m.impl("gather", TORCH_FN(pciethrough::gather));
     m.impl("multi_layer_block_transfer", TORCH_FN(pciethrough::multi_layer_block_transfer));
     m.impl("fused_memcpy_multi_layer_block_transfer", TORCH_FN(pciethrough::fused_memcpy_multi_layer_block_transfer));
+    m.impl("multi_layer_block_table_transfer", TORCH_FN(pciethrough::multi_layer_block_table_transfer));
     m.impl("swap_blocks", TORCH_FN(pciethrough::swap_blocks));
     m.impl("gather_blocks", TORCH_FN(pciethrough::gather_blocks));
 }

@@ -1,0 +1,144 @@
+"""Re-runs the reference's own two benchmark tables (pcieThrough/tests/README.md) on MI355X.
+
+* Embedding-row gather from a host-registered table, fp16 rows of 512 elements (1 KiB),
+  batch sizes 16 ... 1024, one call per batch and "combined" (10 batches per call), timed
+  end to end on the host like pcieThrough/tests/test_gather.py:50-61 and
+  test_gather_combine.py:50-61; next to it the torch CPU index + H2D copy baseline of
+  pcieThrough/tests/test_memcpy.py:18-27.
+* One KV block [blockSize, layers, heads, headdim] int8, host -> per-layer device buffers
+  with layout conversion, direct and staged, per-op event time like
+  pcieThrough/tests/test_transfer_kernel.py:51-52,86-88.
+
+Results are verified (seeded random data, byte compare) before they are printed.
+Usage: python -m heterofusedkernels_amd.reference_shapes_bench [--rows N] [--runs N]
+"""
+import argparse
+import json
+import sys
+import time
+
+import torch
+
+import heterofusedkernels_amd  # noqa: F401
+import pcie_through  # noqa: F401
+from heterofusedkernels import memory
+
+
+def gather_table(rows, runs, out):
+    dev = "cuda"
+    dim = 512
+    embed = memory.alloc_numa_pinned_tensor(rows * dim * 2).view(torch.float16).view(rows, dim)
+    gen = torch.Generator().manual_seed(0)
+    chunk = 1 << 16
+    for r0 in range(0, rows, chunk):        # every row distinct and non-zero
+        r1 = min(rows, r0 + chunk)
+        embed[r0:r1] = torch.randn(r1 - r0, dim, generator=gen).to(torch.float16)
+    for bs in (16, 32, 64, 128, 256, 512, 1024):
+        row = {"bs": bs}
+        # torch CPU advanced index + H2D copy (tests/test_memcpy.py:18,23)
+        ids = torch.randint(0, rows, (runs, bs), dtype=torch.int64, generator=gen)
+        for i in range(3):
+            embed[ids[i % runs]].to(dev)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        cpu_runs = min(runs, 50)
+        for i in range(cpu_runs):
+            x = embed[ids[i]].to(dev)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / cpu_runs
+        row["torch_cpu_index_h2d_ms"] = dt * 1e3
+        row["torch_cpu_index_h2d_GBps"] = bs * dim * 2 / dt / 1e9
+        # one call per batch
+        ids_dev = ids.to(dev)
+        dst = torch.empty(bs, dim, dtype=torch.float16, device=dev)
+        for i in range(10):
+            torch.ops.pcie_through.gather(embed, dst, ids_dev[i % runs], aiv=4)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(runs):
+            torch.ops.pcie_through.gather(embed, dst, ids_dev[i], aiv=4)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / runs
+        assert torch.equal(dst.cpu().view(torch.int16), embed[ids[runs - 1]].view(torch.int16)), "gather mismatch"
+        row["gather_ms"] = dt * 1e3
+        row["gather_GBps"] = bs * dim * 2 / dt / 1e9
+        # combined: 10 batches in one call, default aiv (tests/test_gather_combine.py:47-56)
+        ids10 = torch.randint(0, rows, (runs, bs * 10), dtype=torch.int64, generator=gen)
+        ids10_dev = ids10.to(dev)
+        dst10 = torch.empty(bs * 10, dim, dtype=torch.float16, device=dev)
+        for i in range(10):
+            torch.ops.pcie_through.gather(embed, dst10, ids10_dev[i % runs])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(runs):
+            torch.ops.pcie_through.gather(embed, dst10, ids10_dev[i])
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / runs
+        assert torch.equal(dst10.cpu().view(torch.int16), embed[ids10[runs - 1]].view(torch.int16)), "gather mismatch"
+        row["gather_combined_ms_per_batch"] = dt * 1e3 / 10
+        row["gather_combined_GBps"] = bs * 10 * dim * 2 / dt / 1e9
+        out["gather"].append(row)
+        print("gather bs=%4d: cpu+h2d %.3f ms (%.2f GB/s) | gather %.4f ms (%.2f GB/s) | combined %.4f ms/batch "
+              "(%.2f GB/s)" % (bs, row["torch_cpu_index_h2d_ms"], row["torch_cpu_index_h2d_GBps"], row["gather_ms"],
+                               row["gather_GBps"], row["gather_combined_ms_per_batch"], row["gather_combined_GBps"]),
+              file=sys.stderr, flush=True)
+
+
+def transfer_table(out, blocks=8):
+    dev = "cuda"
+    for (T, L, H, D) in ((1024, 32, 1, 128), (1024, 32, 8, 128), (1024, 64, 1, 128), (1024, 64, 8, 128)):
+        nbytes = T * L * H * D
+        pool = memory.alloc_numa_pinned_tensor(blocks * nbytes)
+        pool.copy_(torch.randint(-128, 128, (blocks * nbytes,), dtype=torch.int8,
+                                 generator=torch.Generator().manual_seed(L * 10 + H)))
+        host_blocks = list(pool.view(blocks, T, L, H, D).unbind(0))
+        dev_blocks = torch.zeros(blocks, L, H, T, D, dtype=torch.int8, device=dev)
+        ptrs = [torch.tensor([dev_blocks[b, l].data_ptr() for l in range(L)], dtype=torch.int64).to(dev)
+                for b in range(blocks)]
+        staging = torch.empty(T, L, H, D, dtype=torch.int8, device=dev)
+        row = {"shape": [T, L, H, D], "block_bytes": nbytes}
+        for name, fused in (("direct", False), ("staged", True)):
+            def call(b):
+                if fused:
+                    torch.ops.pcie_through.fused_memcpy_multi_layer_block_transfer(ptrs[b], host_blocks[b], staging, 4)
+                else:
+                    torch.ops.pcie_through.multi_layer_block_transfer(ptrs[b], host_blocks[b], 4)
+            for b in range(blocks):
+                call(b)
+            torch.cuda.synchronize()
+            times = []
+            for rep in range(3):
+                for b in range(blocks):
+                    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    s.record()
+                    call(b)
+                    e.record()
+                    times.append((s, e))
+            torch.cuda.synchronize()
+            ms = sum(s.elapsed_time(e) for s, e in times) / len(times)
+            got = dev_blocks.cpu()
+            for b in range(blocks):
+                assert torch.equal(got[b].permute(2, 0, 1, 3), host_blocks[b]), "transfer mismatch"
+            row[name + "_ms"] = ms
+            row[name + "_GBps"] = nbytes / (ms * 1e6)
+        out["transfer"].append(row)
+        print("transfer [%d,%d,%d,%d] int8: direct %.3f ms (%.2f GB/s) | staged %.3f ms (%.2f GB/s)" %
+              (T, L, H, D, row["direct_ms"], row["direct_GBps"], row["staged_ms"], row["staged_GBps"]),
+              file=sys.stderr, flush=True)
+        del pool, host_blocks
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--rows", type=int, default=4000000, help="embedding rows (reference: 4 000 000)")
+    ap.add_argument("--runs", type=int, default=200)
+    args = ap.parse_args()
+    assert torch.cuda.is_available()
+    out = {"gather": [], "transfer": [], "rows": args.rows, "runs": args.runs}
+    gather_table(args.rows, args.runs, out)
+    transfer_table(out)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -112,6 +112,37 @@ HFK_API int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_pt
                                                 uint32_t workgroups, hfk_stream_t stream);
 
 /*
+ * The transfer above over a block table, in either direction, all blocks and all
+ * layers in one launch:
+ *   for j < n_pairs, with (pb, db) = block_pairs[j]:
+ *     to_packed == 0:  layer_l[db][(h*T + t)*D + d]  =  packed[pb][((t*L + l)*H + h)*D + d]
+ *     to_packed != 0:  packed[pb][((t*L + l)*H + h)*D + d]  =  layer_l[db][(h*T + t)*D + d]
+ * where packed[pb] starts at packed_blocks + pb * packed_block_stride and layer_l[db]
+ * at dev_layer_ptrs[l] + db * dev_block_stride.
+ *
+ * Replaces the reference's per-block caller loop around multi_layer_block_transfer
+ * (pcieThrough/tests/test_transfer_kernel.py:58-72) with one launch; the
+ * to_packed direction (device caches -> packed host blocks) has no counterpart in
+ * the reference, whose op is host -> device only
+ * (pcieThrough/csrc/kernel/multi_layer_block_transfer_kernel.h:42-72).
+ *
+ *   dev_layer_ptrs   device-visible array of L uint64 addresses: block 0 of each
+ *                    layer's cache [n_dev_blocks][H,T,D]
+ *   packed_blocks    device-visible pool of [T,L,H,D] blocks (pinned host memory)
+ *   block_pairs      device-visible int64 [n_pairs, 2] = (packed_block, dev_block)
+ *   n_packed_blocks, n_dev_blocks  pool sizes; a pair outside them is skipped,
+ *                    0 disables that side's check
+ * Strides must be at least one block of their side. Destination blocks must be distinct.
+ */
+HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t dev_block_stride,
+                                         void* packed_blocks, uint64_t packed_block_stride,
+                                         const int64_t* block_pairs, uint64_t n_pairs,
+                                         uint64_t n_packed_blocks, uint64_t n_dev_blocks,
+                                         uint32_t T, uint32_t L, uint32_t H, uint32_t D,
+                                         uint32_t elem_bytes, int to_packed, uint32_t workgroups,
+                                         hfk_stream_t stream);
+
+/*
  * Block-table swap, all planes (layer x K/V) in one launch:
  *   for p < n_planes, j < n_pairs:
  *     copy block_bytes bytes

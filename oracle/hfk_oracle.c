@@ -96,6 +96,48 @@ ORACLE_API int oracle_multi_layer_block_transfer(void* const* layer_ptrs, const 
 }
 
 /*
+ * The transfer above over a block table: for each pair (packed block pb, layered
+ * block db) either the reference's host -> device conversion (to_packed == 0), which
+ * restates the caller loop pcieThrough/tests/test_transfer_kernel.py:58-72 (one
+ * multi_layer_block_transfer per block, per-block pointer tables :42-47), or its
+ * inverse (to_packed != 0): packed[pb][((t*L + l)*H + h)*D + d] = layer_l[db][(h*T + t)*D + d].
+ * The inverse has no counterpart in the reference; it is pinned as the exact inverse
+ * of the forward direction and by brute force.
+ */
+ORACLE_API int oracle_multi_layer_block_table_transfer(void* const* layer_ptrs, uint64_t layered_stride,
+                                                       void* packed, uint64_t packed_stride,
+                                                       const int64_t* pairs, uint64_t n_pairs, uint32_t T,
+                                                       uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
+                                                       int to_packed, uint32_t cores) {
+    if (n_pairs == 0) return 0;
+    if (!layer_ptrs || !packed || !pairs || elem_bytes == 0 || cores == 0) return -1;
+    void** block_layers = (void**)malloc(sizeof(void*) * (L ? L : 1));
+    if (!block_layers) return -2;
+    const uint64_t row = (uint64_t)D * elem_bytes;
+    for (uint64_t j = 0; j < n_pairs; ++j) {
+        char* pblock = (char*)packed + (uint64_t)pairs[2 * j] * packed_stride;
+        for (uint32_t l = 0; l < L; ++l) {
+            block_layers[l] = (char*)layer_ptrs[l] + (uint64_t)pairs[2 * j + 1] * layered_stride;
+        }
+        if (!to_packed) {
+            int rc = oracle_multi_layer_block_transfer(block_layers, pblock, T, L, H, D, elem_bytes, cores);
+            if (rc != 0) {
+                free(block_layers);
+                return rc;
+            }
+        } else {
+            for (uint64_t t = 0; t < T; ++t)
+                for (uint32_t l = 0; l < L; ++l)
+                    for (uint32_t h = 0; h < H; ++h)
+                        memcpy(pblock + ((t * L + l) * H + h) * row,
+                               (const char*)block_layers[l] + ((uint64_t)h * T + t) * row, row);
+        }
+    }
+    free(block_layers);
+    return 0;
+}
+
+/*
  * Block-table swap over planes: per plane
  *   dst.index_copy_(0, pairs[:,1], src.index_select(0, pairs[:,0]))
  * i.e. first gather the source blocks into a temporary, then scatter them.

@@ -48,6 +48,8 @@ def lib():
         L.oracle_gather_rows.restype = ci
         L.oracle_multi_layer_block_transfer.argtypes = [vp, vp, u32, u32, u32, u32, u32, u32]
         L.oracle_multi_layer_block_transfer.restype = ci
+        L.oracle_multi_layer_block_table_transfer.argtypes = [vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, u32, ci, u32]
+        L.oracle_multi_layer_block_table_transfer.restype = ci
         L.oracle_swap_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64]
         L.oracle_swap_blocks.restype = ci
         _lib = L
@@ -86,6 +88,22 @@ def c_multi_layer_block_transfer(src_u8, T, L, H, D, elem_bytes, cores=2, fill=0
     rc = lib().oracle_multi_layer_block_transfer(ptrs, src_u8.ctypes.data, T, L, H, D, elem_bytes, cores)
     assert rc == 0, rc
     return out
+
+
+def c_multi_layer_block_table_transfer(layers_u8, packed_u8, pairs, T, L, H, D, elem_bytes, to_packed, cores=2):
+    """layers_u8: uint8 [L, dev_blocks, H*T*D*e] (per-layer caches); packed_u8: uint8
+    [packed_blocks, T*L*H*D*e]; pairs int64 [n,2] = (packed_block, layered_block).
+    Mutates layers_u8 (to_packed False) or packed_u8 (to_packed True) in place."""
+    assert layers_u8.dtype == np.uint8 and packed_u8.dtype == np.uint8
+    assert layers_u8.flags.c_contiguous and packed_u8.flags.c_contiguous
+    assert layers_u8.shape[0] == L and layers_u8.shape[2] == H * T * D * elem_bytes
+    assert packed_u8.shape[1] == T * L * H * D * elem_bytes
+    pairs = np.ascontiguousarray(pairs, dtype=np.int64).reshape(-1, 2)
+    ptrs = (ctypes.c_void_p * max(L, 1))(*[layers_u8[l].ctypes.data for l in range(L)])
+    rc = lib().oracle_multi_layer_block_table_transfer(
+        ptrs, layers_u8.shape[2], packed_u8.ctypes.data, packed_u8.shape[1], pairs.ctypes.data, pairs.shape[0],
+        T, L, H, D, elem_bytes, int(bool(to_packed)), cores)
+    assert rc == 0, rc
 
 
 def c_swap_blocks(dst_planes_u8, src_planes_u8, pairs):
@@ -153,6 +171,21 @@ def brute_multi_layer_block_transfer(src_u8, T, L, H, D, elem_bytes):
                         o = ((h * T + t) * D + d) * elem_bytes + b
                         out[l, o] = src[s]
     return out
+
+
+def brute_block_table_transfer(layers_u8, packed_u8, pairs, T, L, H, D, elem_bytes, to_packed):
+    """Element loops for the block-table transfer in either direction (in place)."""
+    for (pb, db) in np.asarray(pairs).reshape(-1, 2):
+        for t in range(T):
+            for l in range(L):
+                for h in range(H):
+                    for d in range(D * elem_bytes):
+                        po = ((t * L + l) * H + h) * D * elem_bytes + d
+                        lo = (h * T + t) * D * elem_bytes + d
+                        if to_packed:
+                            packed_u8[int(pb), po] = layers_u8[l, int(db), lo]
+                        else:
+                            layers_u8[l, int(db), lo] = packed_u8[int(pb), po]
 
 
 def brute_swap_blocks(dst_planes_u8, src_planes_u8, pairs):

@@ -24,6 +24,10 @@ int oracle_gather_rows(const void* table, void* dst, const void* ids, int ids_ar
                        uint64_t row_bytes, uint32_t cores);
 int oracle_multi_layer_block_transfer(void* const* layer_ptrs, const void* src, uint32_t T, uint32_t L,
                                       uint32_t H, uint32_t D, uint32_t elem_bytes, uint32_t cores);
+int oracle_multi_layer_block_table_transfer(void* const* layer_ptrs, uint64_t layered_stride, void* packed,
+                                            uint64_t packed_stride, const int64_t* pairs, uint64_t n_pairs,
+                                            uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
+                                            int to_packed, uint32_t cores);
 int oracle_swap_blocks(void* const* dst_planes, const void* const* src_planes, const int64_t* pairs,
                        uint32_t n_planes, uint64_t n_pairs, uint64_t block_bytes, uint64_t src_stride,
                        uint64_t dst_stride);
@@ -221,6 +225,16 @@ void case_gather_rows(uint64_t table_rows, uint64_t n_ids, uint64_t row_bytes, s
 }
 
 // ---- transpose -------------------------------------------------------------
+template <bool TO_PACKED>
+void walk_transpose(const TransposeArgs& a, uint32_t unit, uint32_t grid_cap) {
+    if (a.n_work == 0) return;
+    const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+    if (unit == 16u) walk(a, grid, transpose_body<vec16, kTransposeUnroll, 3, TO_PACKED>);
+    else if (unit == 4u) walk(a, grid, transpose_body<uint32_t, kTransposeUnroll, 0, TO_PACKED>);
+    else walk(a, grid, transpose_body<uint8_t, kTransposeUnroll, 0, TO_PACKED>);
+}
+
+// single block, the reference's op
 void case_transpose(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem, size_t s_mis, size_t l_mis,
                     uint32_t grid_cap) {
     const uint64_t block = (uint64_t)T * L * H * D * elem, layer = (uint64_t)H * T * D * elem;
@@ -239,14 +253,9 @@ void case_transpose(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t ele
     }
     TransposeArgs a;
     uint32_t unit = 0;
-    int rc = plan_transpose(a, &unit, lp.data(), src.p, T, L, H, D, elem);
+    int rc = plan_transpose(a, &unit, lp.data(), src.p, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem);
     if (rc != HFK_OK) { ++g_failures; std::printf("plan_transpose rc=%d\n", rc); }
-    else if (a.n_work > 0) {
-        const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
-        if (unit == 16u) walk(a, grid, transpose_body<vec16, kTransposeUnroll, 3>);
-        else if (unit == 4u) walk(a, grid, transpose_body<uint32_t, kTransposeUnroll, 0>);
-        else walk(a, grid, transpose_body<uint8_t, kTransposeUnroll, 0>);
-    }
+    else walk_transpose<false>(a, unit, grid_cap);
     oracle_multi_layer_block_transfer(ep.data(), src.p, T, L, H, D, elem, 3);
     char what[128];
     std::snprintf(what, sizeof what, "transpose T=%u L=%u H=%u D=%u elem=%u mis=%zu/%zu grid=%u unit=%u", T, L, H, D, elem,
@@ -254,6 +263,61 @@ void case_transpose(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t ele
     for (uint32_t l = 0; l < L; ++l) expect_equal(dst[l]->p, exp[l]->p, layer, what);
     for (auto* b : dst) delete b;
     for (auto* b : exp) delete b;
+}
+
+// block table, both directions, padded strides, out-of-range pairs
+void case_transpose_table(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem, uint32_t packed_blocks,
+                          uint32_t dev_blocks, uint32_t n_pairs, uint64_t p_pad, uint64_t l_pad, size_t p_mis,
+                          size_t l_mis, bool to_packed, bool with_bad, uint32_t grid_cap) {
+    const uint64_t block = (uint64_t)T * L * H * D * elem, layer_block = (uint64_t)H * T * D * elem;
+    const uint64_t ps = block + p_pad, ls = layer_block + l_pad;
+    Buf packed(packed_blocks * ps - p_pad, p_mis), packed_exp(packed_blocks * ps - p_pad, p_mis);
+    packed.randomize();
+    std::memcpy(packed_exp.p, packed.p, packed.n);
+    std::vector<Buf*> lay, lay_exp;
+    std::vector<uint64_t> lp;
+    std::vector<void*> ep;
+    for (uint32_t l = 0; l < L; ++l) {
+        lay.push_back(new Buf(dev_blocks * ls - l_pad, l_mis));
+        lay_exp.push_back(new Buf(dev_blocks * ls - l_pad, l_mis));
+        lay.back()->randomize();
+        std::memcpy(lay_exp.back()->p, lay.back()->p, lay.back()->n);
+        lp.push_back((uint64_t)(uintptr_t)lay.back()->p);
+        ep.push_back(lay_exp.back()->p);
+    }
+    // distinct destination blocks on whichever side is written
+    std::vector<int64_t> pperm(packed_blocks), dperm(dev_blocks), pairs, good;
+    for (uint32_t i = 0; i < packed_blocks; ++i) pperm[i] = i;
+    for (uint32_t i = 0; i < dev_blocks; ++i) dperm[i] = i;
+    std::shuffle(pperm.begin(), pperm.end(), rng);
+    std::shuffle(dperm.begin(), dperm.end(), rng);
+    for (uint32_t j = 0; j < n_pairs; ++j) {
+        int64_t pb = pperm[j % packed_blocks], db = dperm[j % dev_blocks];
+        bool bad = false;
+        if (with_bad && j % 4 == 1) { pb = (j % 8 == 1) ? -1 : (int64_t)packed_blocks + 2; bad = true; }
+        if (with_bad && j % 5 == 2) { db = (j % 2) ? (int64_t)dev_blocks : -7; bad = true; }
+        pairs.push_back(pb);
+        pairs.push_back(db);
+        if (!bad) { good.push_back(pb); good.push_back(db); }
+    }
+    TransposeArgs a;
+    uint32_t unit = 0;
+    int rc = plan_transpose(a, &unit, lp.data(), packed.p, pairs.data(), n_pairs, ps, ls, packed_blocks, dev_blocks, T,
+                            L, H, D, elem);
+    if (rc != HFK_OK) { ++g_failures; std::printf("plan_transpose(table) rc=%d\n", rc); }
+    else if (to_packed) walk_transpose<true>(a, unit, grid_cap);
+    else walk_transpose<false>(a, unit, grid_cap);
+    oracle_multi_layer_block_table_transfer(ep.data(), ls, packed_exp.p, ps, good.data(), good.size() / 2, T, L, H, D,
+                                            elem, to_packed, 2);
+    char what[192];
+    std::snprintf(what, sizeof what, "transpose_table T=%u L=%u H=%u D=%u e=%u pb=%u db=%u pairs=%u pad=%llu/%llu mis=%zu/%zu "
+                  "to_packed=%d bad=%d grid=%u unit=%u", T, L, H, D, elem, packed_blocks, dev_blocks, n_pairs,
+                  (unsigned long long)p_pad, (unsigned long long)l_pad, p_mis, l_mis, (int)to_packed, (int)with_bad,
+                  grid_cap, unit);
+    expect_equal(packed.p, packed_exp.p, packed.n, what);
+    for (uint32_t l = 0; l < L; ++l) expect_equal(lay[l]->p, lay_exp[l]->p, lay[l]->n, what);
+    for (auto* b : lay) delete b;
+    for (auto* b : lay_exp) delete b;
 }
 
 }  // namespace
@@ -322,6 +386,19 @@ int main() {
     case_transpose(9, 2, 3, 16, 2, 4, 0, 5);          // source 4-byte aligned
     case_transpose(6, 2, 2, 16, 1, 1, 3, 5);          // everything odd
     case_transpose(0, 2, 2, 16, 1, 0, 0, 5);          // empty block
+
+    // block-table transfer, both directions
+    for (bool to_packed : {false, true}) {
+        case_transpose_table(16, 4, 2, 128, 1, 6, 5, 4, 0, 0, 0, 0, to_packed, false, 7);      // int8 rows of 128 B
+        case_transpose_table(8, 3, 2, 64, 2, 5, 7, 5, 0, 0, 0, 0, to_packed, true, 1000);     // bf16 + bad pairs
+        case_transpose_table(33, 2, 3, 16, 2, 4, 4, 4, 32, 64, 0, 0, to_packed, false, 3);     // padded strides, odd T
+        case_transpose_table(5, 2, 2, 20, 2, 4, 4, 3, 0, 0, 0, 0, to_packed, true, 5);         // 40-byte rows: 4-byte units
+        case_transpose_table(5, 2, 2, 7, 1, 4, 4, 3, 0, 0, 0, 0, to_packed, false, 5);         // 7-byte rows: byte units
+        case_transpose_table(9, 2, 3, 16, 2, 3, 3, 3, 0, 0, 0, 4, to_packed, false, 5);        // layer caches 4-byte aligned
+        case_transpose_table(9, 2, 3, 16, 2, 3, 3, 3, 4, 0, 0, 0, to_packed, true, 5);         // packed stride 4-byte aligned
+        case_transpose_table(6, 2, 2, 16, 1, 3, 3, 2, 3, 5, 1, 3, to_packed, false, 5);        // everything odd
+        case_transpose_table(64, 2, 1, 128, 1, 3, 3, 3, 0, 0, 0, 0, to_packed, false, 2);      // one-head blocks
+    }
 
     std::printf("%d comparisons, %d failures\n", g_cases, g_failures);
     return g_failures == 0 ? 0 : 1;

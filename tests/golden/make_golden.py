@@ -39,6 +39,30 @@ def transfer_case(seed, T, L, H, D, elem):
     return dict(src=src, expected=out, geometry=np.array([T, L, H, D, elem], dtype=np.int64))
 
 
+def table_transfer_case(seed, T, L, H, D, elem, packed_blocks, dev_blocks, n_pairs, to_packed):
+    """Block-table form of the transfer, either direction, from single-element loops."""
+    rs = np.random.RandomState(seed)
+    packed = rs.randint(0, 256, size=(packed_blocks, T * L * H * D * elem)).astype(np.uint8)
+    layers = rs.randint(0, 256, size=(L, dev_blocks, H * T * D * elem)).astype(np.uint8)
+    pb = rs.permutation(packed_blocks)[:n_pairs]
+    db = rs.permutation(dev_blocks)[:n_pairs]
+    pairs = np.stack([pb, db], axis=1).astype(np.int64)
+    packed_out, layers_out = packed.copy(), layers.copy()
+    for j in range(n_pairs):
+        for t in range(T):
+            for l in range(L):
+                for h in range(H):
+                    for d in range(D * elem):
+                        po = ((t * L + l) * H + h) * D * elem + d
+                        lo = (h * T + t) * D * elem + d
+                        if to_packed:
+                            packed_out[int(pairs[j, 0]), po] = layers[l, int(pairs[j, 1]), lo]
+                        else:
+                            layers_out[l, int(pairs[j, 1]), lo] = packed[int(pairs[j, 0]), po]
+    return dict(packed=packed, layers=layers, pairs=pairs, packed_expected=packed_out, layers_expected=layers_out,
+                geometry=np.array([T, L, H, D, elem, int(to_packed)], dtype=np.int64))
+
+
 def gather_case(seed, rows, row_bytes, n_ids, id_dtype):
     rs = np.random.RandomState(seed)
     table = rs.randint(0, 256, size=(rows, row_bytes)).astype(np.uint8)
@@ -75,6 +99,11 @@ def main():
         "transfer_T8_L4_H1_D128_e1": transfer_case(5, 8, 4, 1, 128, 1),
         "transfer_T3_L1_H1_D32_e2": transfer_case(6, 3, 1, 1, 32, 2),
         "transfer_T4_L2_H2_D7_e1": transfer_case(7, 4, 2, 2, 7, 1),
+        "tabletransfer_in_T4_L3_H2_D16_e1": table_transfer_case(31, 4, 3, 2, 16, 1, 5, 4, 3, False),
+        "tabletransfer_out_T4_L3_H2_D16_e1": table_transfer_case(32, 4, 3, 2, 16, 1, 5, 4, 3, True),
+        "tabletransfer_in_T3_L2_H2_D32_e2": table_transfer_case(33, 3, 2, 2, 32, 2, 3, 6, 3, False),
+        "tabletransfer_out_T3_L2_H2_D32_e2": table_transfer_case(34, 3, 2, 2, 32, 2, 3, 6, 3, True),
+        "tabletransfer_out_T5_L2_H1_D6_e1": table_transfer_case(35, 5, 2, 1, 6, 1, 4, 4, 2, True),
         "gather_r37_b64_n19_i64": gather_case(11, 37, 64, 19, np.int64),
         "gather_r37_b64_n19_i32": gather_case(12, 37, 64, 19, np.int32),
         "gather_r9_b4096_n5_i64": gather_case(13, 9, 4096, 5, np.int64),

@@ -1,0 +1,102 @@
+"""Block-table form of the layout-converting transfer (both directions) on the GPU:
+golden vectors, the C oracle, equivalence with the reference's per-block loop, and the
+host -> device -> host round trip."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import heterofusedkernels_amd  # noqa: F401
+import pcie_through  # noqa: F401
+from heterofusedkernels import memory
+from heterofusedkernels_amd import capi
+from oracle import oracle as O
+
+from gpu_helpers import announce, stream_handle
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda"
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "tabletransfer_*.npz"))))
+def test_golden_table_transfer(path):
+    announce("golden " + os.path.basename(path))
+    g = np.load(path)
+    T, L, H, D, e, to_packed = (int(x) for x in g["geometry"])
+    packed = torch.from_numpy(g["packed"].copy()).to(DEV)
+    layers = torch.from_numpy(g["layers"].copy()).to(DEV)
+    pairs = torch.from_numpy(g["pairs"]).to(DEV)
+    ptrs = torch.tensor([layers[l].data_ptr() for l in range(L)], dtype=torch.int64).to(DEV)
+    capi.check(capi.multi_layer_block_table_transfer(ptrs.data_ptr(), layers.shape[2], packed.data_ptr(),
+                                                     packed.shape[1], pairs.data_ptr(), pairs.shape[0], packed.shape[0],
+                                                     layers.shape[1], T, L, H, D, e, to_packed, 0, stream_handle()))
+    torch.cuda.synchronize()
+    assert np.array_equal(packed.cpu().numpy(), g["packed_expected"])
+    assert np.array_equal(layers.cpu().numpy(), g["layers_expected"])
+
+
+@pytest.mark.parametrize("T,L,H,D,dtype", [(256, 8, 2, 128, torch.int8), (64, 5, 8, 128, torch.bfloat16),
+                                           (1024, 32, 1, 128, torch.int8), (16, 3, 2, 24, torch.float16)])
+def test_block_table_transfer_host_to_device_and_back(T, L, H, D, dtype):
+    e = torch.empty((), dtype=dtype).element_size()
+    host_blocks, dev_blocks, n = 12, 9, 7
+    announce("block-table transfer T=%d L=%d H=%d D=%d %s, %d pairs" % (T, L, H, D, dtype, n))
+    block_bytes = T * L * H * D * e
+    pool = memory.alloc_numa_pinned_tensor(host_blocks * block_bytes)
+    gen = torch.Generator().manual_seed(T + L)
+    pool.copy_(torch.randint(-128, 128, (host_blocks * block_bytes,), dtype=torch.int8, generator=gen))
+    host_pool = pool.view(dtype).view(host_blocks, T, L, H, D)
+    caches = torch.zeros(L, dev_blocks, H, T, D, dtype=dtype, device=DEV)            # per-layer [blocks, H, T, D]
+    ptrs = torch.tensor([caches[l].data_ptr() for l in range(L)], dtype=torch.int64).to(DEV)
+    hb = torch.randperm(host_blocks, generator=gen)[:n]
+    db = torch.randperm(dev_blocks, generator=gen)[:n]
+    pairs = torch.stack([hb, db], 1).contiguous()
+    stride = H * T * D * e
+    torch.ops.pcie_through.multi_layer_block_table_transfer(ptrs, host_pool, pairs.to(DEV), stride, dev_blocks)
+    torch.cuda.synchronize()
+    got = caches.cpu()
+    # oracle
+    want = np.zeros((L, dev_blocks, stride), dtype=np.uint8)
+    O.c_multi_layer_block_table_transfer(want, pool.view(torch.uint8).numpy().reshape(host_blocks, block_bytes),
+                                         pairs.numpy(), T, L, H, D, e, False)
+    assert np.array_equal(got.view(torch.uint8).numpy().reshape(L, dev_blocks, stride), want)
+    # the reference's permute check per block (tests/test_transfer_kernel.py:77-83) ...
+    for j in range(n):
+        transposed = got[:, db[j]].permute(2, 0, 1, 3).contiguous()      # bytes: random payloads hold NaNs
+        assert torch.equal(transposed.view(torch.uint8), host_pool[hb[j]].view(torch.uint8))
+    # ... and equality with its per-block op loop (:58-72)
+    loop = torch.zeros_like(caches)
+    for j in range(n):
+        bptrs = torch.tensor([loop[l, db[j]].data_ptr() for l in range(L)], dtype=torch.int64).to(DEV)
+        torch.ops.pcie_through.multi_layer_block_transfer(bptrs, host_pool[hb[j]], 4)
+    torch.cuda.synchronize()
+    assert torch.equal(loop.cpu().view(torch.uint8), got.view(torch.uint8))
+    # back to other host slots: device -> host, then byte-compare with the original blocks
+    pool2 = memory.alloc_numa_pinned_tensor(host_blocks * block_bytes)
+    host_pool2 = pool2.view(dtype).view(host_blocks, T, L, H, D)
+    hb2 = torch.randperm(host_blocks, generator=gen)[:n]
+    torch.ops.pcie_through.multi_layer_block_table_transfer(ptrs, host_pool2, torch.stack([hb2, db], 1).contiguous().to(DEV),
+                                                            stride, dev_blocks, True)
+    torch.cuda.synchronize()
+    for j in range(n):
+        assert torch.equal(host_pool2[hb2[j]].view(torch.uint8), host_pool[hb[j]].view(torch.uint8))
+    untouched = torch.ones(host_blocks, dtype=torch.bool)
+    untouched[hb2] = False
+    assert int(pool2.view(host_blocks, block_bytes)[untouched].abs().max()) == 0
+
+
+def test_block_table_transfer_skips_out_of_range_pairs():
+    announce("block-table transfer: out-of-range pairs are skipped")
+    T, L, H, D = 8, 2, 2, 64
+    pool = memory.alloc_numa_pinned_tensor(4 * T * L * H * D)
+    pool.fill_(3)
+    caches = torch.zeros(L, 4, H, T, D, dtype=torch.int8, device=DEV)
+    ptrs = torch.tensor([caches[l].data_ptr() for l in range(L)], dtype=torch.int64).to(DEV)
+    pairs = torch.tensor([[0, 1], [4, 2], [1, -1], [2, 4], [3, 3]], dtype=torch.int64).to(DEV)
+    torch.ops.pcie_through.multi_layer_block_table_transfer(ptrs, pool.view(4, T, L, H, D), pairs, H * T * D, 4)
+    torch.cuda.synchronize()
+    got = caches.cpu()
+    assert (got[:, 1] == 3).all() and (got[:, 3] == 3).all() and (got[:, 0] == 0).all() and (got[:, 2] == 0).all()

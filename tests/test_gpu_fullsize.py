@@ -47,9 +47,10 @@ def _device_cache(cfg, blocks):
     return planes, [W.as_bytes(p) for p in planes]
 
 
-def _host_cache(cfg, blocks, max_alloc_gib=8):
+def _host_cache(cfg, blocks, max_alloc_gib=8, skip_on_failure=True):
     """Pinned host planes, allocated in groups of at most max_alloc_gib (one hipHostMalloc of
-    80 GiB is refused on the test machines; the registry handles any number of ranges)."""
+    80 GiB is refused on the test machines; the registry handles any number of ranges).
+    Returns (None, None) instead of skipping when skip_on_failure is False."""
     t0 = time.time()
     plane_bytes = blocks * cfg.block_bytes
     per_alloc = max(1, int(max_alloc_gib * 2**30) // plane_bytes)
@@ -60,6 +61,9 @@ def _host_cache(cfg, blocks, max_alloc_gib=8):
             pool = memory.alloc_numa_pinned_tensor(count * plane_bytes)
         except RuntimeError as exc:
             del pools, planes
+            if not skip_on_failure:
+                announce("  could not pin %.0f GiB of host memory: %s" % (cfg.planes * plane_bytes / 2**30, exc))
+                return None, None
             pytest.skip("could not pin %.0f GiB of host memory: %s" % (cfg.planes * plane_bytes / 2**30, exc))
         pools.append(pool)
         planes.extend(pool.view(torch.uint8).view(count, blocks, cfg.block_bytes).unbind(0))
@@ -92,9 +96,19 @@ def test_config2_llama8b_swap_out_full():
 
 def test_config3_llama70b_swap_in_full():
     cfg = W.C3_LLAMA70B_SWAP_IN
-    _need(80, 41)
+    _need(40, 41)
     announce("config 3 full: 80 layers x {K,V}, pinned [16384,16,8,128] bf16 -> device [8192,...], 1024 blocks")
-    pool, host = _host_cache(cfg, cfg.host_blocks)
+    pool, host = (None, None)
+    if _mem_available_gib() > 130:
+        pool, host = _host_cache(cfg, cfg.host_blocks, skip_on_failure=False)
+    if host is None:
+        # The test machines pin at most 64 GiB per process. Everything else stays as specified
+        # (160 planes, 1024 blocks per launch, device cache of 8192 blocks); only the host pool
+        # the 1024 source blocks are drawn from shrinks from 16384 to 8192 blocks per plane.
+        cfg = cfg.scaled(host_blocks=8192)
+        announce("  host pool scaled down to %d blocks per plane (%.0f GiB)" %
+                 (cfg.host_blocks, cfg.planes * cfg.host_blocks * cfg.block_bytes / 2**30))
+        pool, host = _host_cache(cfg, cfg.host_blocks)
     t0 = time.time()
     for p in range(cfg.planes):                                          # U(-1,1) generated on the device, copied by hipMemcpy
         layer, kv = divmod(p, cfg.kv)

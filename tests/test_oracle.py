@@ -60,6 +60,36 @@ def test_swap_matches_golden(name, g):
         assert np.array_equal(d.numpy(), g["expected"][p]), (name, p)
 
 
+@pytest.mark.parametrize("name,g", _load("tabletransfer"))
+def test_table_transfer_matches_golden(name, g):
+    T, L, H, D, e, to_packed = (int(x) for x in g["geometry"])
+    layers, packed = g["layers"].copy(), g["packed"].copy()
+    O.c_multi_layer_block_table_transfer(layers, packed, g["pairs"], T, L, H, D, e, to_packed, cores=3)
+    assert np.array_equal(layers, g["layers_expected"]) and np.array_equal(packed, g["packed_expected"]), name
+    layers, packed = g["layers"].copy(), g["packed"].copy()
+    O.brute_block_table_transfer(layers, packed, g["pairs"], T, L, H, D, e, to_packed)
+    assert np.array_equal(layers, g["layers_expected"]) and np.array_equal(packed, g["packed_expected"]), name
+
+
+def test_table_transfer_directions_are_inverse_and_match_per_block_loop():
+    """to_packed undoes the reference's direction exactly; the forward direction equals the
+    reference's caller loop, one multi_layer_block_transfer per block
+    (tests/test_transfer_kernel.py:58-72)."""
+    T, L, H, D, e = 12, 3, 2, 32, 2
+    rs = np.random.RandomState(77)
+    packed = rs.randint(0, 256, size=(6, T * L * H * D * e)).astype(np.uint8)
+    layers = np.zeros((L, 5, H * T * D * e), dtype=np.uint8)
+    pairs = np.array([[4, 0], [1, 3], [5, 2]], dtype=np.int64)
+    O.c_multi_layer_block_table_transfer(layers, packed, pairs, T, L, H, D, e, False)
+    for pb, db in pairs:                                   # the per-block loop
+        one = O.c_multi_layer_block_transfer(packed[pb], T, L, H, D, e, cores=4)
+        assert np.array_equal(layers[:, db, :], one)
+    assert not layers[:, [1, 4], :].any()                  # untouched device blocks
+    back = np.zeros_like(packed)
+    O.c_multi_layer_block_table_transfer(layers, back, pairs, T, L, H, D, e, True)
+    assert np.array_equal(back[[4, 1, 5]], packed[[4, 1, 5]]) and not back[[0, 2, 3]].any()
+
+
 # ---- the reference tests' own expected-value expressions --------------------
 @pytest.mark.parametrize("T,L,H,D,dtype", [
     (64, 32, 1, 128, torch.int8),      # tests/test_transfer_kernel.py:15-21 geometry, T cut from 1024
