@@ -39,7 +39,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"],
                     help="c2 (default) = Llama-3-8B swap-out, the configuration the metric is quoted on")
-    ap.add_argument("--sections", default="swap_out,swap_in,gather",
+    ap.add_argument("--sections", default="swap_out,swap_in,gather,duplex",
                     help="comma list of the GPU sections to run; swap_out is the timed step and always runs unless "
                          "a profile of one other kernel alone is wanted")
     ap.add_argument("--skip-cpu-baseline", action="store_true")
@@ -66,7 +66,7 @@ def main():
     cfg = {"c2": W.C2_LLAMA8B_SWAP_OUT, "c3": W.C3_LLAMA70B_SWAP_IN, "c4": W.C4_MLA_ROUNDTRIP,
            "c5": W.C5_FP8_FRAGMENTED}[args.workload]
     sections = set(x for x in args.sections.split(",") if x)
-    assert sections <= {"swap_out", "swap_in", "gather"}, sections
+    assert sections <= {"swap_out", "swap_in", "gather", "duplex"}, sections
     planes, bb, n = cfg.planes, cfg.block_bytes, cfg.n_blocks
     payload = cfg.payload_bytes
     stream = torch.cuda.current_stream().cuda_stream
@@ -189,6 +189,73 @@ def main():
         torch_gather_gbps = 2 * n * bb / (ms_t * 1e6)
         log("gather: %.1f GB/s of HBM traffic (%.1f payload GB/s, %.3f ms/launch), verified; torch.index_select on one "
             "plane: %.1f GB/s" % (gather_traffic_gbps, gather_payload_gbps, kernel_ms_g, torch_gather_gbps))
+
+    # ---- both directions at once on two streams (the link is full duplex) -------------
+    duplex = None
+    if "duplex" in sections:
+        gen = torch.Generator().manual_seed(cfg.base_seed + 77)
+        free_dev = torch.ones(cfg.dev_blocks, dtype=torch.bool)
+        free_dev[src_ids] = False
+        free_dev[back_ids] = False
+        free_host = torch.ones(cfg.host_blocks, dtype=torch.bool)
+        free_host[dst_ids] = False
+        dev_free, host_free = free_dev.nonzero().flatten(), free_host.nonzero().flatten()
+        n2 = min(n, dev_free.numel(), host_free.numel())
+        in_dev = dev_free[torch.randperm(dev_free.numel(), generator=gen)[:n2]]      # disjoint from the swap-out's blocks
+        in_host = host_free[torch.randperm(host_free.numel(), generator=gen)[:n2]]
+        for p in range(planes):                                                      # give the host slots known content
+            host_planes[p][in_host] = dev_bytes[p].index_select(0, ids_dev[:n2]).cpu()
+        pairs_in2 = W.pairs_tensor(in_host, in_dev).to(dev)
+        s_out, s_in = torch.cuda.Stream(), torch.cuda.Stream()
+
+        def both():
+            with torch.cuda.stream(s_out):
+                capi.check(capi.swap_blocks(host_tab.data_ptr(), dev_tab.data_ptr(), pairs_out.data_ptr(), planes, n, bb,
+                                            bb, bb, cfg.dev_blocks, cfg.host_blocks, 0, s_out.cuda_stream))
+            with torch.cuda.stream(s_in):
+                capi.check(capi.swap_blocks(dev_tab.data_ptr(), host_tab.data_ptr(), pairs_in2.data_ptr(), planes, n2, bb,
+                                            bb, bb, cfg.host_blocks, cfg.dev_blocks, 0, s_in.cuda_stream))
+
+        both()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            both()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        for p in range(planes):
+            assert torch.equal(host_planes[p].index_select(0, dst_ids), dev_bytes[p].index_select(0, ids_dev).cpu())
+            assert torch.equal(dev_bytes[p].index_select(0, in_dev.to(dev)).cpu(), host_planes[p].index_select(0, in_host))
+        total = args.steps * (n + n2) * planes * bb
+        # the copy engines doing the same thing: two opposite 512 MiB pinned copies on the two streams
+        half = min(1 << 29, host_pool.numel() // 2)
+        d_a = torch.empty(half, dtype=torch.int8, device=dev)
+        d_b = torch.empty(half, dtype=torch.int8, device=dev)
+        h_a, h_b = host_pool[-half:], host_pool[-2 * half:-half]
+        keep = h_b.clone()                       # these bytes belong to the host cache: put them back afterwards
+
+        def both_memcpy():
+            with torch.cuda.stream(s_out):
+                h_a.copy_(d_a, non_blocking=True)
+            with torch.cuda.stream(s_in):
+                d_b.copy_(h_b, non_blocking=True)
+
+        keep_a = h_a.clone()
+        both_memcpy()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            both_memcpy()
+        torch.cuda.synchronize()
+        dt_m = time.perf_counter() - t0
+        h_a.copy_(keep_a)
+        h_b.copy_(keep)
+        del d_a, d_b, keep, keep_a
+        duplex = {"GBps_both_directions": total / dt / 1e9, "out_blocks": n, "in_blocks": n2,
+                  "pct_of_2x_pcie5_x16": 100 * total / dt / 1e9 / (2 * PCIE5_X16_GBPS),
+                  "memcpy_both_directions_GBps": 5 * 2 * half / dt_m / 1e9}
+        log("duplex (swap-out and swap-in on two streams): %.2f GB/s summed, verified; two opposite hipMemcpyAsync: "
+            "%.2f GB/s summed" % (duplex["GBps_both_directions"], duplex["memcpy_both_directions_GBps"]))
 
     # ---- plain device copy of known size: yardstick for reachable HBM bandwidth, and the
     # calibration row for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters -----------------
@@ -331,6 +398,7 @@ def main():
                     "pct_of_pcie5_x16": None if in_kernel_gbps is None else 100 * in_kernel_gbps / PCIE5_X16_GBPS},
         "pcie_peak_measured": {"d2h_GBps": d2h_peak, "h2d_GBps": h2d_peak, "theoretical_GBps": PCIE5_X16_GBPS,
                                "how": "mean of 5 back-to-back hipMemcpyAsync of %d MiB pinned" % (big >> 20)},
+        "duplex": duplex,
         "memcpy_block_loop": memcpy_loop,
         "cpu_baseline": cpu_baseline,
         "verified": "bit-exact on every plane: " + ", ".join(sorted(sections)),

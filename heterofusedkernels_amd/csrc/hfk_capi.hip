@@ -220,7 +220,12 @@ void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, bool to_p
 int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64_t* pairs, uint64_t n_pairs,
                      uint64_t packed_stride, uint64_t layered_stride, uint64_t packed_blocks,
                      uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
-                     bool to_packed, uint32_t workgroups, hipStream_t s) {
+                     bool to_packed, bool packed_is_host, uint32_t workgroups, hipStream_t s) {
+    // With the packed side in host memory the PCIe link is the bound and a small grid is
+    // best (measured optimum 64-256 workgroups, both directions); twice the swap default.
+    if (workgroups == 0 && packed_is_host) {
+        workgroups = 2u * (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
+    }
     TransposeArgs a;
     uint32_t unit = 16;
     int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, packed, pairs, n_pairs, packed_stride, layered_stride,
@@ -273,8 +278,8 @@ int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i
 int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* src_block, uint32_t T,
                                    uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
                                    uint32_t workgroups, hfk_stream_t stream) {
-    return launch_transpose(dev_layer_ptrs, src_block, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, workgroups,
-                            static_cast<hipStream_t>(stream));
+    return launch_transpose(dev_layer_ptrs, src_block, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, true,
+                            workgroups, static_cast<hipStream_t>(stream));
 }
 
 int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* host_block,
@@ -288,7 +293,8 @@ int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs, cons
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipMemcpyAsync(staging, host_block, bytes, hipMemcpyHostToDevice, s);
     if (e != hipSuccess) return (int)e;
-    return launch_transpose(dev_layer_ptrs, staging, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, workgroups, s);
+    return launch_transpose(dev_layer_ptrs, staging, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, false,
+                            workgroups, s);
 }
 
 int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t dev_block_stride,
@@ -301,7 +307,7 @@ int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t de
     if (block_pairs == nullptr) return HFK_ERR_NULL_POINTER;
     return launch_transpose(dev_layer_ptrs, packed_blocks, block_pairs, n_pairs, packed_block_stride,
                             dev_block_stride, n_packed_blocks, n_dev_blocks, T, L, H, D, elem_bytes, to_packed != 0,
-                            workgroups, static_cast<hipStream_t>(stream));
+                            true, workgroups, static_cast<hipStream_t>(stream));
 }
 
 int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* block_pairs,

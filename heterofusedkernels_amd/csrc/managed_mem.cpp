@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstring>
 #include <fstream>
+#include <iterator>
 #include <mutex>
 #include <string>
 
@@ -65,7 +66,17 @@ const RegisteredMemoryRecord* HostRegisteredMemoryManager::adoptMapping(void* ho
     const uintptr_t start = reinterpret_cast<uintptr_t>(hostPtr);
     const std::unique_lock<std::shared_mutex> guard(mux_);
     auto hit = records_.find(start);
-    if (hit != records_.end()) return &hit->second;
+    if (hit != records_.end()) {
+        // Same start again: idempotent. A longer range over memory this library does not
+        // own (it was pinned elsewhere and may have been re-used at a new size) grows the
+        // record, provided it still ends before the next one.
+        RegisteredMemoryRecord& r = hit->second;
+        if (bufferSize > r.buffSize && r.kind == HFK_MM_KIND_ADOPTED && kind == HFK_MM_KIND_ADOPTED) {
+            auto next = std::next(hit);
+            if (next == records_.end() || next->first - start >= bufferSize) r.buffSize = bufferSize;
+        }
+        return &r;
+    }
     if (overlapsOther(start, bufferSize)) {
         t_last_error = HFK_MM_ERR_OVERLAP;
         return nullptr;
@@ -84,7 +95,7 @@ const RegisteredMemoryRecord* HostRegisteredMemoryManager::registerHostPtr(void*
     {
         const std::shared_lock<std::shared_mutex> guard(mux_);
         auto hit = records_.find(start);
-        if (hit != records_.end()) return &hit->second;  // idempotent
+        if (hit != records_.end() && bufferSize <= hit->second.buffSize) return &hit->second;  // idempotent
         // A range inside an existing record is already device-visible.
         const RegisteredMemoryRecord* outer = findContaining(start);
         if (outer != nullptr && start + bufferSize <= outer->ptr + outer->buffSize) return outer;

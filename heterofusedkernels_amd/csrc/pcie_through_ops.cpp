@@ -10,6 +10,7 @@
 #include <ATen/ATen.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <hip/hip_runtime_api.h>
 #include <torch/library.h>
 
 #include <optional>
@@ -33,24 +34,24 @@ void check_aiv(const std::optional<int64_t>& aiv) {
     }
 }
 
-// Address a kernel can use for the tensor's first element. Device tensors are
-// used as they are; host tensors must be registered (heterofusedkernels.memory)
-// or at least pinned, in which case their storage is registered on first use.
+// Address a kernel can use for the tensor's first element. Device tensors are used
+// as they are; host tensors must be registered (heterofusedkernels.memory) or at
+// least pinned. A pinned tensor that was never registered is resolved through the
+// HIP runtime on every call and nothing is recorded for it: torch's pinned
+// allocator recycles its blocks, so a recorded range could outlive the tensor.
 // The reference passes an unchecked nullptr to the kernel here
 // (gather_torch.cpp:51, multi_layer_block_transfer_torch.cpp:78).
 void* device_visible(const at::Tensor& t, const char* what) {
     if (t.is_cuda()) return t.data_ptr();
     TORCH_CHECK(t.device().is_cpu(), what, ": unsupported device ", t.device());
-    auto& registry = HostRegisteredMemoryManager::GetInstance();
-    void* dev = registry.getDevicePtr(t.data_ptr());
+    void* dev = HostRegisteredMemoryManager::GetInstance().getDevicePtr(t.data_ptr());
     if (dev != nullptr) return dev;
     TORCH_CHECK(t.is_pinned(), what,
                 ": host tensor is neither registered with heterofusedkernels.memory nor pinned");
-    const auto& storage = t.storage();
-    TORCH_CHECK(registry.registerHostPtr(storage.mutable_data(), storage.nbytes()) != nullptr, what,
-                ": registering the pinned host tensor failed");
-    dev = registry.getDevicePtr(t.data_ptr());
-    TORCH_CHECK(dev != nullptr, what, ": no device-visible address for host tensor");
+    const hipError_t e = hipHostGetDevicePointer(&dev, t.data_ptr(), 0);
+    if (e != hipSuccess) (void)hipGetLastError();
+    TORCH_CHECK(e == hipSuccess && dev != nullptr, what, ": no device-visible address for the pinned host tensor: ",
+                hipGetErrorString(e));
     return dev;
 }
 
@@ -261,6 +262,9 @@ TORCH_LIBRARY(pcie_through, m) {
     m.def(
         "fused_memcpy_multi_layer_block_transfer(Tensor deviceBlockCachePtrs, Tensor hostBlockCache, Tensor "
         "stagingBlockCache, int? aiv=None) -> ()");
+    // Same op with the written tensor annotated as mutated, for tracing / functionalization
+    // (the reference notes the missing annotation at multi_layer_block_transfer_torch.cpp:57).
+    m.def("gather_into(Tensor gmEmbed, Tensor(a!) gmEmbedDst, Tensor gmIds, int? aiv=None) -> ()");
     m.def(
         "multi_layer_block_table_transfer(Tensor deviceLayerCachePtrs, Tensor hostBlockPool, Tensor blockPairs, int "
         "deviceBlockStride, int deviceBlocks=0, bool toHost=False, int? workgroups=None) -> ()");
@@ -279,6 +283,7 @@ TORCH_LIBRARY_IMPL(pcie_through, CUDA, m) {
     m.impl("gather", TORCH_FN(pciethrough::gather));
     m.impl("multi_layer_block_transfer", TORCH_FN(pciethrough::multi_layer_block_transfer));
     m.impl("fused_memcpy_multi_layer_block_transfer", TORCH_FN(pciethrough::fused_memcpy_multi_layer_block_transfer));
+    m.impl("gather_into", TORCH_FN(pciethrough::gather));
     m.impl("multi_layer_block_table_transfer", TORCH_FN(pciethrough::multi_layer_block_table_transfer));
     m.impl("swap_blocks", TORCH_FN(pciethrough::swap_blocks));
     m.impl("gather_blocks", TORCH_FN(pciethrough::gather_blocks));

@@ -121,11 +121,85 @@ def transfer_table(out, blocks=8):
                 assert torch.equal(got[b].permute(2, 0, 1, 3), host_blocks[b]), "transfer mismatch"
             row[name + "_ms"] = ms
             row[name + "_GBps"] = nbytes / (ms * 1e6)
+        # all blocks in one launch through the block table, host -> device and device -> host
+        caches = torch.zeros(L, blocks, H, T, D, dtype=torch.int8, device=dev)
+        lptrs = torch.tensor([caches[l].data_ptr() for l in range(L)], dtype=torch.int64).to(dev)
+        pairs = torch.stack([torch.arange(blocks), torch.arange(blocks).flip(0)], 1).contiguous().to(dev)
+        host_pool = pool.view(blocks, T, L, H, D)
+        back_pool = memory.alloc_numa_pinned_tensor(blocks * nbytes).view(blocks, T, L, H, D)
+        for name, to_host, hp in (("table_in", False, host_pool), ("table_out", True, back_pool)):
+            def call_table():
+                torch.ops.pcie_through.multi_layer_block_table_transfer(lptrs, hp, pairs, H * T * D, blocks, to_host)
+            call_table()
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for _ in range(5):
+                call_table()
+            e.record()
+            torch.cuda.synchronize()
+            ms = s.elapsed_time(e) / 5
+            row[name + "_ms"] = ms
+            row[name + "_GBps"] = blocks * nbytes / (ms * 1e6)
+        got = caches.cpu()
+        for b in range(blocks):
+            assert torch.equal(got[:, blocks - 1 - b].permute(2, 0, 1, 3), host_blocks[b]), "table transfer mismatch"
+        assert torch.equal(back_pool, host_pool), "table transfer round trip mismatch"
         out["transfer"].append(row)
-        print("transfer [%d,%d,%d,%d] int8: direct %.3f ms (%.2f GB/s) | staged %.3f ms (%.2f GB/s)" %
-              (T, L, H, D, row["direct_ms"], row["direct_GBps"], row["staged_ms"], row["staged_GBps"]),
-              file=sys.stderr, flush=True)
+        print("transfer [%d,%d,%d,%d] int8: direct %.3f ms (%.2f GB/s) | staged %.3f ms (%.2f GB/s) | %d blocks in one "
+              "launch: in %.2f GB/s, out %.2f GB/s" %
+              (T, L, H, D, row["direct_ms"], row["direct_GBps"], row["staged_ms"], row["staged_GBps"], blocks,
+               row["table_in_GBps"], row["table_out_GBps"]), file=sys.stderr, flush=True)
+        del back_pool, host_pool
         del pool, host_blocks
+
+
+def config1_latency(out, runs=500):
+    """Single-layer paged KV gather of the benchmark's first configuration: K and V caches
+    [1024, 16, 8, 128] fp16, 32 block ids -> [32, 16, 8, 128] each. 1 MiB per call: launch latency."""
+    from heterofusedkernels_amd import workloads as W
+    cfg = W.C1_GATHER_FP16
+    dev = "cuda"
+    ids = W.gather_ids(cfg).to(dev)
+    planes = [W.make_plane(cfg, 0, kv, cfg.dev_blocks).to(dev) for kv in range(2)]
+    outs = [torch.empty((32,) + cfg.block_shape, dtype=cfg.dtype, device=dev) for _ in range(2)]
+
+    def ours():
+        for kv in range(2):
+            torch.ops.pcie_through.gather(planes[kv], outs[kv], ids)
+
+    def torch_path():
+        for kv in range(2):
+            torch.index_select(planes[kv], 0, ids, out=outs[kv])
+
+    res = {}
+    for name, fn in (("pcie_through.gather", ours), ("torch.index_select", torch_path)):
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(runs):
+            fn()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / runs
+        res[name] = {"us_per_K_and_V": dt * 1e6, "payload_GBps": 2 * 32 * cfg.block_bytes / dt / 1e9}
+    for kv in range(2):
+        torch.ops.pcie_through.gather(planes[kv], outs[kv], ids)
+        torch.cuda.synchronize()
+        assert torch.equal(outs[kv].view(torch.int16), planes[kv].index_select(0, ids).view(torch.int16))
+    cpu_planes = [p.cpu() for p in planes]
+    cpu_ids = ids.cpu()
+    t0 = time.perf_counter()
+    for _ in range(runs):
+        for kv in range(2):
+            cpu_planes[kv].index_select(0, cpu_ids)
+    dt = (time.perf_counter() - t0) / runs
+    res["torch CPU index_select (%d threads)" % torch.get_num_threads()] = {
+        "us_per_K_and_V": dt * 1e6, "payload_GBps": 2 * 32 * cfg.block_bytes / dt / 1e9}
+    out["config1"] = res
+    for k, v in res.items():
+        print("config 1 (K+V, 32 blocks of 32 KiB each): %-40s %.1f us, %.1f GB/s payload" %
+              (k, v["us_per_K_and_V"], v["payload_GBps"]), file=sys.stderr, flush=True)
 
 
 def main():
@@ -135,6 +209,7 @@ def main():
     args = ap.parse_args()
     assert torch.cuda.is_available()
     out = {"gather": [], "transfer": [], "rows": args.rows, "runs": args.runs}
+    config1_latency(out)
     gather_table(args.rows, args.runs, out)
     transfer_table(out)
     print(json.dumps(out))

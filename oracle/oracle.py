@@ -126,7 +126,7 @@ def c_swap_blocks(dst_planes_u8, src_planes_u8, pairs):
 
 
 # ----------------------------------------------------------------------------
-# torch CPU path (the statement the north-star names, and the timed CPU baseline)
+# torch CPU path (index_select / index_copy_ over the same block table; also the timed CPU baseline)
 # ----------------------------------------------------------------------------
 def torch_gather_rows(table, ids):
     """dst = table.index_select(0, ids) == table[ids] (tests/test_memcpy.py:18)."""

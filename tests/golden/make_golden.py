@@ -91,7 +91,7 @@ def swap_case(seed, planes, src_blocks, dst_blocks, block_bytes, n_pairs):
 
 def main():
     cases = {
-        # (T, L, H, D, elem): SURVEY-sized tiny brute force incl. all four element sizes
+        # (T, L, H, D, elem): tiny brute-force shapes covering element sizes 1, 2 and 4
         "transfer_T2_L3_H2_D16_e1": transfer_case(1, 2, 3, 2, 16, 1),
         "transfer_T2_L3_H2_D16_e2": transfer_case(2, 2, 3, 2, 16, 2),
         "transfer_T2_L3_H2_D16_e4": transfer_case(3, 2, 3, 2, 16, 4),

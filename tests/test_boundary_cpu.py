@@ -161,6 +161,19 @@ def test_registry_idempotent_overlap_and_unregister(mm):
     assert b"overlap" in mm.hfk_mm_status_string(-2)
 
 
+def test_registry_adopted_record_grows_but_never_into_its_neighbour(mm):
+    assert mm.hfk_mm_adopt(0x10000, 0x900000, 0x1000, 0) == 0
+    assert mm.hfk_mm_adopt(0x14000, 0xA00000, 0x1000, 0) == 0
+    assert mm.hfk_mm_adopt(0x10000, 0x900000, 0x3000, 0) == 0      # same start, longer: record grows
+    assert mm.hfk_mm_record_size(0x10000) == 0x3000
+    assert mm.hfk_mm_get_device_ptr(0x12fff) == 0x902fff
+    assert mm.hfk_mm_adopt(0x10000, 0x900000, 0x5000, 0) == 0      # would run into 0x14000: size kept
+    assert mm.hfk_mm_record_size(0x10000) == 0x3000
+    assert mm.hfk_mm_get_device_ptr(0x14010) == 0xA00010
+    assert mm.hfk_mm_adopt(0x10000, 0x900000, 0x800, 0) == 0       # shorter: unchanged
+    assert mm.hfk_mm_record_size(0x10000) == 0x3000
+
+
 def test_registry_is_thread_safe(mm):
     # managed_mem.h:31: writers exclude, readers share
     errors = []

@@ -110,6 +110,10 @@ def test_config1_gather_fp16_exact():
         torch.ops.pcie_through.gather(plane.view(cfg.dev_blocks, -1).to(DEV), out2, ids.to(DEV), aiv=4)
         torch.cuda.synchronize()
         assert np.array_equal(bytes_np(out2), bytes_np(want))
+        out3 = torch.zeros_like(out2)                                   # alias-annotated variant
+        torch.ops.pcie_through.gather_into(plane.view(cfg.dev_blocks, -1).to(DEV), out3, ids.to(DEV))
+        torch.cuda.synchronize()
+        assert np.array_equal(bytes_np(out3), bytes_np(want))
 
 
 # ---------------------------------------------------------------------------
@@ -133,6 +137,26 @@ def test_gather_from_registered_host_table(memory, bs, id_dtype):
     torch.ops.pcie_through.gather(embed, dst2, ids.to(DEV))              # default aiv (test_gather_combine.py:51-55)
     torch.cuda.synchronize()
     assert torch.equal(dst2.cpu().view(torch.int16), dst.cpu().view(torch.int16))
+
+
+def test_gather_from_torch_pinned_table_without_registration(memory):
+    """A tensor pinned by torch itself can be handed to the op directly; nothing is recorded for it."""
+    announce("host-table gather from a torch.pin_memory() tensor, never registered")
+    gen = torch.Generator().manual_seed(5)
+    embed = torch.randn(3000, 512, generator=gen).to(torch.float16).pin_memory()
+    ids = torch.randint(0, 3000, (77,), generator=gen)
+    n0 = memory.record_count()
+    dst = torch.zeros(77, 512, dtype=torch.float16, device=DEV)
+    torch.ops.pcie_through.gather(embed, dst, ids.to(DEV))
+    torch.cuda.synchronize()
+    assert np.array_equal(bytes_np(dst), bytes_np(embed[ids]))
+    assert memory.record_count() == n0
+    sub = embed[1000:]                                          # interior view of the pinned block
+    torch.ops.pcie_through.gather(sub, dst, ids.to(DEV) % 2000)
+    torch.cuda.synchronize()
+    assert np.array_equal(bytes_np(dst), bytes_np(sub[ids % 2000]))
+    with pytest.raises(RuntimeError, match="neither registered"):
+        torch.ops.pcie_through.gather(torch.zeros(8, 512, dtype=torch.float16), dst, ids.to(DEV))
 
 
 # ---------------------------------------------------------------------------
