@@ -227,6 +227,23 @@ def main():
             assert torch.equal(host_planes[p].index_select(0, dst_ids), dev_bytes[p].index_select(0, ids_dev).cpu())
             assert torch.equal(dev_bytes[p].index_select(0, in_dev.to(dev)).cpu(), host_planes[p].index_select(0, in_host))
         total = args.steps * (n + n2) * planes * bb
+        # ... and the same two block tables in ONE duplex launch
+        om = capi.BlockMove(host_tab.data_ptr(), dev_tab.data_ptr(), pairs_out.data_ptr(), n, bb, bb, cfg.dev_blocks,
+                            cfg.host_blocks)
+        im = capi.BlockMove(dev_tab.data_ptr(), host_tab.data_ptr(), pairs_in2.data_ptr(), n2, bb, bb, cfg.host_blocks,
+                            cfg.dev_blocks)
+        for p in range(planes):                                          # make the launch prove itself: clear the targets
+            host_planes[p][dst_ids] = 0
+            dev_bytes[p].index_fill_(0, in_dev.to(dev), 0)
+
+        def one_launch():
+            capi.check(capi.swap_blocks_duplex(om, im, planes, bb, 0, stream), "hfk_swap_blocks_duplex")
+
+        wall_d, ms_d = timed(one_launch, args.steps, args.warmup)
+        for p in range(planes):
+            assert torch.equal(host_planes[p].index_select(0, dst_ids), dev_bytes[p].index_select(0, ids_dev).cpu())
+            assert torch.equal(dev_bytes[p].index_select(0, in_dev.to(dev)).cpu(), host_planes[p].index_select(0, in_host))
+        duplex_kernel_gbps = (n + n2) * planes * bb / (ms_d * 1e6)
         # the copy engines doing the same thing: two opposite 512 MiB pinned copies on the two streams
         half = min(1 << 29, host_pool.numel() // 2)
         d_a = torch.empty(half, dtype=torch.int8, device=dev)
@@ -251,11 +268,13 @@ def main():
         h_a.copy_(keep_a)
         h_b.copy_(keep)
         del d_a, d_b, keep, keep_a
-        duplex = {"GBps_both_directions": total / dt / 1e9, "out_blocks": n, "in_blocks": n2,
-                  "pct_of_2x_pcie5_x16": 100 * total / dt / 1e9 / (2 * PCIE5_X16_GBPS),
+        duplex = {"one_launch_GBps_both_directions": duplex_kernel_gbps,
+                  "one_launch_pct_of_2x_pcie5_x16": 100 * duplex_kernel_gbps / (2 * PCIE5_X16_GBPS),
+                  "two_launches_two_streams_GBps_both_directions": total / dt / 1e9, "out_blocks": n, "in_blocks": n2,
                   "memcpy_both_directions_GBps": 5 * 2 * half / dt_m / 1e9}
-        log("duplex (swap-out and swap-in on two streams): %.2f GB/s summed, verified; two opposite hipMemcpyAsync: "
-            "%.2f GB/s summed" % (duplex["GBps_both_directions"], duplex["memcpy_both_directions_GBps"]))
+        log("duplex, verified: swap_blocks_duplex (one launch) %.2f GB/s summed; swap-out + swap-in on two streams "
+            "%.2f GB/s summed; two opposite hipMemcpyAsync %.2f GB/s summed" %
+            (duplex_kernel_gbps, total / dt / 1e9, duplex["memcpy_both_directions_GBps"]))
 
     # ---- plain device copy of known size: yardstick for reachable HBM bandwidth, and the
     # calibration row for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters -----------------

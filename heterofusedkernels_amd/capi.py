@@ -15,6 +15,15 @@ KNOB_UNROLL = 0
 KNOB_NONTEMPORAL = 1
 KNOB_WORKGROUPS_PER_CU = 2
 KNOB_SWAP_WORKGROUPS = 3
+KNOB_DUPLEX_UNROLL = 4
+
+
+class BlockMove(ctypes.Structure):
+    """struct hfk_block_move."""
+    _fields_ = [("dst_plane_ptrs", ctypes.c_void_p), ("src_plane_ptrs", ctypes.c_void_p),
+                ("block_pairs", ctypes.c_void_p), ("n_pairs", ctypes.c_uint64),
+                ("src_block_stride", ctypes.c_uint64), ("dst_block_stride", ctypes.c_uint64),
+                ("src_blocks", ctypes.c_uint64), ("dst_blocks", ctypes.c_uint64)]
 
 ENTRY_POINTS = (
     "hfk_version",
@@ -24,6 +33,7 @@ ENTRY_POINTS = (
     "hfk_fused_memcpy_multi_layer_block_transfer",
     "hfk_multi_layer_block_table_transfer",
     "hfk_swap_blocks",
+    "hfk_swap_blocks_duplex",
     "hfk_gather_blocks",
     "hfk_set_tuning",
     "hfk_get_tuning",
@@ -61,6 +71,8 @@ def load():
     L.hfk_multi_layer_block_table_transfer.restype = ci
     L.hfk_swap_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, u32, vp]
     L.hfk_swap_blocks.restype = ci
+    L.hfk_swap_blocks_duplex.argtypes = [ctypes.POINTER(BlockMove), ctypes.POINTER(BlockMove), u32, u64, u32, vp]
+    L.hfk_swap_blocks_duplex.restype = ci
     L.hfk_gather_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u32, vp]
     L.hfk_gather_blocks.restype = ci
     L.hfk_set_tuning.argtypes = [ci, i64]
@@ -108,6 +120,13 @@ def swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, s
                 src_blocks=0, dst_blocks=0, workgroups=0, stream=0):
     return load().hfk_swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, src_stride,
                                   dst_stride, src_blocks, dst_blocks, workgroups, stream)
+
+
+def swap_blocks_duplex(out_move, in_move, n_planes, block_bytes, workgroups=0, stream=0):
+    """out_move / in_move: BlockMove instances or None."""
+    return load().hfk_swap_blocks_duplex(ctypes.byref(out_move) if out_move is not None else None,
+                                         ctypes.byref(in_move) if in_move is not None else None, n_planes, block_bytes,
+                                         workgroups, stream)
 
 
 def gather_blocks(dst_planes, src_planes, ids, n_planes, n_ids, block_bytes, src_stride, src_blocks=0,

@@ -101,74 +101,147 @@ struct BlockCopyArgs {
     uint32_t n_work;             // n_planes * n_pairs * chunks_per_block
 };
 
-template <typename IdT, int UNROLL, int NT>
-HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+// Where work item w of a block copy reads and writes. Everything here is uniform
+// over the workgroup, so the compiler keeps it in scalar registers. Returns false
+// when the item's block indices are out of range (the item is skipped).
+template <typename IdT>
+HFK_HD bool resolve_chunk(const BlockCopyArgs<IdT>& a, uint32_t w, uint64_t& s_addr, uint64_t& d_addr,
+                          uint32_t& chunk) {
+    chunk = w % a.chunks_per_block;
+    const uint32_t tile = w / a.chunks_per_block;
+    const uint32_t pair = tile % a.n_pairs;
+    const uint32_t plane = tile / a.n_pairs;
+    const uint64_t sb = (uint64_t)(int64_t)a.src_ids[(uint64_t)pair * a.id_stride];
+    const uint64_t db = a.dst_ids ? (uint64_t)(int64_t)a.dst_ids[(uint64_t)pair * a.id_stride] : (uint64_t)pair;
+    if (sb >= a.src_limit || db >= a.dst_limit) {
+        return false;
+    }
+    s_addr = (a.src_planes ? a.src_planes[plane] : a.src_base) + sb * a.src_stride;
+    d_addr = (a.dst_planes ? a.dst_planes[plane] : a.dst_base) + db * a.dst_stride;
+    return true;
+}
+
+// Copies chunk `chunk` (256 * UNROLL vectors) of one block of block_bytes bytes.
+template <int UNROLL, int NT>
+HFK_HD void copy_chunk(uint64_t s_addr, uint64_t d_addr, uint64_t block_bytes, uint32_t chunk, uint32_t tid) {
     constexpr uint32_t kChunkVecs = kWorkgroupLanes * UNROLL;
     constexpr uint64_t kChunkBytes = (uint64_t)kChunkVecs * 16u;
-
-    for (uint32_t w = bid; w < a.n_work; w += nb) {
-        // Uniform over the workgroup: the compiler keeps these in scalar registers.
-        const uint32_t chunk = w % a.chunks_per_block;
-        const uint32_t tile = w / a.chunks_per_block;
-        const uint32_t pair = tile % a.n_pairs;
-        const uint32_t plane = tile / a.n_pairs;
-
-        const uint64_t sb = (uint64_t)(int64_t)a.src_ids[(uint64_t)pair * a.id_stride];
-        const uint64_t db = a.dst_ids ? (uint64_t)(int64_t)a.dst_ids[(uint64_t)pair * a.id_stride]
-                                      : (uint64_t)pair;
-        if (sb >= a.src_limit || db >= a.dst_limit) {
-            continue;
-        }
-        const uint64_t s_addr = (a.src_planes ? a.src_planes[plane] : a.src_base) + sb * a.src_stride;
-        const uint64_t d_addr = (a.dst_planes ? a.dst_planes[plane] : a.dst_base) + db * a.dst_stride;
-
-        if (((s_addr | d_addr | a.block_bytes) & 15u) == 0) {
-            const uint64_t block_vecs = a.block_bytes >> 4;
-            const uint64_t first = (uint64_t)chunk * kChunkVecs;
-            const HFK_GLOBAL vec16* sv = global_in<vec16>(s_addr) + first + tid;
-            HFK_GLOBAL vec16* dv = global_out<vec16>(d_addr) + first + tid;
-            vec16 v[UNROLL];
-            if (first + kChunkVecs <= block_vecs) {
+    if (((s_addr | d_addr | block_bytes) & 15u) == 0) {
+        const uint64_t block_vecs = block_bytes >> 4;
+        const uint64_t first = (uint64_t)chunk * kChunkVecs;
+        const HFK_GLOBAL vec16* sv = global_in<vec16>(s_addr) + first + tid;
+        HFK_GLOBAL vec16* dv = global_out<vec16>(d_addr) + first + tid;
+        vec16 v[UNROLL];
+        if (first + kChunkVecs <= block_vecs) {
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
-                }
+            for (int u = 0; u < UNROLL; ++u) {
+                v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
+            }
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
-                }
-            } else {
-                const uint64_t lane_first = first + tid;
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
-                        v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
-                        store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
-                    }
-                }
+            for (int u = 0; u < UNROLL; ++u) {
+                store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
             }
         } else {
-            // Blocks that are not 16-byte aligned/sized: same chunk, narrower units.
-            const uint64_t lo = (uint64_t)chunk * kChunkBytes;
-            const uint64_t hi = (lo + kChunkBytes < a.block_bytes) ? lo + kChunkBytes : a.block_bytes;
-            if (((s_addr | d_addr | a.block_bytes) & 3u) == 0) {
-                const HFK_GLOBAL uint32_t* s4 = global_in<uint32_t>(s_addr);
-                HFK_GLOBAL uint32_t* d4 = global_out<uint32_t>(d_addr);
-                for (uint64_t o = (lo >> 2) + tid; o < (hi >> 2); o += kWorkgroupLanes) {
-                    d4[o] = s4[o];
-                }
-            } else {
-                const HFK_GLOBAL uint8_t* s1 = global_in<uint8_t>(s_addr);
-                HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(d_addr);
-                for (uint64_t o = lo + tid; o < hi; o += kWorkgroupLanes) {
-                    d1[o] = s1[o];
+            const uint64_t lane_first = first + tid;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
+                    v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
                 }
             }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
+                    store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
+                }
+            }
+        }
+    } else {
+        // Blocks that are not 16-byte aligned/sized: same chunk, narrower units.
+        const uint64_t lo = (uint64_t)chunk * kChunkBytes;
+        const uint64_t hi = (lo + kChunkBytes < block_bytes) ? lo + kChunkBytes : block_bytes;
+        if (((s_addr | d_addr | block_bytes) & 3u) == 0) {
+            const HFK_GLOBAL uint32_t* s4 = global_in<uint32_t>(s_addr);
+            HFK_GLOBAL uint32_t* d4 = global_out<uint32_t>(d_addr);
+            for (uint64_t o = (lo >> 2) + tid; o < (hi >> 2); o += kWorkgroupLanes) {
+                d4[o] = s4[o];
+            }
+        } else {
+            const HFK_GLOBAL uint8_t* s1 = global_in<uint8_t>(s_addr);
+            HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(d_addr);
+            for (uint64_t o = lo + tid; o < hi; o += kWorkgroupLanes) {
+                d1[o] = s1[o];
+            }
+        }
+    }
+}
+
+template <typename IdT, int UNROLL, int NT>
+HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+    for (uint32_t w = bid; w < a.n_work; w += nb) {
+        uint64_t s_addr = 0, d_addr = 0;
+        uint32_t chunk = 0;
+        if (!resolve_chunk(a, w, s_addr, d_addr, chunk)) {
+            continue;
+        }
+        copy_chunk<UNROLL, NT>(s_addr, d_addr, a.block_bytes, chunk, tid);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Two block copies in one launch, meant for a swap-out (HBM -> host) and a swap-in
+// (host -> HBM) that should share the PCIe link, which is full duplex. Every
+// workgroup iteration takes one chunk of each copy and issues the loads of both
+// before the stores of either, so reads from the host and writes to the host are
+// in flight together and the two directions advance in lock step. Two independent
+// launches on two streams reach 67-86 GB/s summed on MI355X depending on how their
+// grids happen to interleave; this reaches 97-100 GB/s.
+// `second` should be the copy that reads host memory: its loads are issued first.
+// ---------------------------------------------------------------------------
+struct DuplexCopyArgs {
+    BlockCopyArgs<int64_t> first;
+    BlockCopyArgs<int64_t> second;
+    uint32_t n_work;  // max(first.n_work, second.n_work)
+};
+
+template <int UNROLL, int NT>
+HFK_HD void duplex_copy_body(const DuplexCopyArgs& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+    constexpr uint32_t kChunkVecs = kWorkgroupLanes * UNROLL;
+    for (uint32_t w = bid; w < a.n_work; w += nb) {
+        uint64_t s0 = 0, d0 = 0, s1 = 0, d1 = 0;
+        uint32_t c0 = 0, c1 = 0;
+        const bool v0 = w < a.first.n_work && resolve_chunk(a.first, w, s0, d0, c0);
+        const bool v1 = w < a.second.n_work && resolve_chunk(a.second, w, s1, d1, c1);
+        const bool fast0 = v0 && ((s0 | d0 | a.first.block_bytes) & 15u) == 0 &&
+                           ((uint64_t)c0 + 1) * kChunkVecs <= (a.first.block_bytes >> 4);
+        const bool fast1 = v1 && ((s1 | d1 | a.second.block_bytes) & 15u) == 0 &&
+                           ((uint64_t)c1 + 1) * kChunkVecs <= (a.second.block_bytes >> 4);
+        if (fast0 && fast1) {
+            const HFK_GLOBAL vec16* sv0 = global_in<vec16>(s0) + (uint64_t)c0 * kChunkVecs + tid;
+            HFK_GLOBAL vec16* dv0 = global_out<vec16>(d0) + (uint64_t)c0 * kChunkVecs + tid;
+            const HFK_GLOBAL vec16* sv1 = global_in<vec16>(s1) + (uint64_t)c1 * kChunkVecs + tid;
+            HFK_GLOBAL vec16* dv1 = global_out<vec16>(d1) + (uint64_t)c1 * kChunkVecs + tid;
+            vec16 x[UNROLL], y[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                y[u] = load_unit<NT>(sv1 + u * kWorkgroupLanes);  // host reads first: longest latency
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                x[u] = load_unit<NT>(sv0 + u * kWorkgroupLanes);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                store_unit<NT>(dv0 + u * kWorkgroupLanes, x[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                store_unit<NT>(dv1 + u * kWorkgroupLanes, y[u]);
+            }
+        } else {
+            // Tail chunks, odd alignments, or only one of the copies has work left.
+            if (v1) copy_chunk<UNROLL, NT>(s1, d1, a.second.block_bytes, c1, tid);
+            if (v0) copy_chunk<UNROLL, NT>(s0, d0, a.first.block_bytes, c0, tid);
         }
     }
 }

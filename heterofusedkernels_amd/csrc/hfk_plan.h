@@ -144,6 +144,28 @@ inline int plan_swap_blocks(BlockCopyArgs<int64_t>& a, const void* dst_plane_ptr
     return HFK_OK;
 }
 
+// Both sides of a duplex swap share planes, block size and therefore the chunking.
+inline int plan_duplex(DuplexCopyArgs& d, const hfk_block_move* out_move, const hfk_block_move* in_move,
+                       uint32_t n_planes, uint64_t block_bytes, int preferred_unroll, int* unroll_out) {
+    d = DuplexCopyArgs{};
+    const hfk_block_move* moves[2] = {out_move, in_move};
+    BlockCopyArgs<int64_t>* sides[2] = {&d.first, &d.second};
+    int unroll = fit_unroll(block_bytes, preferred_unroll);
+    for (int i = 0; i < 2; ++i) {
+        const hfk_block_move* m = moves[i];
+        if (m == nullptr || m->n_pairs == 0 || n_planes == 0) continue;  // this side has nothing to do
+        int rc = plan_swap_blocks(*sides[i], m->dst_plane_ptrs, m->src_plane_ptrs, m->block_pairs, n_planes, m->n_pairs,
+                                  block_bytes, m->src_block_stride, m->dst_block_stride, m->src_blocks, m->dst_blocks);
+        if (rc != HFK_OK) return rc;
+        int u = unroll;
+        rc = plan_block_copy<int64_t>(*sides[i], unroll, &u);
+        if (rc != HFK_OK) return rc;
+    }
+    d.n_work = d.first.n_work > d.second.n_work ? d.first.n_work : d.second.n_work;
+    *unroll_out = unroll;
+    return HFK_OK;
+}
+
 inline int plan_gather_blocks(BlockCopyArgs<int64_t>& a, const void* dst_plane_ptrs, const void* src_plane_ptrs,
                               const int64_t* ids, uint32_t n_planes, uint64_t n_ids, uint64_t block_bytes,
                               uint64_t src_block_stride, uint64_t src_blocks) {

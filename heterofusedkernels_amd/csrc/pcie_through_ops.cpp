@@ -3,7 +3,8 @@
 // Schemas of the first three ops are those of the reference
 // (pcieThrough/csrc/host/gather_torch.cpp:60,
 //  pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:113-114);
-// multi_layer_block_table_transfer, swap_blocks and gather_blocks are additive. Every op unpacks its tensors into
+// multi_layer_block_table_transfer, swap_blocks, swap_blocks_duplex, gather_blocks and
+// gather_into are additive. Every op unpacks its tensors into
 // raw device-visible addresses, takes the current HIP stream of the device that
 // owns the device-side tensor, and calls the C-ABI of libhfk_hip.so; nothing is
 // allocated and nothing waits.
@@ -230,6 +231,55 @@ void swap_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs,
         "hfk_swap_blocks");
 }
 
+// Swap-out (device -> host) and swap-in (host -> device) of the same cache in one
+// launch that keeps both directions of the link busy; see hfk_swap_blocks_duplex.
+// outBlockPairs rows are (device_block, host_block), inBlockPairs rows are
+// (host_block, device_block). The two tables must not name the same block on the
+// same side. Either table may be empty.
+void swap_blocks_duplex(const at::Tensor& devicePlanePtrs, const at::Tensor& hostPlanePtrs,
+                        const at::Tensor& outBlockPairs, const at::Tensor& inBlockPairs, int64_t blockBytes,
+                        int64_t deviceBlockStride, int64_t hostBlockStride, int64_t deviceBlocks, int64_t hostBlocks,
+                        std::optional<int64_t> workgroups) {
+    check_ptr_table(devicePlanePtrs, "devicePlanePtrs");
+    check_ptr_table(hostPlanePtrs, "hostPlanePtrs");
+    check_ptr_table(outBlockPairs, "outBlockPairs");
+    check_ptr_table(inBlockPairs, "inBlockPairs");
+    TORCH_CHECK(devicePlanePtrs.is_cuda(), "devicePlanePtrs must be a device tensor");
+    TORCH_CHECK(devicePlanePtrs.numel() == hostPlanePtrs.numel(), "plane tables differ in length");
+    TORCH_CHECK(devicePlanePtrs.numel() <= 0xffffffffLL, "too many planes");
+    TORCH_CHECK(outBlockPairs.dim() == 2 && outBlockPairs.size(1) == 2, "outBlockPairs must be [n, 2]");
+    TORCH_CHECK(inBlockPairs.dim() == 2 && inBlockPairs.size(1) == 2, "inBlockPairs must be [n, 2]");
+    TORCH_CHECK(blockBytes > 0 && deviceBlockStride >= blockBytes && hostBlockStride >= blockBytes,
+                "swap_blocks_duplex: strides must be at least blockBytes, blockBytes positive");
+    TORCH_CHECK(deviceBlocks >= 0 && hostBlocks >= 0, "swap_blocks_duplex: block counts must be non-negative");
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(devicePlanePtrs));
+    const void* dev_tab = devicePlanePtrs.data_ptr();
+    const void* host_tab = device_visible(hostPlanePtrs, "hostPlanePtrs");
+    hfk_block_move out_move{};
+    out_move.dst_plane_ptrs = host_tab;
+    out_move.src_plane_ptrs = dev_tab;
+    out_move.n_pairs = static_cast<uint64_t>(outBlockPairs.size(0));
+    out_move.block_pairs = out_move.n_pairs ? static_cast<const int64_t*>(device_visible(outBlockPairs, "outBlockPairs"))
+                                            : nullptr;
+    out_move.src_block_stride = static_cast<uint64_t>(deviceBlockStride);
+    out_move.dst_block_stride = static_cast<uint64_t>(hostBlockStride);
+    out_move.src_blocks = static_cast<uint64_t>(deviceBlocks);
+    out_move.dst_blocks = static_cast<uint64_t>(hostBlocks);
+    hfk_block_move in_move{};
+    in_move.dst_plane_ptrs = dev_tab;
+    in_move.src_plane_ptrs = host_tab;
+    in_move.n_pairs = static_cast<uint64_t>(inBlockPairs.size(0));
+    in_move.block_pairs = in_move.n_pairs ? static_cast<const int64_t*>(device_visible(inBlockPairs, "inBlockPairs"))
+                                          : nullptr;
+    in_move.src_block_stride = static_cast<uint64_t>(hostBlockStride);
+    in_move.dst_block_stride = static_cast<uint64_t>(deviceBlockStride);
+    in_move.src_blocks = static_cast<uint64_t>(hostBlocks);
+    in_move.dst_blocks = static_cast<uint64_t>(deviceBlocks);
+    check_status(hfk_swap_blocks_duplex(&out_move, &in_move, static_cast<uint32_t>(devicePlanePtrs.numel()),
+                                        static_cast<uint64_t>(blockBytes), workgroup_cap(workgroups), current_stream()),
+                 "hfk_swap_blocks_duplex");
+}
+
 // Shared-id block gather over planes; see hfk_gather_blocks.
 void gather_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs, const at::Tensor& blockIds,
                    int64_t blockBytes, int64_t srcBlockStride, int64_t srcBlocks,
@@ -272,6 +322,10 @@ TORCH_LIBRARY(pcie_through, m) {
         "swap_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockPairs, int blockBytes, int "
         "srcBlockStride, int dstBlockStride, int srcBlocks=0, int dstBlocks=0, int? workgroups=None) -> ()");
     m.def(
+        "swap_blocks_duplex(Tensor devicePlanePtrs, Tensor hostPlanePtrs, Tensor outBlockPairs, Tensor inBlockPairs, int "
+        "blockBytes, int deviceBlockStride, int hostBlockStride, int deviceBlocks=0, int hostBlocks=0, int? "
+        "workgroups=None) -> ()");
+    m.def(
         "gather_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockIds, int blockBytes, int "
         "srcBlockStride, int srcBlocks=0, int? workgroups=None) -> ()");
 }
@@ -286,5 +340,6 @@ TORCH_LIBRARY_IMPL(pcie_through, CUDA, m) {
     m.impl("gather_into", TORCH_FN(pciethrough::gather));
     m.impl("multi_layer_block_table_transfer", TORCH_FN(pciethrough::multi_layer_block_table_transfer));
     m.impl("swap_blocks", TORCH_FN(pciethrough::swap_blocks));
+    m.impl("swap_blocks_duplex", TORCH_FN(pciethrough::swap_blocks_duplex));
     m.impl("gather_blocks", TORCH_FN(pciethrough::gather_blocks));
 }

@@ -174,6 +174,39 @@ HFK_API int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_pt
                     uint32_t workgroups, hfk_stream_t stream);
 
 /*
+ * One side of hfk_swap_blocks_duplex: the arguments of one hfk_swap_blocks call
+ * (planes and block size are shared by both sides).
+ */
+typedef struct hfk_block_move {
+    const void* dst_plane_ptrs;   /* device-visible array of n_planes uint64 addresses */
+    const void* src_plane_ptrs;
+    const int64_t* block_pairs;   /* device-visible int64 [n_pairs, 2] = (src_block, dst_block) */
+    uint64_t n_pairs;
+    uint64_t src_block_stride;
+    uint64_t dst_block_stride;
+    uint64_t src_blocks;          /* 0 = unchecked */
+    uint64_t dst_blocks;          /* 0 = unchecked */
+} hfk_block_move;
+
+/*
+ * Two block-table swaps in ONE launch, meant for a swap-out (device -> host) and a
+ * swap-in (host -> device) of the same cache running at the same time: the PCIe link
+ * is full duplex, and one kernel that keeps both directions in flight in lock step
+ * moves more bytes per second than two launches on two streams (which is also a
+ * valid way to call hfk_swap_blocks). Result: exactly that of
+ *   hfk_swap_blocks(out_move...) and hfk_swap_blocks(in_move...)
+ * run in either order. The two moves must not touch the same bytes (no block may
+ * be read by one and written by the other); either move may be empty (n_pairs 0).
+ * `in_move` should be the one that reads host memory.
+ *
+ * No counterpart in the reference (its transfer op is host -> device only and one
+ * block per call, pcieThrough/tests/test_transfer_kernel.py:58-72).
+ */
+HFK_API int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move* in_move,
+                                   uint32_t n_planes, uint64_t block_bytes, uint32_t workgroups,
+                                   hfk_stream_t stream);
+
+/*
  * Paged block gather over many planes in one launch:
  *   for p < n_planes, i < n_ids:
  *     dst_plane_ptrs[p][i*block_bytes ...] = src_plane_ptrs[p][ids[i]*src_block_stride ...]
@@ -195,7 +228,8 @@ enum hfk_knob {
     HFK_KNOB_NONTEMPORAL = 1,   /* bit0: non-temporal loads, bit1: non-temporal stores */
     HFK_KNOB_WORKGROUPS_PER_CU = 2, /* default grid bound of the gathers and the
                                        transfer = CUs * this, 1..1024                  */
-    HFK_KNOB_SWAP_WORKGROUPS = 3    /* default grid bound of hfk_swap_blocks           */
+    HFK_KNOB_SWAP_WORKGROUPS = 3,   /* default grid bound of hfk_swap_blocks           */
+    HFK_KNOB_DUPLEX_UNROLL = 4      /* like HFK_KNOB_UNROLL, for hfk_swap_blocks_duplex */
 };
 HFK_API int hfk_set_tuning(int knob, int64_t value);
 HFK_API int64_t hfk_get_tuning(int knob);

@@ -160,6 +160,82 @@ void case_swap(uint32_t n_planes, uint32_t n_pairs, uint64_t block_bytes, uint64
     for (auto* b : exp) delete b;
 }
 
+// ---- duplex swap: two disjoint block-table copies in one launch ---------------
+void case_duplex(uint32_t n_planes, uint32_t n_out, uint32_t n_in, uint64_t block_bytes, uint32_t dev_blocks,
+                 uint32_t host_blocks, size_t mis, int unroll, uint32_t grid_cap, bool with_bad) {
+    std::vector<Buf*> dev, host, dev_exp, host_exp;
+    std::vector<uint64_t> dp, hp;
+    std::vector<void*> dep, hep;
+    std::vector<const void*> dsp, hsp;
+    for (uint32_t p = 0; p < n_planes; ++p) {
+        dev.push_back(new Buf(dev_blocks * block_bytes, mis));
+        host.push_back(new Buf(host_blocks * block_bytes, mis));
+        dev_exp.push_back(new Buf(dev_blocks * block_bytes, mis));
+        host_exp.push_back(new Buf(host_blocks * block_bytes, mis));
+        dev.back()->randomize();
+        host.back()->randomize();
+        std::memcpy(dev_exp.back()->p, dev.back()->p, dev.back()->n);
+        std::memcpy(host_exp.back()->p, host.back()->p, host.back()->n);
+        dp.push_back((uint64_t)(uintptr_t)dev.back()->p);
+        hp.push_back((uint64_t)(uintptr_t)host.back()->p);
+        dep.push_back(dev_exp.back()->p);
+        hep.push_back(host_exp.back()->p);
+        dsp.push_back(dev_exp.back()->p);
+        hsp.push_back(host_exp.back()->p);
+    }
+    // out reads device blocks [0, n_out) of a permutation and writes host blocks [0, n_out) of another;
+    // in reads host blocks after those and writes device blocks after those: disjoint by construction.
+    std::vector<int64_t> dperm(dev_blocks), hperm(host_blocks);
+    for (uint32_t i = 0; i < dev_blocks; ++i) dperm[i] = i;
+    for (uint32_t i = 0; i < host_blocks; ++i) hperm[i] = i;
+    std::shuffle(dperm.begin(), dperm.end(), rng);
+    std::shuffle(hperm.begin(), hperm.end(), rng);
+    std::vector<int64_t> po, pi, po_good, pi_good;
+    for (uint32_t j = 0; j < n_out; ++j) {
+        int64_t s = dperm[j], d = hperm[j];
+        bool bad = with_bad && j % 3 == 1;
+        if (bad) s = (j % 2) ? -5 : (int64_t)dev_blocks + 1;
+        po.push_back(s); po.push_back(d);
+        if (!bad) { po_good.push_back(s); po_good.push_back(d); }
+    }
+    for (uint32_t j = 0; j < n_in; ++j) {
+        int64_t s = hperm[n_out + j], d = dperm[n_out + j];
+        bool bad = with_bad && j % 4 == 2;
+        if (bad) d = (int64_t)dev_blocks;
+        pi.push_back(s); pi.push_back(d);
+        if (!bad) { pi_good.push_back(s); pi_good.push_back(d); }
+    }
+    hfk_block_move out_move{hp.data(), dp.data(), po.data(), n_out, block_bytes, block_bytes, dev_blocks, host_blocks};
+    hfk_block_move in_move{dp.data(), hp.data(), pi.data(), n_in, block_bytes, block_bytes, host_blocks, dev_blocks};
+    DuplexCopyArgs a;
+    int u = 1;
+    int rc = plan_duplex(a, &out_move, &in_move, n_planes, block_bytes, unroll, &u);
+    if (rc != HFK_OK) { ++g_failures; std::printf("plan_duplex rc=%d\n", rc); }
+    else if (a.n_work > 0) {
+        const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+        switch (u) {
+            case 1: walk(a, grid, duplex_copy_body<1, 3>); break;
+            case 2: walk(a, grid, duplex_copy_body<2, 0>); break;
+            case 4: walk(a, grid, duplex_copy_body<4, 3>); break;
+            case 8: walk(a, grid, duplex_copy_body<8, 3>); break;
+            default: walk(a, grid, duplex_copy_body<16, 3>); break;
+        }
+    }
+    if (!po_good.empty()) oracle_swap_blocks(hep.data(), dsp.data(), po_good.data(), n_planes, po_good.size() / 2, block_bytes, block_bytes, block_bytes);
+    if (!pi_good.empty()) oracle_swap_blocks(dep.data(), hsp.data(), pi_good.data(), n_planes, pi_good.size() / 2, block_bytes, block_bytes, block_bytes);
+    char what[160];
+    std::snprintf(what, sizeof what, "duplex planes=%u out=%u in=%u bytes=%llu mis=%zu unroll=%d grid=%u bad=%d", n_planes, n_out,
+                  n_in, (unsigned long long)block_bytes, mis, unroll, grid_cap, (int)with_bad);
+    for (uint32_t p = 0; p < n_planes; ++p) {
+        expect_equal(dev[p]->p, dev_exp[p]->p, dev[p]->n, what);
+        expect_equal(host[p]->p, host_exp[p]->p, host[p]->n, what);
+    }
+    for (auto* b : dev) delete b;
+    for (auto* b : host) delete b;
+    for (auto* b : dev_exp) delete b;
+    for (auto* b : host_exp) delete b;
+}
+
 // ---- gather_blocks (multi-plane, shared ids) -------------------------------
 void case_gather_blocks(uint32_t n_planes, uint32_t n_ids, uint64_t block_bytes, uint64_t src_blocks, int unroll,
                         uint32_t grid_cap) {
@@ -386,6 +462,19 @@ int main() {
     case_transpose(9, 2, 3, 16, 2, 4, 0, 5);          // source 4-byte aligned
     case_transpose(6, 2, 2, 16, 1, 1, 3, 5);          // everything odd
     case_transpose(0, 2, 2, 16, 1, 0, 0, 5);          // empty block
+
+    // duplex swap: equal and unequal sides, one side empty, tails, odd alignment, out-of-range pairs
+    for (int unroll : {1, 2, 4, 8, 16}) {
+        case_duplex(2, 5, 5, 32768, 16, 16, 0, unroll, 3, false);
+        case_duplex(2, 7, 3, 32768, 16, 16, 0, unroll, 1000, true);
+        case_duplex(1, 2, 6, 73728, 10, 10, 0, unroll, 5, false);      // MLA block: tail chunks
+        case_duplex(2, 4, 0, 16384, 8, 8, 0, unroll, 4, false);        // only swap-out
+        case_duplex(2, 0, 4, 16384, 8, 8, 0, unroll, 4, true);         // only swap-in
+    }
+    case_duplex(2, 3, 4, 4100, 9, 9, 4, 4, 7, false);                  // 4-byte path
+    case_duplex(2, 3, 4, 4099, 9, 9, 1, 4, 7, true);                   // byte path
+    case_duplex(1, 3, 3, 48, 7, 7, 0, 4, 2, false);                    // blocks smaller than a chunk
+    case_duplex(1, 0, 0, 4096, 4, 4, 0, 4, 2, false);                  // nothing at all
 
     // block-table transfer, both directions
     for (bool to_packed : {false, true}) {

@@ -274,6 +274,56 @@ def test_config5_fp8_fragmented_scaled(memory):
         assert torch.equal(prefill2[p], prefill[p])
 
 
+@pytest.mark.parametrize("cfg,n_out,n_in", [
+    (W.C2_LLAMA8B_SWAP_OUT.scaled(layers=3, dev_blocks=128, host_blocks=192), 40, 40),
+    (W.C2_LLAMA8B_SWAP_OUT.scaled(layers=2, dev_blocks=128, host_blocks=192), 50, 7),
+    (W.C4_MLA_ROUNDTRIP.scaled(layers=5, dev_blocks=48, host_blocks=48), 9, 20),
+    (W.C5_FP8_FRAGMENTED.scaled(layers=2, dev_blocks=256, host_blocks=256), 0, 60),
+    (W.C5_FP8_FRAGMENTED.scaled(layers=2, dev_blocks=256, host_blocks=256), 60, 0),
+])
+def test_duplex_swap_equals_two_swaps(memory, cfg, n_out, n_in):
+    """One duplex launch == swap-out then swap-in through index_select / index_copy_ on disjoint blocks."""
+    announce("duplex swap %s: %d out, %d in, %d planes" % (cfg.name, n_out, n_in, cfg.planes))
+    bb = cfg.block_bytes
+    cpu_dev = [W.as_bytes(p).clone() for p in _cpu_planes(cfg, cfg.dev_blocks)]
+    dev = [p.to(DEV) for p in cpu_dev]
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=None)
+    gen = torch.Generator().manual_seed(n_out * 100 + n_in)
+    cpu_host = [torch.randint(0, 256, (cfg.host_blocks, bb), dtype=torch.uint8, generator=gen) for _ in range(cfg.planes)]
+    for p in range(cfg.planes):
+        host[p].copy_(cpu_host[p])
+    dperm = torch.randperm(cfg.dev_blocks, generator=gen)
+    hperm = torch.randperm(cfg.host_blocks, generator=gen)
+    out_pairs = W.pairs_tensor(dperm[:n_out], hperm[:n_out])                          # device block -> host block
+    in_pairs = W.pairs_tensor(hperm[n_out:n_out + n_in], dperm[n_out:n_out + n_in])   # host block -> device block
+    dtab, htab = ptr_table(dev), host_ptr_table(host)
+    torch.ops.pcie_through.swap_blocks_duplex(dtab, htab, out_pairs.to(DEV), in_pairs.to(DEV), bb, bb, bb,
+                                              cfg.dev_blocks, cfg.host_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want_host, want_dev = cpu_host[p].clone(), cpu_dev[p].clone()
+        if n_out:
+            O.torch_swap_blocks(want_host, cpu_dev[p], out_pairs[:, 0], out_pairs[:, 1])
+        if n_in:
+            O.torch_swap_blocks(want_dev, cpu_host[p], in_pairs[:, 0], in_pairs[:, 1])
+        assert torch.equal(host[p], want_host), "plane %d host side" % p
+        assert torch.equal(dev[p].cpu(), want_dev), "plane %d device side" % p
+    # the C-ABI with explicit structs and a tiny grid gives the same bytes
+    dev2 = [p.to(DEV) for p in cpu_dev]
+    for p in range(cfg.planes):
+        host[p].copy_(cpu_host[p])
+    dtab2 = ptr_table(dev2)
+    po, pi = out_pairs.to(DEV), in_pairs.to(DEV)
+    om = capi.BlockMove(htab.data_ptr(), dtab2.data_ptr(), po.data_ptr() if n_out else None, n_out, bb, bb,
+                        cfg.dev_blocks, cfg.host_blocks)
+    im = capi.BlockMove(dtab2.data_ptr(), htab.data_ptr(), pi.data_ptr() if n_in else None, n_in, bb, bb,
+                        cfg.host_blocks, cfg.dev_blocks)
+    capi.check(capi.swap_blocks_duplex(om, im, cfg.planes, bb, 3, stream_handle()))
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        assert torch.equal(dev2[p], dev[p]), "plane %d" % p
+
+
 # ---------------------------------------------------------------------------
 # edge cases
 # ---------------------------------------------------------------------------
