@@ -67,6 +67,7 @@ def main():
            "c5": W.C5_FP8_FRAGMENTED}[args.workload]
     sections = set(x for x in args.sections.split(",") if x)
     assert sections <= {"swap_out", "swap_in", "gather", "duplex"}, sections
+    CONFIG_HOST_BLOCKS = cfg.host_blocks
     planes, bb, n = cfg.planes, cfg.block_bytes, cfg.n_blocks
     payload = cfg.payload_bytes
     stream = torch.cuda.current_stream().cuda_stream
@@ -79,10 +80,33 @@ def main():
     log("device cache: %d planes x %d blocks x %d B = %.2f GiB (%.1fs)" %
         (planes, cfg.dev_blocks, bb, planes * cfg.dev_blocks * bb / 2**30, time.time() - t0))
     t0 = time.time()
-    host_pool = memory.alloc_numa_pinned_tensor(planes * cfg.host_blocks * bb)
-    host_planes = list(host_pool.view(torch.uint8).view(planes, cfg.host_blocks, bb).unbind(0))
-    log("pinned host cache: %d blocks per plane = %.2f GiB (%.1fs, NUMA node %d)" %
-        (cfg.host_blocks, planes * cfg.host_blocks * bb / 2**30, time.time() - t0, memory.device_numa_node(0)))
+    # Pinned host cache, in allocations of at most 8 GiB (one huge hipHostMalloc is refused on some
+    # machines). If the machine will not pin the whole pool, the pool is halved and the run says so.
+    host_blocks = cfg.host_blocks
+    while True:
+        plane_bytes = host_blocks * bb
+        per_alloc = max(1, (8 << 30) // plane_bytes)
+        host_pools, host_planes = [], []
+        try:
+            for first in range(0, planes, per_alloc):
+                count = min(per_alloc, planes - first)
+                pool = memory.alloc_numa_pinned_tensor(count * plane_bytes)
+                host_pools.append(pool)
+                host_planes.extend(pool.view(torch.uint8).view(count, host_blocks, bb).unbind(0))
+            break
+        except RuntimeError as exc:
+            del host_pools, host_planes
+            if host_blocks // 2 < 2 * n:
+                raise
+            log("could not pin %.1f GiB (%s); halving the host pool" % (planes * plane_bytes / 2**30, str(exc)[:80]))
+            host_blocks //= 2
+    if host_blocks != cfg.host_blocks:
+        from dataclasses import replace
+        cfg = replace(cfg, host_blocks=host_blocks)
+    host_pool = host_pools[0]
+    log("pinned host cache: %d blocks per plane = %.2f GiB in %d allocations (%.1fs, NUMA node %d)" %
+        (cfg.host_blocks, planes * cfg.host_blocks * bb / 2**30, len(host_pools), time.time() - t0,
+         memory.device_numa_node(0)))
     dev_bytes = [W.as_bytes(t) for t in dev_planes]           # uint8 views, same storage
     dev_tab = pcie_through.plane_pointer_table(dev_planes, dev)
     host_tab = pcie_through.plane_pointer_table(host_planes, dev)
@@ -315,7 +339,7 @@ def main():
     # ---- CPU baseline: the torch CPU path on this box's host cores ----------------
     cpu_baseline = None
     if not args.skip_cpu_baseline:
-        sample_planes = planes       # the whole block table: a few planes alone would sit in the CPU's L3
+        sample_planes = min(planes, 64)   # the whole block table where it fits: a few planes alone sit in the CPU's L3
         cpu_src = [dev_planes[p].cpu() for p in range(sample_planes)]
         if cfg.dtype == torch.float8_e4m3fn:      # CPU index ops on fp8 are not guaranteed: move its bytes
             cpu_src = [s.view(torch.uint8) for s in cpu_src]
@@ -388,6 +412,7 @@ def main():
         "dtype": "u8", "data": "synthetic",
         "config": {"workload": cfg.name, "planes": planes, "layers": cfg.layers, "block_bytes": bb,
                    "blocks_per_launch": n, "device_blocks": cfg.dev_blocks, "host_blocks": cfg.host_blocks,
+                   "host_blocks_specified": CONFIG_HOST_BLOCKS,
                    "payload_bytes_per_step": payload, "cache_dtype": str(cfg.dtype).replace("torch.", "")},
         # Dominant kernel of the step. A swap never touches HBM twice; the resource it saturates is the
         # PCIe Gen5 x16 link, so that is the roofline it is priced against (theoretical link rate as

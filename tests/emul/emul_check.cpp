@@ -489,6 +489,39 @@ int main() {
         case_transpose_table(64, 2, 1, 128, 1, 3, 3, 3, 0, 0, 0, 0, to_packed, false, 2);      // one-head blocks
     }
 
+    // seeded random shapes on top of the hand-picked ones
+    auto pick = [&](std::initializer_list<uint64_t> v) { return *(v.begin() + rng() % v.size()); };
+    const int kUnrolls[5] = {1, 2, 4, 8, 16};
+    for (int it = 0; it < 150; ++it) {
+        const int unroll = kUnrolls[rng() % 5];
+        const uint32_t grid = (uint32_t)pick({1, 2, 3, 7, 33, 100000});
+        const uint64_t bytes = pick({16, 48, 4096, 4112, 8192, 12288 + 16, 16384, 32768, 36864, 65536 + 32, 73728, 1000, 4099, 20});
+        const uint32_t planes = 1 + rng() % 3, sb = 2 + rng() % 9, db = 2 + rng() % 9;
+        const uint32_t np = 1 + rng() % db;   // destination blocks must be distinct
+        const uint64_t pad_s = pick({0, 0, 16, 64}), pad_d = pick({0, 0, 16, 48});
+        const size_t mis = (bytes % 16) ? (size_t)pick({0, 1, 4}) : 0;
+        case_swap(planes, np, bytes, sb, db, (bytes % 16) ? 0 : pad_s, (bytes % 16) ? 0 : pad_d, mis, mis, unroll, grid,
+                  rng() % 2);
+        if (it % 3 == 0) case_gather_blocks(planes, np, bytes - bytes % 16 + 16, sb, unroll, grid);
+        if (it % 3 == 1) case_duplex(planes, rng() % 5, rng() % 5, bytes, 12, 12, mis, unroll, grid, rng() % 2);
+    }
+    for (int it = 0; it < 120; ++it) {
+        const uint64_t rb = pick({1, 3, 16, 20, 64, 100, 256, 1024, 1040, 2048, 4080, 4095, 4096, 5000, 8192, 8200});
+        const uint64_t rows = 1 + rng() % 40, n_ids = rng() % 70;
+        const size_t tm = (rb % 16) ? (size_t)pick({0, 1, 4, 8}) : 0, dm = (rb % 16) ? (size_t)pick({0, 2, 4}) : 0;
+        if (rng() % 2) case_gather_rows<int64_t>(rows, n_ids, rb, tm, dm, kUnrolls[rng() % 5], 1 + rng() % 50, rng() % 2, rng() % 2);
+        else case_gather_rows<int32_t>(rows, n_ids, rb, tm, dm, kUnrolls[rng() % 5], 1 + rng() % 50, rng() % 2, rng() % 2);
+    }
+    for (int it = 0; it < 120; ++it) {
+        const uint32_t T = 1 + rng() % 20, L = 1 + rng() % 4, H = 1 + rng() % 4;
+        const uint32_t D = (uint32_t)pick({1, 4, 7, 8, 16, 24, 32, 64, 128}), e = (uint32_t)pick({1, 2, 4});
+        const bool aligned = ((uint64_t)D * e) % 16 == 0;
+        const size_t m1 = aligned ? 0 : (size_t)pick({0, 1, 4}), m2 = (size_t)pick({0, 0, 4, 3});
+        if (it % 2 == 0) case_transpose(T, L, H, D, e, m1, m2, 1 + rng() % 20);
+        else case_transpose_table(T, L, H, D, e, 3 + rng() % 4, 3 + rng() % 4, 1 + rng() % 3, aligned ? pick({0, 16, 64}) : 0,
+                                  aligned ? pick({0, 32}) : 0, m1, m2, rng() % 2, rng() % 2, 1 + rng() % 20);
+    }
+
     std::printf("%d comparisons, %d failures\n", g_cases, g_failures);
     return g_failures == 0 ? 0 : 1;
 }
