@@ -39,9 +39,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"],
                     help="c2 (default) = Llama-3-8B swap-out, the configuration the metric is quoted on")
-    ap.add_argument("--sections", default="swap_out,swap_in,gather,duplex",
+    ap.add_argument("--sections", default="swap_out,swap_in,gather,duplex,staged",
                     help="comma list of the GPU sections to run; swap_out is the timed step and always runs unless "
                          "a profile of one other kernel alone is wanted")
+    ap.add_argument("--tune", default="", help="comma list of library knobs for experiments, e.g. unroll=4,nt=0 "
+                    "(unroll, nt, wg_per_cu, swap_wgs, duplex_unroll); defaults are the shipped ones")
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--skip-memcpy-loop", action="store_true")
     args = ap.parse_args()
@@ -60,17 +62,27 @@ def main():
     from heterofusedkernels_amd import _build, capi
     from heterofusedkernels_amd import workloads as W
 
+    knobs = {"unroll": capi.KNOB_UNROLL, "nt": capi.KNOB_NONTEMPORAL, "wg_per_cu": capi.KNOB_WORKGROUPS_PER_CU,
+             "swap_wgs": capi.KNOB_SWAP_WORKGROUPS, "duplex_unroll": capi.KNOB_DUPLEX_UNROLL}
+    tuned = {}
+    for item in filter(None, args.tune.split(",")):
+        key, val = item.split("=")
+        capi.check(capi.set_tuning(knobs[key], int(val)), "hfk_set_tuning(%s)" % item)
+        tuned[key] = int(val)
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
     cfg = {"c2": W.C2_LLAMA8B_SWAP_OUT, "c3": W.C3_LLAMA70B_SWAP_IN, "c4": W.C4_MLA_ROUNDTRIP,
            "c5": W.C5_FP8_FRAGMENTED}[args.workload]
     sections = set(x for x in args.sections.split(",") if x)
-    assert sections <= {"swap_out", "swap_in", "gather", "duplex"}, sections
+    assert sections <= {"swap_out", "swap_in", "gather", "duplex", "staged"}, sections
     CONFIG_HOST_BLOCKS = cfg.host_blocks
     planes, bb, n = cfg.planes, cfg.block_bytes, cfg.n_blocks
     payload = cfg.payload_bytes
     stream = torch.cuda.current_stream().cuda_stream
+    # Two extra streams for the sections that run things side by side. Created once, first: HIP maps
+    # streams onto a few hardware queues round-robin, and two streams that share a queue do not overlap.
+    stream_a, stream_b = torch.cuda.Stream(), torch.cuda.Stream()
 
     # ---- caches -------------------------------------------------------------
     t0 = time.time()
@@ -230,7 +242,7 @@ def main():
         for p in range(planes):                                                      # give the host slots known content
             host_planes[p][in_host] = dev_bytes[p].index_select(0, ids_dev[:n2]).cpu()
         pairs_in2 = W.pairs_tensor(in_host, in_dev).to(dev)
-        s_out, s_in = torch.cuda.Stream(), torch.cuda.Stream()
+        s_out, s_in = stream_a, stream_b
 
         def both():
             with torch.cuda.stream(s_out):
@@ -299,6 +311,97 @@ def main():
         log("duplex, verified: swap_blocks_duplex (one launch) %.2f GB/s summed; swap-out + swap-in on two streams "
             "%.2f GB/s summed; two opposite hipMemcpyAsync %.2f GB/s summed" %
             (duplex_kernel_gbps, total / dt / 1e9, duplex["memcpy_both_directions_GBps"]))
+
+    # ---- staged swap (gather kernel on HBM + DMA copies) and what each path costs a kernel beside it ----
+    staged = None
+    if "staged" in sections:
+        run_start = 0          # the earlier sections' results are verified by now: their host slots may be reused
+        host_run = torch.arange(run_start, run_start + n)
+        host_addrs = torch.tensor([t.data_ptr() for t in host_planes], dtype=torch.int64)
+        staging_buf = torch.empty(planes, n, bb, dtype=torch.uint8, device=dev)
+
+        def staged_out(st=None):
+            capi.check(capi.swap_blocks_staged(dev_tab.data_ptr(), host_addrs.data_ptr(), ids_dev.data_ptr(),
+                                               host_run.data_ptr(), planes, n, bb, bb, bb, cfg.dev_blocks,
+                                               cfg.host_blocks, staging_buf.data_ptr(), True, 0,
+                                               stream if st is None else st), "hfk_swap_blocks_staged(out)")
+
+        back_dev = back_ids.to(dev)
+
+        def staged_in():
+            capi.check(capi.swap_blocks_staged(dev_tab.data_ptr(), host_addrs.data_ptr(), back_dev.data_ptr(),
+                                               host_run.data_ptr(), planes, n, bb, bb, bb, cfg.dev_blocks,
+                                               cfg.host_blocks, staging_buf.data_ptr(), False, 0, stream),
+                       "hfk_swap_blocks_staged(in)")
+
+        _, ms_so = timed(staged_out, args.steps, args.warmup)
+        for p in range(planes):
+            assert torch.equal(host_planes[p][run_start:run_start + n], dev_bytes[p].index_select(0, ids_dev).cpu())
+        _, ms_si = timed(staged_in, args.steps, args.warmup)
+        for p in range(planes):
+            assert torch.equal(dev_bytes[p].index_select(0, back_dev).cpu(), host_planes[p][run_start:run_start + n])
+        # both directions at once on two streams (two DMA engines); disjoint device blocks and host runs
+        staging_b = torch.empty(planes, n, bb, dtype=torch.uint8, device=dev)
+        run_b = torch.arange(run_start + n, run_start + 2 * n)
+
+        def staged_both():
+            capi.check(capi.swap_blocks_staged(dev_tab.data_ptr(), host_addrs.data_ptr(), ids_dev.data_ptr(),
+                                               host_run.data_ptr(), planes, n, bb, bb, bb, cfg.dev_blocks,
+                                               cfg.host_blocks, staging_buf.data_ptr(), True, 0, stream_a.cuda_stream))
+            capi.check(capi.swap_blocks_staged(dev_tab.data_ptr(), host_addrs.data_ptr(), back_dev.data_ptr(),
+                                               run_b.data_ptr(), planes, n, bb, bb, bb, cfg.dev_blocks,
+                                               cfg.host_blocks, staging_b.data_ptr(), False, 0, stream_b.cuda_stream))
+
+        staged_both()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            staged_both()
+        torch.cuda.synchronize()
+        staged_duplex_gbps = args.steps * 2 * payload / (time.perf_counter() - t0) / 1e9
+        del staging_b
+        # a compute kernel on another stream: alone, beside the direct swap-out, beside the staged swap-out
+        side, comp = stream_a, stream_b
+        ga = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        gb = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        for _ in range(3):
+            torch.mm(ga, gb)
+
+        def gemm_ms(side_fn, reps):
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            if side_fn is not None:
+                for _ in range(reps):
+                    side_fn(side.cuda_stream)
+            with torch.cuda.stream(comp):
+                e0.record()
+                for _ in range(40):
+                    torch.mm(ga, gb)
+                e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / 40
+
+        def direct_out(st):
+            capi.check(capi.swap_blocks(host_tab.data_ptr(), dev_tab.data_ptr(), pairs_out.data_ptr(), planes, n, bb, bb,
+                                        bb, cfg.dev_blocks, cfg.host_blocks, 0, st), "hfk_swap_blocks(out)")
+
+        gemm_alone = gemm_ms(None, 0)
+        reps = max(1, int(round(40 * gemm_alone / (payload / 55e6))))      # side work lasting about as long as the GEMMs
+        gemm_direct = gemm_ms(direct_out, reps)
+        gemm_staged = gemm_ms(staged_out, reps)
+        del ga, gb, staging_buf
+        staged = {"swap_out_GBps": payload / (ms_so * 1e6), "swap_in_GBps": payload / (ms_si * 1e6),
+                  "out_and_in_on_two_streams_GBps": staged_duplex_gbps,
+                  "host_slots": "one run of %d consecutive slots per plane (%d DMA copies of %.1f MiB per launch)" %
+                                (n, planes, n * bb / 2**20),
+                  "gemm_8192_bf16_ms_alone": gemm_alone, "gemm_ms_beside_direct_swap_out": gemm_direct,
+                  "gemm_ms_beside_staged_swap_out": gemm_staged,
+                  "gemm_slowdown_pct_direct": 100 * (gemm_direct / gemm_alone - 1),
+                  "gemm_slowdown_pct_staged": 100 * (gemm_staged / gemm_alone - 1)}
+        log("staged swap, verified: out %.2f GB/s, in %.2f GB/s, both on two streams %.2f GB/s summed; a bf16 8192^3 GEMM on another stream takes %.3f ms "
+            "alone, %.3f ms (%+.0f %%) beside the direct swap-out, %.3f ms (%+.0f %%) beside the staged one" %
+            (staged["swap_out_GBps"], staged["swap_in_GBps"], staged_duplex_gbps, gemm_alone, gemm_direct,
+             staged["gemm_slowdown_pct_direct"], gemm_staged, staged["gemm_slowdown_pct_staged"]))
 
     # ---- plain device copy of known size: yardstick for reachable HBM bandwidth, and the
     # calibration row for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters -----------------
@@ -413,7 +516,8 @@ def main():
         "config": {"workload": cfg.name, "planes": planes, "layers": cfg.layers, "block_bytes": bb,
                    "blocks_per_launch": n, "device_blocks": cfg.dev_blocks, "host_blocks": cfg.host_blocks,
                    "host_blocks_specified": CONFIG_HOST_BLOCKS,
-                   "payload_bytes_per_step": payload, "cache_dtype": str(cfg.dtype).replace("torch.", "")},
+                   "payload_bytes_per_step": payload, "cache_dtype": str(cfg.dtype).replace("torch.", ""),
+                   "tuning_overrides": tuned},
         # Dominant kernel of the step. A swap never touches HBM twice; the resource it saturates is the
         # PCIe Gen5 x16 link, so that is the roofline it is priced against (theoretical link rate as
         # `peak`, the rate one large pinned hipMemcpyAsync reaches in this run as `peak_measured`).
@@ -443,6 +547,7 @@ def main():
         "pcie_peak_measured": {"d2h_GBps": d2h_peak, "h2d_GBps": h2d_peak, "theoretical_GBps": PCIE5_X16_GBPS,
                                "how": "mean of 5 back-to-back hipMemcpyAsync of %d MiB pinned" % (big >> 20)},
         "duplex": duplex,
+        "staged": staged,
         "memcpy_block_loop": memcpy_loop,
         "cpu_baseline": cpu_baseline,
         "verified": "bit-exact on every plane: " + ", ".join(sorted(sections)),

@@ -34,6 +34,7 @@ ENTRY_POINTS = (
     "hfk_multi_layer_block_table_transfer",
     "hfk_swap_blocks",
     "hfk_swap_blocks_duplex",
+    "hfk_swap_blocks_staged",
     "hfk_gather_blocks",
     "hfk_set_tuning",
     "hfk_get_tuning",
@@ -73,6 +74,8 @@ def load():
     L.hfk_swap_blocks.restype = ci
     L.hfk_swap_blocks_duplex.argtypes = [ctypes.POINTER(BlockMove), ctypes.POINTER(BlockMove), u32, u64, u32, vp]
     L.hfk_swap_blocks_duplex.restype = ci
+    L.hfk_swap_blocks_staged.argtypes = [vp, vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, vp, ci, u32, vp]
+    L.hfk_swap_blocks_staged.restype = ci
     L.hfk_gather_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u32, vp]
     L.hfk_gather_blocks.restype = ci
     L.hfk_set_tuning.argtypes = [ci, i64]
@@ -127,6 +130,14 @@ def swap_blocks_duplex(out_move, in_move, n_planes, block_bytes, workgroups=0, s
     return load().hfk_swap_blocks_duplex(ctypes.byref(out_move) if out_move is not None else None,
                                          ctypes.byref(in_move) if in_move is not None else None, n_planes, block_bytes,
                                          workgroups, stream)
+
+
+def swap_blocks_staged(dev_planes, host_plane_addrs, dev_ids, host_ids, n_planes, n_blocks, block_bytes, dev_stride,
+                       host_stride, dev_blocks, host_blocks, staging, to_host, workgroups=0, stream=0):
+    """host_plane_addrs / host_ids: addresses of HOST arrays (e.g. numpy .ctypes.data)."""
+    return load().hfk_swap_blocks_staged(dev_planes, host_plane_addrs, dev_ids, host_ids, n_planes, n_blocks,
+                                         block_bytes, dev_stride, host_stride, dev_blocks, host_blocks, staging,
+                                         int(bool(to_host)), workgroups, stream)
 
 
 def gather_blocks(dst_planes, src_planes, ids, n_planes, n_ids, block_bytes, src_stride, src_blocks=0,

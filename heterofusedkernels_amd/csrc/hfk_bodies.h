@@ -83,11 +83,13 @@ HFK_HD uint8_t unit_byte(vec16 v, uint32_t k) {
 // ---------------------------------------------------------------------------
 template <typename IdT>
 struct BlockCopyArgs {
-    const uint64_t* dst_planes;  // device array of plane base addresses, or null -> dst_base
-    const uint64_t* src_planes;  // device array of plane base addresses, or null -> src_base
+    const uint64_t* dst_planes;  // device array of plane base addresses, or null ->
+    const uint64_t* src_planes;  //   plane p starts at {dst,src}_base + p * {dst,src}_plane_stride
     uint64_t dst_base;
     uint64_t src_base;
-    const IdT* src_ids;          // entry j at src_ids[j * id_stride]
+    uint64_t dst_plane_stride;
+    uint64_t src_plane_stride;
+    const IdT* src_ids;          // entry j at src_ids[j * id_stride]; null -> src block j
     const IdT* dst_ids;          // entry j at dst_ids[j * id_stride]; null -> dst block j
     uint32_t id_stride;
     uint32_t n_planes;
@@ -111,13 +113,15 @@ HFK_HD bool resolve_chunk(const BlockCopyArgs<IdT>& a, uint32_t w, uint64_t& s_a
     const uint32_t tile = w / a.chunks_per_block;
     const uint32_t pair = tile % a.n_pairs;
     const uint32_t plane = tile / a.n_pairs;
-    const uint64_t sb = (uint64_t)(int64_t)a.src_ids[(uint64_t)pair * a.id_stride];
+    const uint64_t sb = a.src_ids ? (uint64_t)(int64_t)a.src_ids[(uint64_t)pair * a.id_stride] : (uint64_t)pair;
     const uint64_t db = a.dst_ids ? (uint64_t)(int64_t)a.dst_ids[(uint64_t)pair * a.id_stride] : (uint64_t)pair;
     if (sb >= a.src_limit || db >= a.dst_limit) {
         return false;
     }
-    s_addr = (a.src_planes ? a.src_planes[plane] : a.src_base) + sb * a.src_stride;
-    d_addr = (a.dst_planes ? a.dst_planes[plane] : a.dst_base) + db * a.dst_stride;
+    s_addr = (a.src_planes ? a.src_planes[plane] : a.src_base + (uint64_t)plane * a.src_plane_stride) +
+             sb * a.src_stride;
+    d_addr = (a.dst_planes ? a.dst_planes[plane] : a.dst_base + (uint64_t)plane * a.dst_plane_stride) +
+             db * a.dst_stride;
     return true;
 }
 

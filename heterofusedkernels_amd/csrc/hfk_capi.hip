@@ -28,7 +28,7 @@ using hfk::vec16;
 
 // One body, three kernel names: the block-copy body serves the swap, the multi-plane
 // block gather and wide-row gathers, and a profile should say which one ran.
-enum class Role { kSwapBlocks, kGatherBlocks, kGatherRows };
+enum class Role { kSwapBlocks, kGatherBlocks, kGatherRows, kScatterBlocks };
 
 template <int UNROLL, int NT>
 __global__ __launch_bounds__(256) void swap_blocks_kernel(const BlockCopyArgs<int64_t> a) {
@@ -37,6 +37,11 @@ __global__ __launch_bounds__(256) void swap_blocks_kernel(const BlockCopyArgs<in
 
 template <int UNROLL, int NT>
 __global__ __launch_bounds__(256) void gather_blocks_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void scatter_blocks_kernel(const BlockCopyArgs<int64_t> a) {
     hfk::block_copy_body<int64_t, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
@@ -132,6 +137,8 @@ void launch_block_copy_one(const BlockCopyArgs<IdT>& a, uint32_t grid, hipStream
         hipLaunchKernelGGL((swap_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
     } else if constexpr (ROLE == Role::kGatherBlocks) {
         hipLaunchKernelGGL((gather_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
+    } else if constexpr (ROLE == Role::kScatterBlocks) {
+        hipLaunchKernelGGL((scatter_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
     } else {
         hipLaunchKernelGGL((gather_rows_wide_kernel<IdT, UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
     }
@@ -364,6 +371,66 @@ int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move*
         default: launch_duplex_nt<16>(a, grid, nt, s); break;
     }
     return finish_launch();
+}
+
+int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host_plane_addrs, const int64_t* dev_block_ids,
+                           const int64_t* host_block_ids, uint32_t n_planes, uint64_t n_blocks, uint64_t block_bytes,
+                           uint64_t dev_block_stride, uint64_t host_block_stride, uint64_t dev_blocks,
+                           uint64_t host_blocks, void* staging, int to_host, uint32_t workgroups,
+                           hfk_stream_t stream) {
+    if (n_planes == 0 || n_blocks == 0) return HFK_OK;
+    if (host_plane_addrs == nullptr || host_block_ids == nullptr) return HFK_ERR_NULL_POINTER;
+    if (host_block_stride < block_bytes) return HFK_ERR_BAD_SIZE;
+    BlockCopyArgs<int64_t> a;
+    int rc = hfk::plan_stage_blocks(a, dev_plane_ptrs, staging, dev_block_ids, n_planes, n_blocks, block_bytes,
+                                    dev_block_stride, dev_blocks, to_host != 0);
+    if (rc != 0) return rc;
+    for (uint32_t p = 0; p < n_planes; ++p) {
+        if (host_plane_addrs[p] == nullptr) return HFK_ERR_NULL_POINTER;
+    }
+    for (uint64_t i = 0; i < n_blocks; ++i) {  // nothing is enqueued unless every host slot is valid
+        if (host_block_ids[i] < 0 || (host_blocks != 0 && (uint64_t)host_block_ids[i] >= host_blocks)) {
+            return HFK_ERR_BAD_SIZE;
+        }
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // One copy per plane and per run of consecutive host slots; with a contiguous block stride on
+    // the host side a run of k slots is one copy of k * block_bytes, otherwise k strided copies
+    // collapse into one 2-D copy.
+    auto copy_runs = [&]() -> int {
+        for (uint32_t p = 0; p < n_planes; ++p) {
+            char* host_plane = static_cast<char*>(host_plane_addrs[p]);
+            char* stage_plane = static_cast<char*>(staging) + (uint64_t)p * n_blocks * block_bytes;
+            uint64_t first = 0;
+            while (first < n_blocks) {
+                uint64_t len = 1;
+                while (first + len < n_blocks && host_block_ids[first + len] == host_block_ids[first] + (int64_t)len) ++len;
+                char* h = host_plane + (uint64_t)host_block_ids[first] * host_block_stride;
+                char* d = stage_plane + first * block_bytes;
+                hipError_t e;
+                if (host_block_stride == block_bytes) {
+                    e = to_host ? hipMemcpyAsync(h, d, len * block_bytes, hipMemcpyDeviceToHost, s)
+                                : hipMemcpyAsync(d, h, len * block_bytes, hipMemcpyHostToDevice, s);
+                } else {
+                    e = to_host ? hipMemcpy2DAsync(h, host_block_stride, d, block_bytes, block_bytes, len,
+                                                   hipMemcpyDeviceToHost, s)
+                                : hipMemcpy2DAsync(d, block_bytes, h, host_block_stride, block_bytes, len,
+                                                   hipMemcpyHostToDevice, s);
+                }
+                if (e != hipSuccess) return (int)e;
+                first += len;
+            }
+        }
+        return HFK_OK;
+    };
+    if (to_host) {
+        rc = launch_block_copy<Role::kGatherBlocks, int64_t>(a, workgroups, s);
+        if (rc != 0) return rc;
+        return copy_runs();
+    }
+    rc = copy_runs();
+    if (rc != 0) return rc;
+    return launch_block_copy<Role::kScatterBlocks, int64_t>(a, workgroups, s);
 }
 
 int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* ids,

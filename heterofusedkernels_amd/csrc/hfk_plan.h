@@ -188,6 +188,43 @@ inline int plan_gather_blocks(BlockCopyArgs<int64_t>& a, const void* dst_plane_p
     return HFK_OK;
 }
 
+// The kernel half of a staged swap: blocks between the device planes and a
+// contiguous staging buffer [n_planes][n_blocks][block_bytes] in device memory.
+// to_staging: staging[p][i] = plane_p[ids[i]]  (gather);  else  plane_p[ids[i]] = staging[p][i]  (scatter).
+inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_ptrs, void* staging,
+                             const int64_t* dev_block_ids, uint32_t n_planes, uint64_t n_blocks, uint64_t block_bytes,
+                             uint64_t dev_block_stride, uint64_t dev_blocks, bool to_staging) {
+    if (dev_plane_ptrs == nullptr || staging == nullptr || dev_block_ids == nullptr) return HFK_ERR_NULL_POINTER;
+    if (block_bytes == 0 || dev_block_stride < block_bytes) return HFK_ERR_BAD_SIZE;
+    if (n_blocks > kU32Max) return HFK_ERR_TOO_LARGE;
+    a = BlockCopyArgs<int64_t>{};
+    a.id_stride = 1;
+    a.n_planes = n_planes;
+    a.n_pairs = (uint32_t)n_blocks;
+    a.block_bytes = block_bytes;
+    const uint64_t limit = dev_blocks ? dev_blocks : kUnchecked;
+    if (to_staging) {
+        a.src_planes = static_cast<const uint64_t*>(dev_plane_ptrs);
+        a.src_ids = dev_block_ids;
+        a.src_stride = dev_block_stride;
+        a.src_limit = limit;
+        a.dst_base = (uint64_t)(uintptr_t)staging;
+        a.dst_plane_stride = n_blocks * block_bytes;
+        a.dst_stride = block_bytes;
+        a.dst_limit = kUnchecked;
+    } else {
+        a.dst_planes = static_cast<const uint64_t*>(dev_plane_ptrs);
+        a.dst_ids = dev_block_ids;
+        a.dst_stride = dev_block_stride;
+        a.dst_limit = limit;
+        a.src_base = (uint64_t)(uintptr_t)staging;
+        a.src_plane_stride = n_blocks * block_bytes;
+        a.src_stride = block_bytes;
+        a.src_limit = kUnchecked;
+    }
+    return HFK_OK;
+}
+
 // Wide-row gather expressed as a single-plane block copy with dst block i = i.
 template <typename IdT>
 inline int plan_wide_gather(BlockCopyArgs<IdT>& a, const void* table, void* dst, const IdT* ids, uint64_t n_ids,

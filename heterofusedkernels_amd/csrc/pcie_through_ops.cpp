@@ -3,8 +3,8 @@
 // Schemas of the first three ops are those of the reference
 // (pcieThrough/csrc/host/gather_torch.cpp:60,
 //  pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:113-114);
-// multi_layer_block_table_transfer, swap_blocks, swap_blocks_duplex, gather_blocks and
-// gather_into are additive. Every op unpacks its tensors into
+// multi_layer_block_table_transfer, swap_blocks, swap_blocks_duplex, swap_blocks_staged,
+// gather_blocks and gather_into are additive. Every op unpacks its tensors into
 // raw device-visible addresses, takes the current HIP stream of the device that
 // owns the device-side tensor, and calls the C-ABI of libhfk_hip.so; nothing is
 // allocated and nothing waits.
@@ -280,6 +280,48 @@ void swap_blocks_duplex(const at::Tensor& devicePlanePtrs, const at::Tensor& hos
                  "hfk_swap_blocks_duplex");
 }
 
+// Staged block-table swap: one gather/scatter kernel on HBM plus DMA copies, so no
+// compute unit touches host memory; see hfk_swap_blocks_staged. hostPlaneAddrs and
+// hostBlockIds are CPU int64 tensors (host addresses of the pinned planes, host slots);
+// deviceBlockIds lives on the device. Block-table form of the reference's staged
+// variant (multi_layer_block_transfer_torch.cpp:82-106).
+void swap_blocks_staged(const at::Tensor& devicePlanePtrs, const at::Tensor& hostPlaneAddrs,
+                        const at::Tensor& deviceBlockIds, const at::Tensor& hostBlockIds, const at::Tensor& staging,
+                        int64_t blockBytes, int64_t deviceBlockStride, int64_t hostBlockStride, bool toHost,
+                        int64_t deviceBlocks, int64_t hostBlocks, std::optional<int64_t> workgroups) {
+    check_ptr_table(devicePlanePtrs, "devicePlanePtrs");
+    check_ptr_table(hostPlaneAddrs, "hostPlaneAddrs");
+    check_ptr_table(deviceBlockIds, "deviceBlockIds");
+    check_ptr_table(hostBlockIds, "hostBlockIds");
+    TORCH_CHECK(devicePlanePtrs.is_cuda(), "devicePlanePtrs must be a device tensor");
+    TORCH_CHECK(hostPlaneAddrs.device().is_cpu() && hostBlockIds.device().is_cpu(),
+                "hostPlaneAddrs and hostBlockIds must be CPU tensors");
+    TORCH_CHECK(staging.is_cuda() && staging.is_contiguous(), "staging must be a contiguous device tensor");
+    TORCH_CHECK(devicePlanePtrs.numel() == hostPlaneAddrs.numel(), "plane tables differ in length");
+    TORCH_CHECK(devicePlanePtrs.numel() <= 0xffffffffLL, "too many planes");
+    TORCH_CHECK(deviceBlockIds.dim() == 1 && hostBlockIds.dim() == 1 && deviceBlockIds.numel() == hostBlockIds.numel(),
+                "deviceBlockIds and hostBlockIds must be 1-dimensional and equally long");
+    TORCH_CHECK(blockBytes > 0 && deviceBlockStride >= blockBytes && hostBlockStride >= blockBytes,
+                "swap_blocks_staged: strides must be at least blockBytes, blockBytes positive");
+    TORCH_CHECK(deviceBlocks >= 0 && hostBlocks >= 0, "swap_blocks_staged: block counts must be non-negative");
+    const uint64_t planes = static_cast<uint64_t>(devicePlanePtrs.numel());
+    const uint64_t n = static_cast<uint64_t>(deviceBlockIds.numel());
+    TORCH_CHECK(static_cast<uint64_t>(staging.nbytes()) >= planes * n * static_cast<uint64_t>(blockBytes),
+                "staging holds ", staging.nbytes(), " bytes, ", planes * n * static_cast<uint64_t>(blockBytes),
+                " needed");
+    if (planes == 0 || n == 0) return;
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(devicePlanePtrs));
+    check_status(hfk_swap_blocks_staged(devicePlanePtrs.data_ptr(),
+                                        reinterpret_cast<void* const*>(hostPlaneAddrs.data_ptr<int64_t>()),
+                                        static_cast<const int64_t*>(device_visible(deviceBlockIds, "deviceBlockIds")),
+                                        hostBlockIds.data_ptr<int64_t>(), static_cast<uint32_t>(planes), n,
+                                        static_cast<uint64_t>(blockBytes), static_cast<uint64_t>(deviceBlockStride),
+                                        static_cast<uint64_t>(hostBlockStride), static_cast<uint64_t>(deviceBlocks),
+                                        static_cast<uint64_t>(hostBlocks), staging.data_ptr(), toHost ? 1 : 0,
+                                        workgroup_cap(workgroups), current_stream()),
+                 "hfk_swap_blocks_staged");
+}
+
 // Shared-id block gather over planes; see hfk_gather_blocks.
 void gather_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs, const at::Tensor& blockIds,
                    int64_t blockBytes, int64_t srcBlockStride, int64_t srcBlocks,
@@ -326,6 +368,10 @@ TORCH_LIBRARY(pcie_through, m) {
         "blockBytes, int deviceBlockStride, int hostBlockStride, int deviceBlocks=0, int hostBlocks=0, int? "
         "workgroups=None) -> ()");
     m.def(
+        "swap_blocks_staged(Tensor devicePlanePtrs, Tensor hostPlaneAddrs, Tensor deviceBlockIds, Tensor hostBlockIds, "
+        "Tensor(a!) staging, int blockBytes, int deviceBlockStride, int hostBlockStride, bool toHost, int "
+        "deviceBlocks=0, int hostBlocks=0, int? workgroups=None) -> ()");
+    m.def(
         "gather_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockIds, int blockBytes, int "
         "srcBlockStride, int srcBlocks=0, int? workgroups=None) -> ()");
 }
@@ -341,5 +387,6 @@ TORCH_LIBRARY_IMPL(pcie_through, CUDA, m) {
     m.impl("multi_layer_block_table_transfer", TORCH_FN(pciethrough::multi_layer_block_table_transfer));
     m.impl("swap_blocks", TORCH_FN(pciethrough::swap_blocks));
     m.impl("swap_blocks_duplex", TORCH_FN(pciethrough::swap_blocks_duplex));
+    m.impl("swap_blocks_staged", TORCH_FN(pciethrough::swap_blocks_staged));
     m.impl("gather_blocks", TORCH_FN(pciethrough::gather_blocks));
 }

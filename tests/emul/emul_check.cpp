@@ -236,6 +236,49 @@ void case_duplex(uint32_t n_planes, uint32_t n_out, uint32_t n_in, uint64_t bloc
     for (auto* b : host_exp) delete b;
 }
 
+// ---- kernel half of the staged swap: planes <-> contiguous staging buffer ------
+void case_stage(uint32_t n_planes, uint32_t n_blocks, uint64_t block_bytes, uint32_t dev_blocks, uint64_t pad, bool to_staging,
+                int unroll, uint32_t grid_cap, bool with_bad) {
+    const uint64_t ds = block_bytes + pad;
+    std::vector<Buf*> dev, dev_exp;
+    std::vector<uint64_t> dp;
+    Buf staging((uint64_t)n_planes * n_blocks * block_bytes), staging_exp((uint64_t)n_planes * n_blocks * block_bytes);
+    staging.randomize();
+    std::memcpy(staging_exp.p, staging.p, staging.n);
+    for (uint32_t p = 0; p < n_planes; ++p) {
+        dev.push_back(new Buf(dev_blocks * ds - pad));
+        dev_exp.push_back(new Buf(dev_blocks * ds - pad));
+        dev.back()->randomize();
+        std::memcpy(dev_exp.back()->p, dev.back()->p, dev.back()->n);
+        dp.push_back((uint64_t)(uintptr_t)dev.back()->p);
+    }
+    std::vector<int64_t> perm(dev_blocks), ids(n_blocks);
+    for (uint32_t i = 0; i < dev_blocks; ++i) perm[i] = i;
+    std::shuffle(perm.begin(), perm.end(), rng);
+    for (uint32_t i = 0; i < n_blocks; ++i) {
+        ids[i] = perm[i % dev_blocks];
+        if (with_bad && i % 3 == 2) ids[i] = (i % 2) ? -1 : (int64_t)dev_blocks + 3;
+    }
+    BlockCopyArgs<int64_t> a;
+    int rc = plan_stage_blocks(a, dp.data(), staging.p, ids.data(), n_planes, n_blocks, block_bytes, ds, dev_blocks, to_staging);
+    if (rc != HFK_OK) { ++g_failures; std::printf("plan_stage_blocks rc=%d\n", rc); }
+    else run_block_copy<int64_t, 3>(a, unroll, grid_cap);
+    for (uint32_t p = 0; p < n_planes; ++p)
+        for (uint32_t i = 0; i < n_blocks; ++i) {
+            if (ids[i] < 0 || ids[i] >= (int64_t)dev_blocks) continue;
+            uint8_t* st = staging_exp.p + ((uint64_t)p * n_blocks + i) * block_bytes;
+            uint8_t* dv = dev_exp[p]->p + (uint64_t)ids[i] * ds;
+            if (to_staging) std::memcpy(st, dv, block_bytes); else std::memcpy(dv, st, block_bytes);
+        }
+    char what[160];
+    std::snprintf(what, sizeof what, "stage planes=%u blocks=%u bytes=%llu pad=%llu to_staging=%d unroll=%d grid=%u bad=%d", n_planes,
+                  n_blocks, (unsigned long long)block_bytes, (unsigned long long)pad, (int)to_staging, unroll, grid_cap, (int)with_bad);
+    expect_equal(staging.p, staging_exp.p, staging.n, what);
+    for (uint32_t p = 0; p < n_planes; ++p) expect_equal(dev[p]->p, dev_exp[p]->p, dev[p]->n, what);
+    for (auto* b : dev) delete b;
+    for (auto* b : dev_exp) delete b;
+}
+
 // ---- gather_blocks (multi-plane, shared ids) -------------------------------
 void case_gather_blocks(uint32_t n_planes, uint32_t n_ids, uint64_t block_bytes, uint64_t src_blocks, int unroll,
                         uint32_t grid_cap) {
@@ -475,6 +518,15 @@ int main() {
     case_duplex(2, 3, 4, 4099, 9, 9, 1, 4, 7, true);                   // byte path
     case_duplex(1, 3, 3, 48, 7, 7, 0, 4, 2, false);                    // blocks smaller than a chunk
     case_duplex(1, 0, 0, 4096, 4, 4, 0, 4, 2, false);                  // nothing at all
+
+    // staged swap, kernel half: gather into and scatter out of the staging buffer
+    for (bool to_staging : {true, false})
+        for (int unroll : {1, 4, 8, 16}) {
+            case_stage(3, 7, 32768, 12, 0, to_staging, unroll, 5, false);
+            case_stage(2, 5, 73728, 9, 0, to_staging, unroll, 1000, true);
+            case_stage(2, 6, 16384, 8, 64, to_staging, unroll, 3, true);
+            case_stage(1, 4, 4100, 6, 0, to_staging, unroll, 2, false);
+        }
 
     // block-table transfer, both directions
     for (bool to_packed : {false, true}) {

@@ -324,6 +324,59 @@ def test_duplex_swap_equals_two_swaps(memory, cfg, n_out, n_in):
         assert torch.equal(dev2[p], dev[p]), "plane %d" % p
 
 
+@pytest.mark.parametrize("cfg,n,pattern", [
+    (W.C2_LLAMA8B_SWAP_OUT.scaled(layers=3, dev_blocks=128, host_blocks=192), 48, "run"),
+    (W.C2_LLAMA8B_SWAP_OUT.scaled(layers=2, dev_blocks=128, host_blocks=192), 40, "runs"),
+    (W.C4_MLA_ROUNDTRIP.scaled(layers=3, dev_blocks=48, host_blocks=64), 17, "scattered"),
+    (W.C5_FP8_FRAGMENTED.scaled(layers=2, dev_blocks=256, host_blocks=256), 100, "runs"),
+])
+def test_staged_swap_equals_direct_swap(memory, cfg, n, pattern):
+    """Staged swap-out then staged swap-in (kernel on HBM + DMA copies) == index_select / index_copy_,
+    and the staging buffer holds the moved blocks (as the reference's staged op leaves its staging block)."""
+    announce("staged swap %s: %d blocks, host slots %s" % (cfg.name, n, pattern))
+    bb = cfg.block_bytes
+    cpu_dev = [W.as_bytes(p).clone() for p in _cpu_planes(cfg, cfg.dev_blocks)]
+    dev = [p.to(DEV) for p in cpu_dev]
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0x2B)
+    gen = torch.Generator().manual_seed(n)
+    dev_ids = torch.randperm(cfg.dev_blocks, generator=gen)[:n].contiguous()
+    if pattern == "run":
+        host_ids = torch.arange(5, 5 + n)
+    elif pattern == "runs":
+        host_ids = W.fragmented_ids(cfg.host_blocks, n, seed=n)
+    else:
+        host_ids = torch.randperm(cfg.host_blocks, generator=gen)[:n].contiguous()
+    dtab = ptr_table(dev)
+    host_addrs = torch.tensor([t.data_ptr() for t in host], dtype=torch.int64)          # host addresses, CPU tensor
+    staging = torch.zeros(cfg.planes, n, bb, dtype=torch.uint8, device=DEV)
+    torch.ops.pcie_through.swap_blocks_staged(dtab, host_addrs, dev_ids.to(DEV), host_ids, staging, bb, bb, bb, True,
+                                              cfg.dev_blocks, cfg.host_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.host_blocks, bb), 0x2B, dtype=torch.uint8)
+        O.torch_swap_blocks(want, cpu_dev[p], dev_ids, host_ids)
+        assert torch.equal(host[p], want), "plane %d host side" % p
+        assert torch.equal(staging[p].cpu(), cpu_dev[p][dev_ids]), "plane %d staging" % p
+        assert torch.equal(dev[p].cpu(), cpu_dev[p]), "plane %d source changed" % p
+    # back in, to other device blocks
+    back_ids = torch.roll(dev_ids, 3)
+    fresh = [torch.full((cfg.dev_blocks, bb), 0x4D, dtype=torch.uint8, device=DEV) for _ in range(cfg.planes)]
+    staging.zero_()
+    torch.ops.pcie_through.swap_blocks_staged(ptr_table(fresh), host_addrs, back_ids.to(DEV), host_ids, staging, bb, bb,
+                                              bb, False, cfg.dev_blocks, cfg.host_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.dev_blocks, bb), 0x4D, dtype=torch.uint8)
+        O.torch_swap_blocks(want, host[p], host_ids, back_ids)
+        assert torch.equal(fresh[p].cpu(), want), "plane %d device side" % p
+    # a host slot out of range rejects the call before anything is enqueued
+    bad = host_ids.clone()
+    bad[0] = cfg.host_blocks
+    with pytest.raises(RuntimeError, match="hfk_swap_blocks_staged"):
+        torch.ops.pcie_through.swap_blocks_staged(dtab, host_addrs, dev_ids.to(DEV), bad, staging, bb, bb, bb, True,
+                                                  cfg.dev_blocks, cfg.host_blocks)
+
+
 # ---------------------------------------------------------------------------
 # edge cases
 # ---------------------------------------------------------------------------
