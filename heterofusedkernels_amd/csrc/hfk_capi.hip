@@ -6,8 +6,11 @@
 // MI355X (256 CUs, 8 XCDs) both fills every XCD evenly -- workgroups are handed
 // to XCDs round-robin, and a work item's neighbours bid+-1 sit on other XCDs while
 // the item itself streams one contiguous span, so no XCD's L2 sees another's lines
-// -- and lets a caller shrink the footprint (the `workgroups` argument) when the
-// copy should overlap with compute.
+// -- and lets a caller bound the grid (the `workgroups` argument). PCIe-bound
+// launches default to a small grid: the link needs no more. A small grid does NOT
+// make a swap cheap for kernels running beside it, though: any kernel that touches
+// host memory slows its neighbours by 1.8-2.1x on MI355X whatever its size, which
+// is what hfk_swap_blocks_staged (HBM-only kernel + DMA copies) is for.
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
 //    workgroups lost 5-10 %), so the bound is set high enough to be inactive up to
 //    256 Ki chunks; beyond that the loop takes over.
 //  * PCIe-bound swaps peak at 32-128 workgroups (more only adds queueing on the
-//    link), so a swap defaults to 64 workgroups: a quarter of the CUs, one wave per SIMD.
+//    link), so a swap defaults to 64 workgroups.
 std::atomic<int> g_unroll{8};
 std::atomic<int> g_nontemporal{3};
 std::atomic<int> g_wg_per_cu{1024};
@@ -342,8 +345,8 @@ int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, cons
     int rc = hfk::plan_swap_blocks(a, dst_plane_ptrs, src_plane_ptrs, block_pairs, n_planes, n_pairs, block_bytes,
                                    src_block_stride, dst_block_stride, src_blocks, dst_blocks);
     if (rc != 0) return rc;
-    // A swap is bound by the PCIe link, which a fraction of the CUs saturates; a
-    // small grid leaves the rest of the chip to whatever runs beside the swap.
+    // A swap is bound by the PCIe link, which a fraction of the CUs saturates; more
+    // workgroups only queue on the link (1-3 % slower).
     if (workgroups == 0) workgroups = (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
     return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
 }
