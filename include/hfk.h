@@ -214,9 +214,11 @@ HFK_API int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_blo
  *                 host_plane_p[host_block_ids[i]] = staging[p][i]       (copies)
  *   to_host == 0: staging[p][i] = host_plane_p[host_block_ids[i]]      (copies)
  *                 dev_plane_p[dev_block_ids[i]] = staging[p][i]         (one scatter kernel)
- * all on `stream`, in that order. One copy is issued per plane and per run of
- * consecutive host_block_ids, so it is efficient when the host slots of a transfer are
- * (mostly) consecutive: 256 consecutive 32 KiB slots are one 8 MiB copy per plane.
+ * all on `stream`, in that order. One copy is issued per run of consecutive
+ * host_block_ids (a 2-D copy spanning all planes when the host planes are evenly
+ * spaced, else one copy per plane), so it is efficient when the host slots of a
+ * transfer are (mostly) consecutive: 256 consecutive 32 KiB slots of 64 planes are
+ * one 2-D copy of 64 rows of 8 MiB.
  * Result: identical to hfk_swap_blocks with the same table; staging holds the moved
  * blocks afterwards.
  *

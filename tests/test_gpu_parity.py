@@ -369,6 +369,19 @@ def test_staged_swap_equals_direct_swap(memory, cfg, n, pattern):
         want = torch.full((cfg.dev_blocks, bb), 0x4D, dtype=torch.uint8)
         O.torch_swap_blocks(want, host[p], host_ids, back_ids)
         assert torch.equal(fresh[p].cpu(), want), "plane %d device side" % p
+    # host planes that are NOT evenly spaced (reversed order) take the per-plane copy path: same bytes
+    for p in range(cfg.planes):
+        host[p].fill_(0x2B)
+    rev = list(reversed(range(cfg.planes)))
+    host_addrs_rev = torch.tensor([host[p].data_ptr() for p in rev], dtype=torch.int64)
+    dtab_rev = ptr_table([dev[p] for p in rev])
+    torch.ops.pcie_through.swap_blocks_staged(dtab_rev, host_addrs_rev, dev_ids.to(DEV), host_ids, staging, bb, bb, bb,
+                                              True, cfg.dev_blocks, cfg.host_blocks)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.host_blocks, bb), 0x2B, dtype=torch.uint8)
+        O.torch_swap_blocks(want, cpu_dev[p], dev_ids, host_ids)
+        assert torch.equal(host[p], want), "plane %d host side (per-plane copies)" % p
     # a host slot out of range rejects the call before anything is enqueued
     bad = host_ids.clone()
     bad[0] = cfg.host_blocks
