@@ -29,8 +29,9 @@ using hfk::TransposeArgs;
 using hfk::kWorkgroupLanes;
 using hfk::vec16;
 
-// One body, three kernel names: the block-copy body serves the swap, the multi-plane
-// block gather and wide-row gathers, and a profile should say which one ran.
+// One body, four kernel names: the block-copy body serves the swap, the multi-plane
+// block gather, the scatter out of a staging buffer and wide-row gathers, and a
+// profile should say which one ran.
 enum class Role { kSwapBlocks, kGatherBlocks, kGatherRows, kScatterBlocks };
 
 template <int UNROLL, int NT>
@@ -77,8 +78,8 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
 
 // ---- tuning state ---------------------------------------------------------
 // Defaults are the measured best on MI355X:
-//  * 8 x 16 B in flight per lane and non-temporal loads + stores: +15 % HBM copy
-//    bandwidth over plain accesses (the data is touched once, keep it out of L2).
+//  * 8 x 16 B in flight per lane and non-temporal loads + stores: +15-20 % HBM copy
+//    bandwidth over plain accesses (5.1 -> 6.1 TB/s; the data is touched once).
 //  * HBM-bound launches want one workgroup per chunk (a grid-stride loop over fewer
 //    workgroups lost 5-10 %), so the bound is set high enough to be inactive up to
 //    256 Ki chunks; beyond that the loop takes over.
@@ -281,6 +282,7 @@ const char* hfk_status_string(int status) {
         case HFK_ERR_BAD_SIZE: return "hfk: size or stride is zero or inconsistent";
         case HFK_ERR_TOO_LARGE: return "hfk: count exceeds what one launch can index";
         case HFK_ERR_BAD_KNOB: return "hfk: unknown tuning knob or value out of range";
+        case HFK_ERR_OUT_OF_RANGE: return "hfk: host-side index outside the declared range";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -393,7 +395,7 @@ int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host_plane_a
     }
     for (uint64_t i = 0; i < n_blocks; ++i) {  // nothing is enqueued unless every host slot is valid
         if (host_block_ids[i] < 0 || (host_blocks != 0 && (uint64_t)host_block_ids[i] >= host_blocks)) {
-            return HFK_ERR_BAD_SIZE;
+            return HFK_ERR_OUT_OF_RANGE;
         }
     }
     hipStream_t s = static_cast<hipStream_t>(stream);

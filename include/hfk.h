@@ -39,7 +39,8 @@ enum hfk_status {
     HFK_ERR_NULL_POINTER = -1, /* a required pointer argument is NULL            */
     HFK_ERR_BAD_SIZE = -2,     /* a size/stride is zero or inconsistent          */
     HFK_ERR_TOO_LARGE = -3,    /* a count exceeds what one launch can index      */
-    HFK_ERR_BAD_KNOB = -4      /* unknown tuning knob or value out of range      */
+    HFK_ERR_BAD_KNOB = -4,     /* unknown tuning knob or value out of range      */
+    HFK_ERR_OUT_OF_RANGE = -5  /* an index passed in host memory is out of range */
 };
 
 /* HFK_VERSION_MAJOR * 1000 + HFK_VERSION_MINOR of the loaded library. */
@@ -237,8 +238,13 @@ HFK_API int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_blo
  *   dev_block_ids     device-visible int64[n_blocks]
  *   host_block_ids    HOST int64[n_blocks] (read before the call returns)
  *   staging           device buffer of n_planes * n_blocks * block_bytes bytes
- *   dev_blocks / host_blocks  blocks per plane; 0 = unchecked. A device id out of range
- *                     is skipped by the kernel; a host id out of range rejects the call.
+ *   dev_blocks / host_blocks  blocks per plane; 0 = unchecked. A host id out of range
+ *                     rejects the call (HFK_ERR_OUT_OF_RANGE) before anything is enqueued.
+ *                     A device id out of range is skipped by the kernel as everywhere
+ *                     else; since the ids live on the device the copies cannot skip it
+ *                     too, so on the way out its host slot receives whatever
+ *                     staging[p][i] held before the call. Validate device ids upstream
+ *                     if that matters.
  */
 HFK_API int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host_plane_addrs,
                                    const int64_t* dev_block_ids, const int64_t* host_block_ids,

@@ -70,6 +70,21 @@ def test_argument_errors_are_reported_before_any_gpu_work():
     assert capi.multi_layer_block_transfer(8, 8, 0, 4, 4, 4, 2) == 0   # empty block
     assert capi.multi_layer_block_transfer(8, 8, 1 << 20, 1 << 10, 8, 128, 2) == -3
     assert capi.fused_memcpy_multi_layer_block_transfer(8, 8, 0, 4, 4, 4, 4, 2) == -1
+    # staged swap: host-side arrays are validated on the host before anything is enqueued
+    import numpy as np
+    planes = np.array([4096, 8192], dtype=np.uint64)
+    ids = np.array([0, 1, 9], dtype=np.int64)
+    args = (8, planes.ctypes.data, 8, ids.ctypes.data, 2, 3, 64, 64, 64, 0, 8, 8, True)
+    assert capi.swap_blocks_staged(*args) == -5                        # host id 9 >= 8 host blocks
+    assert capi.swap_blocks_staged(8, 0, 8, ids.ctypes.data, 2, 3, 64, 64, 64, 0, 8, 8, True) == -1
+    assert capi.swap_blocks_staged(8, planes.ctypes.data, 8, ids.ctypes.data, 2, 3, 64, 64, 32, 0, 0, 8, True) == -2
+    assert capi.swap_blocks_staged(8, planes.ctypes.data, 8, ids.ctypes.data, 2, 0, 64, 64, 64, 0, 0, 8, True) == 0
+    assert capi.swap_blocks_duplex(None, None, 4, 4096) == 0           # both sides empty
+    assert capi.swap_blocks_duplex(None, None, 4, 0) == -2
+    bad = capi.BlockMove(8, 8, None, 3, 4096, 4096, 0, 0)              # pairs missing
+    assert capi.swap_blocks_duplex(bad, None, 4, 4096) == -1
+    assert capi.multi_layer_block_table_transfer(8, 64, 8, 64, 0, 3, 0, 0, 2, 2, 2, 8, 1, False) == -1
+    assert capi.multi_layer_block_table_transfer(8, 8, 8, 64, 8, 3, 0, 0, 2, 2, 2, 8, 1, False) == -2   # stride < block
 
 
 # ---- torch ops: schemas are the reference's ---------------------------------
