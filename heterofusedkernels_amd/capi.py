@@ -42,6 +42,19 @@ ENTRY_POINTS = (
 
 
 def library_path():
+    """In-tree build output, or the copy installed next to libpcie_through.so."""
+    if os.path.exists(_build.HFK_HIP_SO):
+        return _build.HFK_HIP_SO
+    try:
+        import importlib.util
+
+        spec = importlib.util.find_spec("pcie_through")
+        if spec is not None and spec.submodule_search_locations:
+            installed = os.path.join(list(spec.submodule_search_locations)[0], "lib", "libhfk_hip.so")
+            if os.path.exists(installed):
+                return installed
+    except (ImportError, ValueError):
+        pass
     return _build.HFK_HIP_SO
 
 
