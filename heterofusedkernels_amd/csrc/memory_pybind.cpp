@@ -12,6 +12,16 @@
 
 namespace {
 
+// torch answers Tensor::is_pinned() through its device hooks, which report "not pinned"
+// until torch itself has initialised the device; a tensor handed out here must say it is pinned.
+// Without a usable GPU the initialisation throws; the callers' own checks then report the problem.
+void ensure_torch_device_ready() {
+    try {
+        at::globalContext().lazyInitDevice(c10::DeviceType::CUDA);
+    } catch (const c10::Error&) {
+    }
+}
+
 int current_hip_device() {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -24,6 +34,7 @@ int current_hip_device() {
 // Mirrors common/csrc/mem_alloc.cpp:17-64.
 torch::Tensor alloc_numa_pinned_tensor(std::size_t size) {
     TORCH_CHECK(size > 0, "alloc_numa_pinned_tensor: size must be positive");
+    ensure_torch_device_ready();
     const int dev = current_hip_device();
     int node = -1;
     int rc = hfk_mm_device_numa_node(dev, &node);
@@ -50,6 +61,7 @@ torch::Tensor alloc_numa_pinned_tensor(std::size_t size) {
 // Mirrors common/csrc/managed_memory/managed_mem.cpp:336-364 (`register_tensor`):
 // a tensor that is not on the CPU or not pinned is rejected with the same message.
 uintptr_t host_register(torch::Tensor& tensor) {
+    if (tensor.device().is_cpu()) ensure_torch_device_ready();
     if (!tensor.device().is_cpu() || !tensor.is_pinned()) {
         TORCH_CHECK(false, "Invalid device. Device must be CPU and tensor must be pinned.");
     }

@@ -47,6 +47,8 @@ void* device_visible(const at::Tensor& t, const char* what) {
     TORCH_CHECK(t.device().is_cpu(), what, ": unsupported device ", t.device());
     void* dev = HostRegisteredMemoryManager::GetInstance().getDevicePtr(t.data_ptr());
     if (dev != nullptr) return dev;
+    // (an op call always has a device tensor among its arguments, so torch's device hooks are up
+    // and is_pinned() answers truthfully)
     TORCH_CHECK(t.is_pinned(), what,
                 ": host tensor is neither registered with heterofusedkernels.memory nor pinned");
     const hipError_t e = hipHostGetDevicePointer(&dev, t.data_ptr(), 0);

@@ -141,3 +141,40 @@ def test_memory_module_on_gpu(memory):
         memory.host_register(torch.zeros(8))
     with pytest.raises(RuntimeError, match="must be pinned"):
         memory.host_register(torch.zeros(8, device="cuda"))
+
+
+def test_pinned_allocation_bound_to_an_explicit_numa_node():
+    """hfk_mm_alloc_pinned with a node number takes the MPOL_BIND + hipHostMallocNumaUser route (the boxes
+    report node -1 for the GPU, so alloc_numa_pinned_tensor alone never takes it)."""
+    import ctypes
+
+    from heterofusedkernels_amd import _build
+
+    announce("pinned allocation bound to NUMA node 0, then used by a kernel")
+    mm = ctypes.CDLL(_build.MANAGED_MEMORY_SO)
+    mm.hfk_mm_alloc_pinned.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_uint, ctypes.POINTER(ctypes.c_void_p)]
+    mm.hfk_mm_free_pinned.argtypes = [ctypes.c_void_p]
+    mm.hfk_mm_get_device_ptr.argtypes = [ctypes.c_void_p]
+    mm.hfk_mm_get_device_ptr.restype = ctypes.c_void_p
+    mm.hfk_mm_record_size.argtypes = [ctypes.c_void_p]
+    mm.hfk_mm_record_size.restype = ctypes.c_size_t
+    torch.cuda.init()
+    nbytes = 8 << 20
+    ptr = ctypes.c_void_p()
+    assert mm.hfk_mm_alloc_pinned(nbytes, 0, 0, ctypes.byref(ptr)) == 0 and ptr.value
+    dev_ptr = mm.hfk_mm_get_device_ptr(ptr.value)
+    assert dev_ptr and mm.hfk_mm_record_size(ptr.value + 100) == nbytes
+    host = (ctypes.c_uint8 * nbytes).from_address(ptr.value)
+    assert not any(host[i] for i in range(0, nbytes, 4099))                 # zero-filled
+    # a kernel writes it through the mapped address: gather 8 rows of 1 MiB from a device table into it
+    from heterofusedkernels_amd import capi
+    table = torch.randint(0, 256, (16, 1 << 20), dtype=torch.uint8, device="cuda")
+    ids = torch.tensor([3, 1, 4, 1, 5, 9, 2, 6], dtype=torch.int64, device="cuda")
+    capi.check(capi.gather_rows(table.data_ptr(), dev_ptr, ids.data_ptr(), True, 8, 1 << 20, 16, 0,
+                                torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    got = torch.frombuffer(host, dtype=torch.uint8).view(8, 1 << 20)
+    assert torch.equal(got, table.cpu()[ids.cpu()])
+    del got
+    assert mm.hfk_mm_free_pinned(ptr.value) == 0
+    assert mm.hfk_mm_get_device_ptr(ptr.value) is None
