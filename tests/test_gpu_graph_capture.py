@@ -79,3 +79,86 @@ def test_swap_and_gather_replay_in_a_hip_graph():
         run()
         torch.cuda.synchronize()
         check(src2, slot2, dst2, "eager %d" % replay)
+
+
+def test_duplex_staged_and_table_transfer_replay_in_a_hip_graph():
+    """The newer entry points record as well: the duplex swap (one kernel), the staged swap (kernel +
+    DMA copy nodes; its host slot list is read at capture time and therefore fixed for the graph) and the
+    block-table transfer in both directions."""
+    announce("HIP graph: duplex swap + staged swap + block-table transfer, replayed 3 times")
+    planes, blocks, bb, n = 4, 48, 32768, 10
+    dev = [torch.zeros(blocks, bb, dtype=torch.uint8, device=DEV) for _ in range(planes)]
+    pool = memory.alloc_numa_pinned_tensor(planes * blocks * bb)
+    host = list(pool.view(torch.uint8).view(planes, blocks, bb).unbind(0))
+    dtab, htab = pcie_through.plane_pointer_table(dev, DEV), pcie_through.plane_pointer_table(host, DEV)
+    host_addrs = torch.tensor([h.data_ptr() for h in host], dtype=torch.int64)
+    out_pairs = torch.zeros(n, 2, dtype=torch.int64, device=DEV)
+    in_pairs = torch.zeros(n, 2, dtype=torch.int64, device=DEV)
+    staged_ids = torch.zeros(n, dtype=torch.int64, device=DEV)
+    staged_slots = torch.arange(30, 30 + n)                               # fixed at capture
+    staging = torch.zeros(planes, n, bb, dtype=torch.uint8, device=DEV)
+    T, L, H, D = 32, 3, 2, 64
+    tpool = memory.alloc_numa_pinned_tensor(6 * T * L * H * D).view(6, T, L, H, D)
+    tback = memory.alloc_numa_pinned_tensor(6 * T * L * H * D).view(6, T, L, H, D)
+    caches = torch.zeros(L, 5, H, T, D, dtype=torch.int8, device=DEV)
+    lptrs = torch.tensor([caches[l].data_ptr() for l in range(L)], dtype=torch.int64).to(DEV)
+    tpairs = torch.zeros(4, 2, dtype=torch.int64, device=DEV)
+
+    def run():
+        torch.ops.pcie_through.swap_blocks_duplex(dtab, htab, out_pairs, in_pairs, bb, bb, bb, blocks, blocks)
+        torch.ops.pcie_through.swap_blocks_staged(dtab, host_addrs, staged_ids, staged_slots, staging, bb, bb, bb, True,
+                                                  blocks, blocks)
+        torch.ops.pcie_through.multi_layer_block_table_transfer(lptrs, tpool, tpairs, H * T * D, 5, False)
+        torch.ops.pcie_through.multi_layer_block_table_transfer(lptrs, tback, tpairs, H * T * D, 5, True)
+
+    def set_inputs(seed):
+        gen = torch.Generator().manual_seed(seed)
+        state = {}
+        for p in range(planes):
+            dev[p].copy_(torch.randint(0, 256, (blocks, bb), dtype=torch.uint8, generator=gen))
+            host[p].copy_(torch.randint(0, 256, (blocks, bb), dtype=torch.uint8, generator=gen))
+        state["dev"] = [d.cpu() for d in dev]
+        state["host"] = [h.clone() for h in host]
+        dperm = torch.randperm(30, generator=gen)                       # device blocks 0..29, host slots 0..29 for the duplex
+        hperm = torch.randperm(30, generator=gen)
+        state["out"] = torch.stack([dperm[:n], hperm[:n]], 1)
+        state["in"] = torch.stack([hperm[n:2 * n], dperm[n:2 * n]], 1)
+        state["staged"] = 30 + torch.randperm(blocks - 30, generator=gen)[:n]   # device blocks 30.. -> host slots 30..
+        out_pairs.copy_(state["out"])
+        in_pairs.copy_(state["in"])
+        staged_ids.copy_(state["staged"])
+        tpool.copy_(torch.randint(-128, 128, tuple(tpool.shape), dtype=torch.int8, generator=gen))
+        tback.zero_()
+        state["tpairs"] = torch.stack([torch.randperm(6, generator=gen)[:4], torch.randperm(5, generator=gen)[:4]], 1)
+        tpairs.copy_(state["tpairs"])
+        return state
+
+    def check(st, tag):
+        for p in range(planes):
+            h, d = host[p], dev[p].cpu()
+            assert torch.equal(h[st["out"][:, 1]], st["dev"][p][st["out"][:, 0]]), tag + " duplex out"
+            assert torch.equal(d[st["in"][:, 1]], st["host"][p][st["in"][:, 0]]), tag + " duplex in"
+            assert torch.equal(h[30:30 + n], st["dev"][p][st["staged"]]), tag + " staged"
+        for hb, _ in st["tpairs"].tolist():
+            assert torch.equal(tback[hb], tpool[hb]), tag + " table transfer round trip"
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        set_inputs(1)
+        run()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    for replay in range(3):
+        st = set_inputs(50 + replay)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        check(st, "replay %d" % replay)
+        st = set_inputs(50 + replay)
+        run()
+        torch.cuda.synchronize()
+        check(st, "eager %d" % replay)
