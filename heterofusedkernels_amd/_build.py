@@ -8,6 +8,7 @@ Artefacts (all in-tree, git-ignored):
     dropin/heterofusedkernels/libmanaged_memory.so   host-memory registry + allocator
     dropin/heterofusedkernels/memory*.so         Python module heterofusedkernels.memory
     dropin/heterofusedkernels/include/*.h        headers shipped for native users
+    bin/hfk_c_client                             plain-C99 client of the C-ABI (csrc/examples)
 
 Run as ``python -m heterofusedkernels_amd._build`` or through ``build_all()``.
 """
@@ -33,6 +34,7 @@ PCIE_THROUGH_SO = os.path.join(PCIE_LIB, "libpcie_through.so")
 HFK_BENCH_SO = os.path.join(PCIE_LIB, "libhfk_bench.so")
 MANAGED_MEMORY_SO = os.path.join(COMMON, "libmanaged_memory.so")
 MEMORY_EXT_SO = os.path.join(COMMON, "memory" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+C_CLIENT = os.path.join(PKG, "bin", "hfk_c_client")
 
 
 def _run(cmd, quiet_patterns=()):
@@ -127,6 +129,22 @@ def build_pcie_through():
     )
 
 
+def build_c_client():
+    """The C-ABI as a foreign runtime sees it: C99, the two public headers, the HIP runtime's C API."""
+    os.makedirs(os.path.dirname(C_CLIENT), exist_ok=True)
+    _run(
+        [
+            "gcc", "-std=c99", "-O2", "-Wall", "-Wextra", "-Werror", "-D__HIP_PLATFORM_AMD__=1",
+            "-I" + os.path.join(ROCM, "include"), "-I" + INCLUDE,
+            os.path.join(CSRC, "examples", "hfk_c_client.c"), "-o", C_CLIENT,
+            "-L" + PCIE_LIB, "-lhfk_hip", "-L" + COMMON, "-lmanaged_memory",
+            "-L" + os.path.join(ROCM, "lib"), "-lamdhip64",
+            "-Wl,-rpath,$ORIGIN/../dropin/pcie_through/lib", "-Wl,-rpath,$ORIGIN/../dropin/heterofusedkernels",
+            "-Wl,-rpath," + os.path.join(ROCM, "lib"),
+        ]
+    )
+
+
 def build_all():
     """Compile everything, every time it is called."""
     build_hfk_hip()
@@ -134,10 +152,11 @@ def build_all():
     build_managed_memory()
     build_memory_ext()
     build_pcie_through()
+    build_c_client()
 
 
 def artefacts():
-    return [HFK_HIP_SO, HFK_BENCH_SO, PCIE_THROUGH_SO, MANAGED_MEMORY_SO, MEMORY_EXT_SO]
+    return [HFK_HIP_SO, HFK_BENCH_SO, PCIE_THROUGH_SO, MANAGED_MEMORY_SO, MEMORY_EXT_SO, C_CLIENT]
 
 
 if __name__ == "__main__":

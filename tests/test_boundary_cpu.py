@@ -220,3 +220,23 @@ def test_memory_module_cpu_behaviour():
     assert memory.get_device_ptr(0x1234) == 0                    # managed_mem.cpp:372-375
     with pytest.raises(RuntimeError, match="Device must be CPU and tensor must be pinned"):
         memory.host_register(torch.zeros(16))                    # managed_mem.cpp:336-340
+
+
+def test_public_headers_are_strict_c99(tmp_path):
+    """A foreign runtime binds the headers from C: they must compile as C99 with -pedantic -Werror,
+    alone and in either order."""
+    src = tmp_path / "headers.c"
+    for order in (("hfk.h", "hfk_managed_memory.h"), ("hfk_managed_memory.h", "hfk.h")):
+        src.write_text("".join('#include "%s"\n' % h for h in order) + "int main(void) { return HFK_OK + HFK_MM_OK; }\n")
+        subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only",
+                        "-I" + _build.INCLUDE, str(src)], check=True)
+
+
+def test_c_client_fails_cleanly_without_a_gpu():
+    """The plain-C client links against the two libraries and, with no device, stops at its first HIP call
+    with a message and a non-zero status (no crash)."""
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present; the GPU test runs the client for real")
+    proc = subprocess.run([_build.C_CLIENT], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert proc.returncode == 2, (proc.returncode, proc.stdout, proc.stderr)
+    assert "hipSetDevice" in proc.stderr

@@ -471,3 +471,17 @@ def test_strided_planes():
     d, s = dst.cpu(), src.cpu()
     assert torch.equal(d[11, 1], s[0, 0]) and torch.equal(d[0, 1], s[9, 0]) and torch.equal(d[4, 1], s[4, 0])
     assert (d[:, 0] == 0).all() and d[:, 1].sum() == s[[0, 9, 4], 0].sum()
+
+
+@pytest.mark.parametrize("args", [(), ("3", "40", "4112", "20"), ("64", "128", "32768", "64")],
+                         ids=["defaults", "odd_block_size", "config2_planes"])
+def test_plain_c_client_runs_the_swap_path(args):
+    """The C-ABI bound from C99 with no torch in the process: swap-out, swap-in, staged swap and gather,
+    each checked byte for byte inside the client against the pattern it wrote."""
+    import subprocess
+    from heterofusedkernels_amd import _build
+
+    announce("plain-C client %s" % (" ".join(args) or "(defaults)"))
+    proc = subprocess.run([_build.C_CLIENT, *args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=100)
+    assert proc.returncode == 0, (proc.returncode, proc.stdout[-2000:], proc.stderr[-2000:])
+    assert proc.stdout.strip().endswith("hfk_c_client: OK")
