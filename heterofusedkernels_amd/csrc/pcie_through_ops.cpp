@@ -194,13 +194,17 @@ void multi_layer_block_table_transfer(const at::Tensor& deviceLayerCachePtrs, co
     TORCH_CHECK(deviceBlocks >= 0, "deviceBlocks must be non-negative");
     if (blockPairs.size(0) == 0 || blockBytes == 0) return;
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(deviceLayerCachePtrs));
+    // The library's default grid is sized for a pool in host memory (the PCIe link saturates with
+    // few workgroups). A pool in device memory - the staging buffer of a DMA-staged transfer - is
+    // HBM-bound and wants one workgroup per chunk.
+    uint32_t cap = workgroup_cap(workgroups);
+    if (cap == 0 && hostBlockPool.is_cuda()) cap = 0x7fffffffu;
     check_status(hfk_multi_layer_block_table_transfer(
                      deviceLayerCachePtrs.data_ptr(), static_cast<uint64_t>(deviceBlockStride),
                      device_visible(hostBlockPool, "hostBlockPool"), blockBytes,
                      static_cast<const int64_t*>(device_visible(blockPairs, "blockPairs")),
                      static_cast<uint64_t>(blockPairs.size(0)), static_cast<uint64_t>(hostBlockPool.size(0)),
-                     static_cast<uint64_t>(deviceBlocks), T, L, H, D, elem, toHost ? 1 : 0,
-                     workgroup_cap(workgroups), current_stream()),
+                     static_cast<uint64_t>(deviceBlocks), T, L, H, D, elem, toHost ? 1 : 0, cap, current_stream()),
                  "hfk_multi_layer_block_table_transfer");
 }
 

@@ -100,3 +100,41 @@ def test_block_table_transfer_skips_out_of_range_pairs():
     torch.cuda.synchronize()
     got = caches.cpu()
     assert (got[:, 1] == 3).all() and (got[:, 3] == 3).all() and (got[:, 0] == 0).all() and (got[:, 2] == 0).all()
+
+
+def test_block_table_transfer_staged_through_a_device_pool():
+    """The reference's staged idea (DMA copy into device staging, then a kernel that reads only HBM,
+    multi_layer_block_transfer_torch.cpp:82-106) over a block table, composed from existing pieces: one
+    hipMemcpyAsync per run of consecutive host blocks into a device pool, then the block-table transfer
+    with the pool as its packed side. Same result as the direct host-memory transfer."""
+    T, L, H, D, dtype = 128, 6, 4, 128, torch.bfloat16
+    e, host_blocks, dev_blocks = 2, 20, 11
+    announce("block-table transfer staged through a device pool, T=%d L=%d H=%d D=%d" % (T, L, H, D))
+    gen = torch.Generator().manual_seed(77)
+    pool = memory.alloc_numa_pinned_tensor(host_blocks * T * L * H * D * e)
+    pool.copy_(torch.randint(-128, 128, (pool.numel(),), dtype=torch.int8, generator=gen))
+    host_pool = pool.view(dtype).view(host_blocks, T, L, H, D)
+    runs = [(3, 4), (12, 5)]                                            # (first host block, count)
+    host_ids = torch.cat([torch.arange(a, a + c) for a, c in runs])
+    dev_ids = torch.randperm(dev_blocks, generator=gen)[:host_ids.numel()]
+    stride = H * T * D * e
+
+    def fresh():
+        caches = torch.zeros(L, dev_blocks, H, T, D, dtype=dtype, device=DEV)
+        return caches, torch.tensor([caches[l].data_ptr() for l in range(L)], dtype=torch.int64).to(DEV)
+
+    direct, dptrs = fresh()
+    torch.ops.pcie_through.multi_layer_block_table_transfer(dptrs, host_pool, torch.stack([host_ids, dev_ids], 1).to(DEV),
+                                                            stride, dev_blocks)
+    staged, sptrs = fresh()
+    staging = torch.empty(host_ids.numel(), T, L, H, D, dtype=dtype, device=DEV)
+    at = 0
+    for first, count in runs:
+        staging[at:at + count].copy_(host_pool[first:first + count], non_blocking=True)      # one DMA copy per run
+        at += count
+    torch.ops.pcie_through.multi_layer_block_table_transfer(
+        sptrs, staging, torch.stack([torch.arange(host_ids.numel()), dev_ids], 1).to(DEV), stride, dev_blocks)
+    torch.cuda.synchronize()
+    assert torch.equal(staged.view(torch.uint8), direct.view(torch.uint8))
+    want = torch.stack(O.torch_multi_layer_block_transfer(host_pool[host_ids[0]]))     # [L, H, T, D] of the first moved block
+    assert torch.equal(staged[:, dev_ids[0]].cpu().contiguous().view(torch.uint8), want.view(torch.uint8))
