@@ -1,0 +1,275 @@
+"""Seeded random sweep of every C-ABI entry point against the C oracle: odd block sizes,
+strides larger than a block, bases off every alignment, planes on either side of the PCIe
+link, int32 and int64 ids, out-of-range entries, random grid bounds. Each case checks the
+whole destination buffer, gaps between strided blocks included."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import heterofusedkernels_amd  # noqa: F401
+import pcie_through  # noqa: F401
+from heterofusedkernels import memory
+from heterofusedkernels_amd import capi
+from oracle import oracle as O
+
+from gpu_helpers import announce, stream_handle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+BLOCK_BYTES = [1, 3, 16, 48, 100, 528, 4096, 4112, 12288, 32768, 33001]
+PADS = [0, 0, 16, 5, 4096]
+OFFSETS = [0, 0, 16, 4, 1, 7]
+CASES = 40
+
+
+class Arena:
+    """A byte buffer on one side of the link, its numpy mirror and the address a kernel uses."""
+
+    def __init__(self, nbytes, on_host, rng, fill=None):
+        nbytes = max(int(nbytes), 1)
+        init = rng.integers(0, 256, nbytes, dtype=np.uint8) if fill is None else np.full(nbytes, fill, np.uint8)
+        self.on_host = on_host
+        if on_host:
+            self.t = memory.alloc_numa_pinned_tensor(nbytes).view(torch.uint8)
+            self.t.copy_(torch.from_numpy(init))
+            self.addr = memory.get_device_ptr(self.t.data_ptr())
+            self.host_addr = self.t.data_ptr()
+            assert self.addr != 0
+        else:
+            self.t = torch.from_numpy(init).to(DEV)
+            self.addr = self.t.data_ptr()
+        self.before = init
+
+    def now(self):
+        return self.t.cpu().numpy().copy()
+
+
+def _planes(base, offset, n_planes, blocks, stride):
+    """addresses of n_planes strided planes laid out back to back from base + offset"""
+    return [base + offset + p * blocks * stride for p in range(n_planes)]
+
+
+def _view(buf, offset, plane, blocks, stride, bb):
+    """[blocks, bb] strided numpy view of one plane inside a flat byte buffer"""
+    start = offset + plane * blocks * stride
+    return np.lib.stride_tricks.as_strided(buf[start:], shape=(blocks, bb), strides=(stride, 1), writeable=True)
+
+
+def _table(addresses):
+    return torch.tensor(addresses, dtype=torch.int64).to(DEV)
+
+
+def _pairs(rng, n, src_blocks, dst_blocks, with_bad):
+    """n (src, dst) pairs with distinct in-range destinations, plus out-of-range rows when asked"""
+    dst = rng.permutation(dst_blocks)[:n]
+    src = rng.integers(0, src_blocks, dst.shape[0])
+    pairs = np.stack([src, dst], 1).astype(np.int64).reshape(-1, 2)
+    if with_bad:
+        bad = np.array([[-1, 0], [src_blocks, 0], [0, dst_blocks], [0, -3], [2 ** 40, 0]], dtype=np.int64)
+        pairs = np.concatenate([pairs, bad[rng.integers(0, len(bad), 3)]])
+        pairs = pairs[rng.permutation(pairs.shape[0])]
+    ok = (pairs[:, 0] >= 0) & (pairs[:, 0] < src_blocks) & (pairs[:, 1] >= 0) & (pairs[:, 1] < dst_blocks)
+    return pairs, pairs[ok]
+
+
+def _expect_swap(dst_buf, src_buf, doff, soff, n_planes, dst_blocks, src_blocks, dstride, sstride, bb, valid):
+    want = dst_buf.copy()
+    for p in range(n_planes):
+        d = np.ascontiguousarray(_view(want, doff, p, dst_blocks, dstride, bb))
+        s = np.ascontiguousarray(_view(src_buf, soff, p, src_blocks, sstride, bb))
+        O.c_swap_blocks([d], [s], valid)
+        _view(want, doff, p, dst_blocks, dstride, bb)[:] = d
+    return want
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_swap_blocks(seed):
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(CASES):
+        n_planes = int(rng.integers(1, 9))
+        src_blocks, dst_blocks = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        bb = int(rng.choice(BLOCK_BYTES))
+        sstride, dstride = bb + int(rng.choice(PADS)), bb + int(rng.choice(PADS))
+        soff, doff = int(rng.choice(OFFSETS)), int(rng.choice(OFFSETS))
+        src_host, dst_host = [(False, False), (False, True), (True, False)][int(rng.integers(0, 3))]
+        n = int(rng.integers(0, dst_blocks + 1))
+        with_bad = bool(rng.integers(0, 2))
+        wg = int(rng.choice([0, 0, 1, 3, 1000]))
+        announce("random swap seed %d case %d: planes %d, blocks %d->%d, %d B (strides %d/%d, offsets %d/%d), "
+                 "src_host %s dst_host %s, %d pairs, bad %s, workgroups %d"
+                 % (seed, case, n_planes, src_blocks, dst_blocks, bb, sstride, dstride, soff, doff, src_host, dst_host,
+                    n, with_bad, wg))
+        src = Arena(soff + n_planes * src_blocks * sstride, src_host, rng)
+        dst = Arena(doff + n_planes * dst_blocks * dstride, dst_host, rng)
+        pairs, valid = _pairs(rng, n, src_blocks, dst_blocks, with_bad)
+        pairs_d = torch.from_numpy(pairs).to(DEV)
+        stab = _table(_planes(src.addr, soff, n_planes, src_blocks, sstride))
+        dtab = _table(_planes(dst.addr, doff, n_planes, dst_blocks, dstride))
+        capi.check(capi.swap_blocks(dtab.data_ptr(), stab.data_ptr(), pairs_d.data_ptr() if pairs.shape[0] else None,
+                                    n_planes, pairs.shape[0], bb, sstride, dstride, src_blocks, dst_blocks, wg,
+                                    stream_handle()), "hfk_swap_blocks")
+        torch.cuda.synchronize()
+        want = _expect_swap(dst.before, src.before, doff, soff, n_planes, dst_blocks, src_blocks, dstride, sstride, bb, valid)
+        assert np.array_equal(dst.now(), want)
+        assert np.array_equal(src.now(), src.before), "source changed"
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_gather_rows_and_blocks(seed):
+    rng = np.random.default_rng(2000 + seed)
+    for case in range(CASES):
+        rows = int(rng.integers(1, 200))
+        rb = int(rng.choice(BLOCK_BYTES + [7, 1000, 8212]))
+        toff, doff = int(rng.choice(OFFSETS)), int(rng.choice(OFFSETS))
+        table_host = bool(rng.integers(0, 2))
+        n = int(rng.integers(0, 300))
+        id_dtype = np.int64 if rng.integers(0, 2) else np.int32
+        with_bad = bool(rng.integers(0, 2))
+        wg = int(rng.choice([0, 0, 1, 5]))
+        announce("random gather_rows seed %d case %d: %d rows of %d B (offsets %d/%d), host table %s, %d ids %s, bad %s, "
+                 "workgroups %d" % (seed, case, rows, rb, toff, doff, table_host, n, id_dtype.__name__, with_bad, wg))
+        table = Arena(toff + rows * rb, table_host, rng)
+        dst = Arena(doff + n * rb, False, rng)
+        ids = rng.integers(0, rows, n).astype(id_dtype)
+        if with_bad and n:
+            ids[rng.integers(0, n, 3)] = np.array([-1, rows, rows + 5], dtype=id_dtype)
+        ids_d = torch.from_numpy(ids).to(DEV) if n else torch.zeros(1, dtype=torch.int64, device=DEV)
+        capi.check(capi.gather_rows(table.addr + toff, dst.addr + doff, ids_d.data_ptr(), id_dtype is np.int64, n, rb,
+                                    rows, wg, stream_handle()), "hfk_gather_rows")
+        torch.cuda.synchronize()
+        want = dst.before.copy()
+        ok = (ids >= 0) & (ids < rows)
+        got_rows = O.c_gather_rows(table.before[toff:toff + rows * rb].reshape(rows, rb), ids[ok])
+        want[doff:doff + n * rb].reshape(n, rb)[ok] = got_rows
+        assert np.array_equal(dst.now(), want)
+
+        # the same ids over several strided planes: hfk_gather_blocks
+        n_planes = int(rng.integers(1, 7))
+        stride = rb + int(rng.choice(PADS))
+        announce("random gather_blocks seed %d case %d: %d planes, stride %d" % (seed, case, n_planes, stride))
+        src = Arena(toff + n_planes * rows * stride, table_host, rng)
+        out = Arena(doff + n_planes * n * rb, False, rng)
+        ids64 = torch.from_numpy(ids.astype(np.int64)).to(DEV) if n else torch.zeros(1, dtype=torch.int64, device=DEV)
+        stab = _table(_planes(src.addr, toff, n_planes, rows, stride))
+        dtab = _table(_planes(out.addr, doff, n_planes, n, rb))
+        capi.check(capi.gather_blocks(dtab.data_ptr(), stab.data_ptr(), ids64.data_ptr(), n_planes, n, rb, stride, rows,
+                                      wg, stream_handle()), "hfk_gather_blocks")
+        torch.cuda.synchronize()
+        want = out.before.copy()
+        for p in range(n_planes):
+            plane = np.ascontiguousarray(_view(src.before, toff, p, rows, stride, rb))
+            start = doff + p * n * rb
+            want[start:start + n * rb].reshape(n, rb)[ok] = O.c_gather_rows(plane, ids[ok])
+        assert np.array_equal(out.now(), want)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_block_table_transfer(seed):
+    rng = np.random.default_rng(3000 + seed)
+    for case in range(CASES):
+        T, L, H = int(rng.integers(1, 40)), int(rng.integers(1, 6)), int(rng.integers(1, 5))
+        D, e = int(rng.choice([1, 3, 8, 16, 24, 64, 128])), int(rng.choice([1, 2, 4]))
+        packed_blocks, dev_blocks = int(rng.integers(1, 12)), int(rng.integers(1, 12))
+        to_packed = bool(rng.integers(0, 2))
+        packed_host = bool(rng.integers(0, 2))
+        poff = int(rng.choice(OFFSETS))
+        wg = int(rng.choice([0, 0, 1, 7]))
+        layer_bytes, block_bytes = H * T * D * e, T * L * H * D * e
+        n_dst = packed_blocks if to_packed else dev_blocks
+        n = int(rng.integers(0, n_dst + 1))
+        announce("random table transfer seed %d case %d: T%d L%d H%d D%d e%d, blocks %d/%d, to_packed %s, host pool %s, "
+                 "offset %d, %d pairs, workgroups %d"
+                 % (seed, case, T, L, H, D, e, packed_blocks, dev_blocks, to_packed, packed_host, poff, n, wg))
+        packed = Arena(poff + packed_blocks * block_bytes, packed_host, rng)
+        layers = Arena(L * dev_blocks * layer_bytes, False, rng)
+        if to_packed:      # pairs are (packed_block, dev_block); the destination side must be distinct
+            pb, db = rng.permutation(packed_blocks)[:n], rng.integers(0, dev_blocks, n)
+        else:
+            pb, db = rng.integers(0, packed_blocks, n), rng.permutation(dev_blocks)[:n]
+        pairs = np.stack([pb, db], 1).astype(np.int64).reshape(-1, 2)
+        bad = np.array([[-1, 0], [packed_blocks, 0], [0, dev_blocks]], dtype=np.int64)
+        pairs_all = np.concatenate([pairs, bad[rng.integers(0, 3, 2)]]) if rng.integers(0, 2) else pairs
+        pairs_d = torch.from_numpy(pairs_all).to(DEV) if pairs_all.shape[0] else None
+        lptrs = _table([layers.addr + l * dev_blocks * layer_bytes for l in range(L)])
+        capi.check(capi.multi_layer_block_table_transfer(
+            lptrs.data_ptr(), layer_bytes, packed.addr + poff, block_bytes, pairs_d.data_ptr() if pairs_d is not None else None,
+            pairs_all.shape[0], packed_blocks, dev_blocks, T, L, H, D, e, int(to_packed), wg, stream_handle()),
+            "hfk_multi_layer_block_table_transfer")
+        torch.cuda.synchronize()
+        want_layers = layers.before.copy().reshape(L, dev_blocks, layer_bytes)
+        want_packed = packed.before.copy()
+        pk = np.ascontiguousarray(want_packed[poff:poff + packed_blocks * block_bytes].reshape(packed_blocks, block_bytes))
+        O.c_multi_layer_block_table_transfer(want_layers, pk, pairs, T, L, H, D, e, to_packed)
+        want_packed[poff:poff + packed_blocks * block_bytes] = pk.reshape(-1)
+        assert np.array_equal(layers.now(), want_layers.reshape(-1))
+        assert np.array_equal(packed.now(), want_packed)
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_duplex_and_staged(seed):
+    rng = np.random.default_rng(4000 + seed)
+    for case in range(CASES):
+        n_planes = int(rng.integers(1, 7))
+        dev_blocks, host_blocks = int(rng.integers(4, 40)), int(rng.integers(4, 40))
+        bb = int(rng.choice(BLOCK_BYTES))
+        dstride, hstride = bb + int(rng.choice(PADS)), bb + int(rng.choice(PADS))
+        doff, hoff = int(rng.choice(OFFSETS)), int(rng.choice(OFFSETS))
+        wg = int(rng.choice([0, 0, 1, 3]))
+        most = min(dev_blocks, host_blocks) // 2
+        n_out, n_in = int(rng.integers(0, most + 1)), int(rng.integers(0, most + 1))
+        announce("random duplex seed %d case %d: %d planes, blocks %d/%d, %d B (strides %d/%d, offsets %d/%d), out %d in %d, "
+                 "workgroups %d" % (seed, case, n_planes, dev_blocks, host_blocks, bb, dstride, hstride, doff, hoff, n_out,
+                                    n_in, wg))
+        dev = Arena(doff + n_planes * dev_blocks * dstride, False, rng)
+        host = Arena(hoff + n_planes * host_blocks * hstride, True, rng)
+        dperm, hperm = rng.permutation(dev_blocks), rng.permutation(host_blocks)
+        out_pairs = np.stack([dperm[:n_out], hperm[:n_out]], 1).astype(np.int64).reshape(-1, 2)
+        in_pairs = np.stack([hperm[n_out:n_out + n_in], dperm[n_out:n_out + n_in]], 1).astype(np.int64).reshape(-1, 2)
+        po = torch.from_numpy(out_pairs).to(DEV) if n_out else None
+        pi = torch.from_numpy(in_pairs).to(DEV) if n_in else None
+        dtab = _table(_planes(dev.addr, doff, n_planes, dev_blocks, dstride))
+        htab = _table(_planes(host.addr, hoff, n_planes, host_blocks, hstride))
+        om = capi.BlockMove(htab.data_ptr(), dtab.data_ptr(), po.data_ptr() if n_out else None, n_out, dstride, hstride,
+                            dev_blocks, host_blocks)
+        im = capi.BlockMove(dtab.data_ptr(), htab.data_ptr(), pi.data_ptr() if n_in else None, n_in, hstride, dstride,
+                            host_blocks, dev_blocks)
+        capi.check(capi.swap_blocks_duplex(om, im, n_planes, bb, wg, stream_handle()), "hfk_swap_blocks_duplex")
+        torch.cuda.synchronize()
+        want_host = _expect_swap(host.before, dev.before, hoff, doff, n_planes, host_blocks, dev_blocks, hstride, dstride, bb,
+                                 out_pairs)
+        want_dev = _expect_swap(dev.before, host.before, doff, hoff, n_planes, dev_blocks, host_blocks, dstride, hstride, bb,
+                                in_pairs)
+        assert np.array_equal(host.now(), want_host), "host side"
+        assert np.array_equal(dev.now(), want_dev), "device side"
+
+        # staged, both directions, on fresh buffers of the same geometry
+        n = int(rng.integers(1, min(dev_blocks, host_blocks) + 1))
+        dev_ids = rng.permutation(dev_blocks)[:n].astype(np.int64)
+        first = int(rng.integers(0, host_blocks - n + 1))
+        host_ids = np.arange(first, first + n, dtype=np.int64)
+        if rng.integers(0, 2):
+            host_ids = rng.permutation(host_blocks)[:n].astype(np.int64)          # scattered slots
+        to_host = bool(rng.integers(0, 2))
+        announce("random staged seed %d case %d: %d blocks, to_host %s" % (seed, case, n, to_host))
+        dev2 = Arena(doff + n_planes * dev_blocks * dstride, False, rng)
+        host2 = Arena(hoff + n_planes * host_blocks * hstride, True, rng)
+        staging = torch.zeros(n_planes * n * bb, dtype=torch.uint8, device=DEV)
+        dtab2 = _table(_planes(dev2.addr, doff, n_planes, dev_blocks, dstride))
+        host_addrs = (ctypes.c_void_p * n_planes)(*_planes(host2.host_addr, hoff, n_planes, host_blocks, hstride))
+        ids_d = torch.from_numpy(dev_ids).to(DEV)
+        capi.check(capi.swap_blocks_staged(dtab2.data_ptr(), host_addrs, ids_d.data_ptr(), host_ids.ctypes.data, n_planes, n,
+                                           bb, dstride, hstride, dev_blocks, host_blocks, staging.data_ptr(), int(to_host),
+                                           wg, stream_handle()), "hfk_swap_blocks_staged")
+        torch.cuda.synchronize()
+        if to_host:
+            want = _expect_swap(host2.before, dev2.before, hoff, doff, n_planes, host_blocks, dev_blocks, hstride, dstride,
+                                bb, np.stack([dev_ids, host_ids], 1))
+            assert np.array_equal(host2.now(), want), "staged host side"
+            assert np.array_equal(dev2.now(), dev2.before)
+        else:
+            want = _expect_swap(dev2.before, host2.before, doff, hoff, n_planes, dev_blocks, host_blocks, dstride, hstride,
+                                bb, np.stack([host_ids, dev_ids], 1))
+            assert np.array_equal(dev2.now(), want), "staged device side"
+            assert np.array_equal(host2.now(), host2.before)
