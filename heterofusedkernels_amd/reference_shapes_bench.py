@@ -84,9 +84,12 @@ def gather_table(rows, runs, out):
               file=sys.stderr, flush=True)
 
 
-def transfer_table(out, blocks=8):
+README_TRANSFER_SHAPES = ((1024, 32, 1, 128), (1024, 32, 8, 128), (1024, 64, 1, 128), (1024, 64, 8, 128))
+
+
+def transfer_table(out, blocks=8, shapes=README_TRANSFER_SHAPES):
     dev = "cuda"
-    for (T, L, H, D) in ((1024, 32, 1, 128), (1024, 32, 8, 128), (1024, 64, 1, 128), (1024, 64, 8, 128)):
+    for (T, L, H, D) in shapes:
         nbytes = T * L * H * D
         pool = memory.alloc_numa_pinned_tensor(blocks * nbytes)
         pool.copy_(torch.randint(-128, 128, (blocks * nbytes,), dtype=torch.int8,
@@ -206,12 +209,24 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--rows", type=int, default=4000000, help="embedding rows (reference: 4 000 000)")
     ap.add_argument("--runs", type=int, default=200)
+    ap.add_argument("--only", default="config1,gather,transfer", help="comma list of: config1, gather, transfer")
+    ap.add_argument("--transfer-shape", default=None,
+                    help="one T,L,H,D instead of the README's four shapes (e.g. 1024,64,8,128), for profiling")
     args = ap.parse_args()
     assert torch.cuda.is_available()
+    parts = set(args.only.split(","))
+    assert parts <= {"config1", "gather", "transfer"}, "unknown part in --only"
     out = {"gather": [], "transfer": [], "rows": args.rows, "runs": args.runs}
-    config1_latency(out)
-    gather_table(args.rows, args.runs, out)
-    transfer_table(out)
+    if "config1" in parts:
+        config1_latency(out)
+    if "gather" in parts:
+        gather_table(args.rows, args.runs, out)
+    if "transfer" in parts:
+        shapes = README_TRANSFER_SHAPES
+        if args.transfer_shape:
+            shapes = (tuple(int(x) for x in args.transfer_shape.split(",")),)
+            assert len(shapes[0]) == 4, "--transfer-shape takes T,L,H,D"
+        transfer_table(out, shapes=shapes)
     print(json.dumps(out))
 
 
