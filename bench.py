@@ -159,6 +159,27 @@ def main():
         wall = time.perf_counter() - t0
         return wall, start.elapsed_time(end) / iters
 
+    def launch_spread(fn, iters):
+        """The same launch timed one at a time (an event pair per launch, a synchronize between launches):
+        the first call of the process (module load and first-touch included, by the host clock), then
+        median / min / max of `iters` isolated launches by HIP events."""
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        first_ms = (time.perf_counter() - t0) * 1e3
+        times = []
+        for _ in range(iters):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            fn()
+            end.record()
+            torch.cuda.synchronize()
+            times.append(start.elapsed_time(end))
+        times.sort()
+        return {"first_call_ms": first_ms, "median_ms": times[len(times) // 2], "min_ms": times[0], "max_ms": times[-1],
+                "isolated_launches": iters}
+
     # ---- PCIe peak as one large pinned copy sees it --------------------------
     big = min(1 << 30, host_pool.numel())
     big_d = torch.empty(big, dtype=torch.int8, device=dev)
@@ -174,7 +195,9 @@ def main():
 
     # ---- the timed steps: swap-out -------------------------------------------
     value = ms_per_step = kernel_ms_out = None
+    spread_out = spread_in = spread_gather = None
     if "swap_out" in sections:
+        spread_out = launch_spread(swap_out, min(args.steps, 10))
         wall, kernel_ms_out = timed(swap_out, args.steps, args.warmup)
         value = args.steps * payload / wall / 1e9
         ms_per_step = wall * 1e3 / args.steps
@@ -204,6 +227,7 @@ def main():
     swap_in_gbps = kernel_ms_in = None
     if "swap_in" in sections:
         expect_in = {p: host_planes[p].index_select(0, dst_ids).clone() for p in range(planes)}
+        spread_in = launch_spread(swap_in, min(args.steps, 10))
         wall_in, kernel_ms_in = timed(swap_in, args.steps, args.warmup)
         for p in range(planes):
             got = dev_bytes[p].index_select(0, back_ids.to(dev)).cpu()
@@ -216,6 +240,7 @@ def main():
     gather_alg_bytes = 2 * payload + 8 * n             # read + write + the id list
     kernel_ms_g = gather_traffic_gbps = gather_payload_gbps = torch_gather_gbps = None
     if "gather" in sections:
+        spread_gather = launch_spread(gather, min(args.steps, 10))
         wall_g, kernel_ms_g = timed(gather, args.steps, args.warmup)
         for p in range(planes):
             assert torch.equal(prefill[p], dev_bytes[p].index_select(0, ids_dev)), "gather mismatch %d" % p
@@ -536,12 +561,12 @@ def main():
             "frac": frac(gather_traffic_gbps, HBM_PEAK_GBPS), "traffic": traffic.get("gather_hbm_bytes_per_launch"),
             "algorithmic_bytes_per_launch": gather_alg_bytes, "avg_launch_ms": kernel_ms_g,
             "payload_GBps": gather_payload_gbps, "torch_index_select_GBps": torch_gather_gbps,
-            "torch_device_copy_GBps": d2d_copy_gbps,
+            "torch_device_copy_GBps": d2d_copy_gbps, "launch_spread": spread_gather,
         },
-        "swap_out": {"GBps": value, "kernel_GBps": out_kernel_gbps,
+        "swap_out": {"GBps": value, "kernel_GBps": out_kernel_gbps, "launch_spread": spread_out,
                      "pct_of_measured_d2h": None if out_kernel_gbps is None else 100 * out_kernel_gbps / d2h_peak,
                      "pct_of_pcie5_x16": None if out_kernel_gbps is None else 100 * out_kernel_gbps / PCIE5_X16_GBPS},
-        "swap_in": {"GBps": swap_in_gbps, "kernel_GBps": in_kernel_gbps,
+        "swap_in": {"GBps": swap_in_gbps, "kernel_GBps": in_kernel_gbps, "launch_spread": spread_in,
                     "pct_of_measured_h2d": None if in_kernel_gbps is None else 100 * in_kernel_gbps / h2d_peak,
                     "pct_of_pcie5_x16": None if in_kernel_gbps is None else 100 * in_kernel_gbps / PCIE5_X16_GBPS},
         "pcie_peak_measured": {"d2h_GBps": d2h_peak, "h2d_GBps": h2d_peak, "theoretical_GBps": PCIE5_X16_GBPS,
