@@ -16,6 +16,12 @@ KNOB_NONTEMPORAL = 1
 KNOB_WORKGROUPS_PER_CU = 2
 KNOB_SWAP_WORKGROUPS = 3
 KNOB_DUPLEX_UNROLL = 4
+KNOB_SWAP_UNROLL = 5
+KNOB_SWAP_PACE_MBPS = 6
+KNOB_LINK_MBPS = 7
+SWAP_DST_HOST = 1
+SWAP_SRC_HOST = 2
+SWAP_BESIDE_COMPUTE = 4
 
 
 class BlockMove(ctypes.Structure):
@@ -83,7 +89,7 @@ def load():
     L.hfk_multi_layer_block_table_transfer.argtypes = [vp, u64, vp, u64, vp, u64, u64, u64, u32, u32, u32, u32, u32, ci,
                                                        u32, vp]
     L.hfk_multi_layer_block_table_transfer.restype = ci
-    L.hfk_swap_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, u32, vp]
+    L.hfk_swap_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, u32, u32, vp]
     L.hfk_swap_blocks.restype = ci
     L.hfk_swap_blocks_duplex.argtypes = [ctypes.POINTER(BlockMove), ctypes.POINTER(BlockMove), u32, u64, u32, vp]
     L.hfk_swap_blocks_duplex.restype = ci
@@ -133,9 +139,9 @@ def multi_layer_block_table_transfer(layer_ptrs, dev_block_stride, packed_blocks
 
 
 def swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, src_stride, dst_stride,
-                src_blocks=0, dst_blocks=0, workgroups=0, stream=0):
+                src_blocks=0, dst_blocks=0, workgroups=0, stream=0, flags=0):
     return load().hfk_swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, src_stride,
-                                  dst_stride, src_blocks, dst_blocks, workgroups, stream)
+                                  dst_stride, src_blocks, dst_blocks, flags, workgroups, stream)
 
 
 def swap_blocks_duplex(out_move, in_move, n_planes, block_bytes, workgroups=0, stream=0):

@@ -140,7 +140,7 @@ int main(int argc, char** argv) {
     for (i = 0; i < n; ++i) { pairs_h[2 * i] = perm_a[i]; pairs_h[2 * i + 1] = perm_b[i]; }
     CHECK_HIP(hipMemcpy(pairs_d, pairs_h, 2 * n * sizeof(int64_t), hipMemcpyHostToDevice));
     printf("step swap-out\n"); fflush(stdout);
-    CHECK_HFK(hfk_swap_blocks(host_tab, dev_tab, (const int64_t*)pairs_d, planes, n, bb, bb, bb, blocks, blocks, 0, stream));
+    CHECK_HFK(hfk_swap_blocks(host_tab, dev_tab, (const int64_t*)pairs_d, planes, n, bb, bb, bb, blocks, blocks, 0, 0, stream));
     CHECK_HIP(hipStreamSynchronize(stream));
     for (p = 0; p < planes; ++p) {
         const uint8_t* h = (const uint8_t*)host_plane[p];
@@ -155,7 +155,8 @@ int main(int argc, char** argv) {
     for (i = 0; i < n; ++i) { pairs_h[2 * i] = perm_b[i]; pairs_h[2 * i + 1] = perm_a[n + i]; }
     CHECK_HIP(hipMemcpy(pairs_d, pairs_h, 2 * n * sizeof(int64_t), hipMemcpyHostToDevice));
     printf("step swap-in\n"); fflush(stdout);
-    CHECK_HFK(hfk_swap_blocks(dev_tab, host_tab, (const int64_t*)pairs_d, planes, n, bb, bb, bb, blocks, blocks, 0, stream));
+    CHECK_HFK(hfk_swap_blocks(dev_tab, host_tab, (const int64_t*)pairs_d, planes, n, bb, bb, bb, blocks, blocks,
+                              HFK_SWAP_SRC_HOST | HFK_SWAP_BESIDE_COMPUTE, 0, stream));   /* the gentle launch shape: same bytes */
     CHECK_HIP(hipStreamSynchronize(stream));
     for (p = 0; p < planes; ++p) {
         CHECK_HIP(hipMemcpy(scratch, dev_plane[p], plane_bytes, hipMemcpyDeviceToHost));

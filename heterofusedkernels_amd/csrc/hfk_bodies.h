@@ -32,6 +32,18 @@
 #define HFK_GLOBAL
 #endif
 
+// Pacing support: a constant-rate 100 MHz counter (independent of the shader clock) and a
+// short sleep. The CPU build walks the same index math without pacing.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define HFK_CAN_PACE 1
+#define HFK_TICKS_100MHZ() wall_clock64()
+#define HFK_NAP() __builtin_amdgcn_s_sleep(2)
+#else
+#define HFK_CAN_PACE 0
+#define HFK_TICKS_100MHZ() ((uint64_t)0)
+#define HFK_NAP() ((void)0)
+#endif
+
 namespace hfk {
 
 constexpr uint32_t kWorkgroupLanes = 256;
@@ -101,6 +113,9 @@ struct BlockCopyArgs {
     uint64_t src_limit;          // block indices must be < limit (unsigned compare,
     uint64_t dst_limit;          // so negative ids are rejected as well)
     uint32_t n_work;             // n_planes * n_pairs * chunks_per_block
+    uint32_t pace_q8;            // != 0: workgroup b starts its k-th chunk no earlier than
+                                 //       (k + b / workgroups) * pace_q8 / 256 ticks of the 100 MHz counter
+                                 //       after it began, i.e. the launch offers a fixed byte rate
 };
 
 // Where work item w of a block copy reads and writes. Everything here is uniform
@@ -182,7 +197,20 @@ HFK_HD void copy_chunk(uint64_t s_addr, uint64_t d_addr, uint64_t block_bytes, u
 
 template <typename IdT, int UNROLL, int NT>
 HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+    // Pacing (swaps that run beside other kernels): offering the PCIe link more than it drains
+    // fills the queues that every other kernel's memory traffic shares; offering it a fixed rate
+    // just under its capacity keeps them empty at the same throughput.
+    const bool paced = HFK_CAN_PACE && a.pace_q8 != 0;
+    const uint64_t t0 = paced ? HFK_TICKS_100MHZ() : 0;
+    uint64_t due_q8 = paced ? (uint64_t)a.pace_q8 * bid / nb : 0;  // workgroups take turns within an interval
     for (uint32_t w = bid; w < a.n_work; w += nb) {
+        if (paced) {
+            // The counter always advances; the spin limit ends the wait regardless.
+            for (uint32_t spin = 0; spin < (1u << 16) && ((HFK_TICKS_100MHZ() - t0) << 8) < due_q8; ++spin) {
+                HFK_NAP();
+            }
+            due_q8 += a.pace_q8;
+        }
         uint64_t s_addr = 0, d_addr = 0;
         uint32_t chunk = 0;
         if (!resolve_chunk(a, w, s_addr, d_addr, chunk)) {

@@ -14,7 +14,10 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cctype>
 #include <cstdint>
+#include <cstdio>
+#include <cstdlib>
 
 #include "hfk.h"
 #include "hfk_bodies.h"
@@ -93,6 +96,27 @@ std::atomic<int> g_swap_workgroups{64};
 // one vector per lane and direction on 96-192 workgroups is a flat 97.5-99 GB/s summed
 // for 16, 32 and 72 KiB blocks (unroll 8 loses 6 %); its grid defaults to twice the swap's.
 std::atomic<int> g_duplex_unroll{1};
+std::atomic<int> g_swap_unroll{8};
+// Explicit offered rate of a swap that runs beside compute, MB/s; 0 = derive it from the link.
+std::atomic<int> g_swap_pace_mbps{0};
+// PCIe link rate override, MB/s; -1 = read each device's link from sysfs on first use.
+std::atomic<int> g_link_mbps_override{-1};
+
+// A swap that shares the GPU with other kernels (HFK_SWAP_BESIDE_COMPUTE) runs a grid this small:
+// enough workgroups to keep the link busy, few enough that what they hold in flight stays near the
+// link's bandwidth-delay product. Measured on MI355X, 16-72 KiB blocks:
+//  * writes to host: 8 workgroups x 4 vectors per lane, paced, sustain 56.8 GB/s (more than any
+//    unpaced grid: 55.5) and slow a memory-bound neighbour by 3-30 % where the 64-workgroup
+//    grid slows it 4-5x;
+//  * reads from host: pacing changes nothing, the neighbour's slowdown grows with the number of
+//    resident workgroups (8: 1.15-1.3x, 16: 1.3-1.8x, 64: 4-5x) while 8 already reach 57.5 GB/s on
+//    blocks that are whole 16 KiB chunks; other block sizes need 16.
+constexpr uint32_t kBesideWorkgroups = 8;
+constexpr int kBesideUnroll = 4;
+// Share of the link's raw rate offered to host writes when pacing. 256-byte transaction payloads
+// cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured); from 0.92 on throughput collapses to
+// 0.84 and the neighbours' slowdown doubles, so stay clear of the edge.
+constexpr double kPaceShareOfLink = 0.86;
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
@@ -134,6 +158,51 @@ int finish_launch() {
     return e == hipSuccess ? HFK_OK : (int)e;
 }
 
+// Raw PCIe rate of a device's link in MB/s (lanes x GT/s x line encoding), from sysfs; 0 if unknown.
+std::atomic<int> g_link_mbps[kMaxDevices];   // 0 = not read yet, -1 = unknown
+
+int read_link_mbps(int dev) {
+    char bdf[32] = {0};
+    if (hipDeviceGetPCIBusId(bdf, (int)sizeof(bdf), dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    for (char* c = bdf; *c; ++c) *c = (char)std::tolower((unsigned char)*c);
+    char path[128];
+    double gts = 0.0;
+    int width = 0;
+    std::snprintf(path, sizeof(path), "/sys/bus/pci/devices/%s/current_link_speed", bdf);
+    if (FILE* f = std::fopen(path, "r")) {
+        if (std::fscanf(f, "%lf", &gts) != 1) gts = 0.0;
+        std::fclose(f);
+    }
+    std::snprintf(path, sizeof(path), "/sys/bus/pci/devices/%s/current_link_width", bdf);
+    if (FILE* f = std::fopen(path, "r")) {
+        if (std::fscanf(f, "%d", &width) != 1) width = 0;
+        std::fclose(f);
+    }
+    if (gts <= 0.0 || width <= 0 || width > 32) return -1;
+    const double encoding = gts >= 8.0 ? 128.0 / 130.0 : 0.8;     // 8b/10b below 8 GT/s
+    return (int)(gts * 1000.0 * width * encoding / 8.0);
+}
+
+int current_link_mbps() {
+    const int forced = g_link_mbps_override.load(std::memory_order_relaxed);
+    if (forced >= 0) return forced;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    if (dev < 0 || dev >= kMaxDevices) return 0;
+    int v = g_link_mbps[dev].load(std::memory_order_relaxed);
+    if (v == 0) {
+        v = read_link_mbps(dev);
+        g_link_mbps[dev].store(v, std::memory_order_relaxed);
+    }
+    return v > 0 ? v : 0;
+}
+
 // ---- block copy -----------------------------------------------------------
 template <Role ROLE, typename IdT, int UNROLL, int NT>
 void launch_block_copy_one(const BlockCopyArgs<IdT>& a, uint32_t grid, hipStream_t s) {
@@ -159,13 +228,21 @@ void launch_block_copy_nt(const BlockCopyArgs<IdT>& a, uint32_t grid, int nt, hi
 }
 
 template <Role ROLE, typename IdT>
-int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s) {
+int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, int preferred_unroll = 0,
+                      uint32_t pace_mbps = 0) {
     int unroll = 1;
-    int rc = hfk::plan_block_copy<IdT>(a, g_unroll.load(std::memory_order_relaxed), &unroll);
+    if (preferred_unroll == 0) preferred_unroll = g_unroll.load(std::memory_order_relaxed);
+    int rc = hfk::plan_block_copy<IdT>(a, preferred_unroll, &unroll);
     if (rc != 0) return rc;
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
+    if (pace_mbps != 0) {
+        // bytes per work item (average over a block) * workgroups / rate, in 1/256 ticks of 10 ns
+        const double item_bytes = (double)a.block_bytes / a.chunks_per_block;
+        const double ticks = item_bytes * grid / ((double)pace_mbps * 1e6) * 1e8;
+        a.pace_q8 = (uint32_t)(ticks * 256.0 + 0.5);
+    }
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
     switch (unroll) {
         case 1: launch_block_copy_nt<ROLE, IdT, 1>(a, grid, nt, s); break;
@@ -283,6 +360,7 @@ const char* hfk_status_string(int status) {
         case HFK_ERR_TOO_LARGE: return "hfk: count exceeds what one launch can index";
         case HFK_ERR_BAD_KNOB: return "hfk: unknown tuning knob or value out of range";
         case HFK_ERR_OUT_OF_RANGE: return "hfk: host-side index outside the declared range";
+        case HFK_ERR_BAD_FLAGS: return "hfk: unknown flag bits";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -340,17 +418,35 @@ int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t de
 
 int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* block_pairs,
                     uint32_t n_planes, uint64_t n_pairs, uint64_t block_bytes, uint64_t src_block_stride,
-                    uint64_t dst_block_stride, uint64_t src_blocks, uint64_t dst_blocks,
+                    uint64_t dst_block_stride, uint64_t src_blocks, uint64_t dst_blocks, uint32_t flags,
                     uint32_t workgroups, hfk_stream_t stream) {
+    if ((flags & ~(uint32_t)(HFK_SWAP_DST_HOST | HFK_SWAP_SRC_HOST | HFK_SWAP_BESIDE_COMPUTE)) != 0) {
+        return HFK_ERR_BAD_FLAGS;
+    }
     if (n_planes == 0 || n_pairs == 0) return HFK_OK;
     BlockCopyArgs<int64_t> a;
     int rc = hfk::plan_swap_blocks(a, dst_plane_ptrs, src_plane_ptrs, block_pairs, n_planes, n_pairs, block_bytes,
                                    src_block_stride, dst_block_stride, src_blocks, dst_blocks);
     if (rc != 0) return rc;
-    // A swap is bound by the PCIe link, which a fraction of the CUs saturates; more
-    // workgroups only queue on the link (1-3 % slower).
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool host_side = (flags & (HFK_SWAP_DST_HOST | HFK_SWAP_SRC_HOST)) != 0;
+    if ((flags & HFK_SWAP_BESIDE_COMPUTE) != 0 && host_side) {
+        uint32_t pace_mbps = 0;
+        if ((flags & HFK_SWAP_DST_HOST) != 0) {
+            pace_mbps = (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed);
+            if (pace_mbps == 0) pace_mbps = (uint32_t)(kPaceShareOfLink * current_link_mbps());
+        }
+        if (workgroups == 0) {
+            const bool whole_chunks = block_bytes % ((uint64_t)kWorkgroupLanes * 16u * kBesideUnroll) == 0;
+            workgroups = ((flags & HFK_SWAP_SRC_HOST) != 0 && !whole_chunks) ? 2 * kBesideWorkgroups : kBesideWorkgroups;
+        }
+        return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, kBesideUnroll, pace_mbps);
+    }
+    // Throughput mode. A swap is bound by the PCIe link, which a small grid saturates; more
+    // workgroups only queue on the link.
     if (workgroups == 0) workgroups = (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
-    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
+    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s,
+                                                         g_swap_unroll.load(std::memory_order_relaxed));
 }
 
 int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move* in_move, uint32_t n_planes,
@@ -505,6 +601,18 @@ int hfk_set_tuning(int knob, int64_t value) {
             if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return HFK_ERR_BAD_KNOB;
             g_duplex_unroll.store((int)value);
             return HFK_OK;
+        case HFK_KNOB_SWAP_UNROLL:
+            if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return HFK_ERR_BAD_KNOB;
+            g_swap_unroll.store((int)value);
+            return HFK_OK;
+        case HFK_KNOB_SWAP_PACE_MBPS:
+            if (value < 0 || value > 1000000) return HFK_ERR_BAD_KNOB;
+            g_swap_pace_mbps.store((int)value);
+            return HFK_OK;
+        case HFK_KNOB_LINK_MBPS:
+            if (value < -1 || value > 1000000) return HFK_ERR_BAD_KNOB;
+            g_link_mbps_override.store((int)value);
+            return HFK_OK;
         default:
             return HFK_ERR_BAD_KNOB;
     }
@@ -517,6 +625,9 @@ int64_t hfk_get_tuning(int knob) {
         case HFK_KNOB_WORKGROUPS_PER_CU: return g_wg_per_cu.load();
         case HFK_KNOB_SWAP_WORKGROUPS: return g_swap_workgroups.load();
         case HFK_KNOB_DUPLEX_UNROLL: return g_duplex_unroll.load();
+        case HFK_KNOB_SWAP_UNROLL: return g_swap_unroll.load();
+        case HFK_KNOB_SWAP_PACE_MBPS: return g_swap_pace_mbps.load();
+        case HFK_KNOB_LINK_MBPS: return current_link_mbps();
         default: return HFK_ERR_BAD_KNOB;
     }
 }

@@ -215,10 +215,11 @@ void multi_layer_block_table_transfer(const at::Tensor& deviceLayerCachePtrs, co
 // (pcieThrough/tests/test_transfer_kernel.py:42-47).
 void swap_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs, const at::Tensor& blockPairs,
                  int64_t blockBytes, int64_t srcBlockStride, int64_t dstBlockStride, int64_t srcBlocks,
-                 int64_t dstBlocks, std::optional<int64_t> workgroups) {
+                 int64_t dstBlocks, std::optional<int64_t> workgroups, int64_t flags) {
     check_ptr_table(dstPlanePtrs, "dstPlanePtrs");
     check_ptr_table(srcPlanePtrs, "srcPlanePtrs");
     check_ptr_table(blockPairs, "blockPairs");
+    TORCH_CHECK(flags >= 0 && flags <= 0xffffffffLL, "swap_blocks: flags out of range");
     TORCH_CHECK(dstPlanePtrs.is_cuda(), "dstPlanePtrs must be a device tensor");
     TORCH_CHECK(dstPlanePtrs.numel() == srcPlanePtrs.numel(), "plane tables differ in length");
     TORCH_CHECK(blockPairs.dim() == 2 && blockPairs.size(1) == 2, "blockPairs must be [n, 2]");
@@ -233,7 +234,8 @@ void swap_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs,
                         static_cast<uint32_t>(dstPlanePtrs.numel()), static_cast<uint64_t>(blockPairs.size(0)),
                         static_cast<uint64_t>(blockBytes), static_cast<uint64_t>(srcBlockStride),
                         static_cast<uint64_t>(dstBlockStride), static_cast<uint64_t>(srcBlocks),
-                        static_cast<uint64_t>(dstBlocks), workgroup_cap(workgroups), current_stream()),
+                        static_cast<uint64_t>(dstBlocks), static_cast<uint32_t>(flags), workgroup_cap(workgroups),
+                        current_stream()),
         "hfk_swap_blocks");
 }
 
@@ -368,7 +370,7 @@ TORCH_LIBRARY(pcie_through, m) {
         "deviceBlockStride, int deviceBlocks=0, bool toHost=False, int? workgroups=None) -> ()");
     m.def(
         "swap_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockPairs, int blockBytes, int "
-        "srcBlockStride, int dstBlockStride, int srcBlocks=0, int dstBlocks=0, int? workgroups=None) -> ()");
+        "srcBlockStride, int dstBlockStride, int srcBlocks=0, int dstBlocks=0, int? workgroups=None, int flags=0) -> ()");
     m.def(
         "swap_blocks_duplex(Tensor devicePlanePtrs, Tensor hostPlanePtrs, Tensor outBlockPairs, Tensor inBlockPairs, int "
         "blockBytes, int deviceBlockStride, int hostBlockStride, int deviceBlocks=0, int hostBlocks=0, int? "

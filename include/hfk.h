@@ -40,7 +40,8 @@ enum hfk_status {
     HFK_ERR_BAD_SIZE = -2,     /* a size/stride is zero or inconsistent          */
     HFK_ERR_TOO_LARGE = -3,    /* a count exceeds what one launch can index      */
     HFK_ERR_BAD_KNOB = -4,     /* unknown tuning knob or value out of range      */
-    HFK_ERR_OUT_OF_RANGE = -5  /* an index passed in host memory is out of range */
+    HFK_ERR_OUT_OF_RANGE = -5, /* an index passed in host memory is out of range */
+    HFK_ERR_BAD_FLAGS = -6     /* a flags argument has unknown bits set            */
 };
 
 /* HFK_VERSION_MAJOR * 1000 + HFK_VERSION_MINOR of the loaded library. */
@@ -162,17 +163,35 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *   block_pairs   device-visible int64 [n_pairs, 2] = (src_block, dst_block)
  *   src_blocks, dst_blocks  blocks per plane on each side; a pair with an index
  *                 outside its range is skipped. 0 disables that side's check.
- *   workgroups    0 = library default, which is sized for the PCIe link (a small
- *                 grid saturates it); pass a large bound (e.g. 64 per CU) when both
- *                 sides are device memory.
+ *   flags         what the caller knows about the call, any combination of
+ *                   HFK_SWAP_DST_HOST        the destination planes are host memory (swap-out)
+ *                   HFK_SWAP_SRC_HOST        the source planes are host memory (swap-in)
+ *                   HFK_SWAP_BESIDE_COMPUTE  other kernels run at the same time and matter
+ *                 0 is always valid and means "move the blocks as fast as possible". The result
+ *                 never depends on flags; they select the launch shape:
+ *                 - without HFK_SWAP_BESIDE_COMPUTE the grid keeps far more in flight than the
+ *                   link needs. That is the fastest way to drain a swap when the GPU is otherwise
+ *                   idle, and the excess queues in the memory fabric in front of every other
+ *                   kernel's traffic: a memory-bound kernel on another stream runs 4-5x slower
+ *                   while such a swap is in flight (measured on MI355X);
+ *                 - with HFK_SWAP_BESIDE_COMPUTE and a host side named, the swap runs 8-16
+ *                   workgroups and, toward the host, offers a fixed rate just under the link's
+ *                   capacity (HFK_KNOB_LINK_MBPS). Same throughput (-2 % out, +1 % in), the
+ *                   neighbour's slowdown drops to 3-30 %.
+ *   workgroups    0 = the default of the mode chosen by flags; otherwise an upper bound on the
+ *                 grid. The throughput default is sized for the PCIe link: pass a large bound
+ *                 (e.g. 64 per CU) when both sides are device memory.
  * Destination blocks must be distinct (as index_copy_ requires for a
  * deterministic result); source and destination ranges must not overlap.
  */
+#define HFK_SWAP_DST_HOST 1u
+#define HFK_SWAP_SRC_HOST 2u
+#define HFK_SWAP_BESIDE_COMPUTE 4u
 HFK_API int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs,
                     const int64_t* block_pairs, uint32_t n_planes, uint64_t n_pairs,
                     uint64_t block_bytes, uint64_t src_block_stride,
                     uint64_t dst_block_stride, uint64_t src_blocks, uint64_t dst_blocks,
-                    uint32_t workgroups, hfk_stream_t stream);
+                    uint32_t flags, uint32_t workgroups, hfk_stream_t stream);
 
 /*
  * One side of hfk_swap_blocks_duplex: the arguments of one hfk_swap_blocks call
@@ -276,7 +295,14 @@ enum hfk_knob {
     HFK_KNOB_WORKGROUPS_PER_CU = 2, /* default grid bound of the gathers and the
                                        transfer = CUs * this, 1..1024                  */
     HFK_KNOB_SWAP_WORKGROUPS = 3,   /* default grid bound of hfk_swap_blocks           */
-    HFK_KNOB_DUPLEX_UNROLL = 4      /* like HFK_KNOB_UNROLL, for hfk_swap_blocks_duplex */
+    HFK_KNOB_DUPLEX_UNROLL = 4,     /* like HFK_KNOB_UNROLL, for hfk_swap_blocks_duplex */
+    HFK_KNOB_SWAP_UNROLL = 5,       /* like HFK_KNOB_UNROLL, for hfk_swap_blocks (throughput mode) */
+    HFK_KNOB_SWAP_PACE_MBPS = 6,    /* rate a HFK_SWAP_BESIDE_COMPUTE swap offers toward the host, MB/s;
+                                       0 (default) = 86 % of HFK_KNOB_LINK_MBPS               */
+    HFK_KNOB_LINK_MBPS = 7          /* raw rate of the current device's PCIe link, MB/s. Default: lanes x
+                                       GT/s x line encoding read from sysfs (0 if unreadable: such swaps
+                                       then run unpaced). Setting it overrides every device; -1 restores
+                                       the default                                                  */
 };
 HFK_API int hfk_set_tuning(int knob, int64_t value);
 HFK_API int64_t hfk_get_tuning(int knob);

@@ -51,6 +51,14 @@ def test_capi_loads_and_reports():
     assert capi.get_tuning(capi.KNOB_UNROLL) in (1, 2, 4, 8, 16)
     assert capi.set_tuning(capi.KNOB_UNROLL, 3) == -4
     assert capi.set_tuning(99, 1) == -4
+    assert "flag" in capi.status_string(-6)
+    # the PCIe link rate: an override is reported back, -1 returns to auto-detection (0 = unknown without a device)
+    assert capi.set_tuning(capi.KNOB_LINK_MBPS, 31500) == 0
+    assert capi.get_tuning(capi.KNOB_LINK_MBPS) == 31500
+    assert capi.set_tuning(capi.KNOB_LINK_MBPS, -1) == 0
+    assert capi.get_tuning(capi.KNOB_LINK_MBPS) >= 0
+    assert capi.set_tuning(capi.KNOB_LINK_MBPS, -2) == -4
+    assert capi.set_tuning(capi.KNOB_SWAP_PACE_MBPS, 0) == 0
 
 
 def test_argument_errors_are_reported_before_any_gpu_work():
@@ -63,6 +71,8 @@ def test_argument_errors_are_reported_before_any_gpu_work():
     assert capi.swap_blocks(8, 8, 8, 2, 2, 32, 16, 32) == -2           # stride < block
     assert capi.swap_blocks(8, 8, 8, 2, 2, 0, 16, 32) == -2
     assert capi.swap_blocks(8, 8, 8, 2, 1 << 33, 16, 16, 16) == -3
+    assert capi.swap_blocks(8, 8, 8, 2, 2, 16, 16, 16, flags=8) == -6  # unknown flag bit
+    assert capi.swap_blocks(0, 0, 0, 0, 0, 16, 16, 16, flags=capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE) == 0
     assert capi.gather_blocks(8, 8, 0, 2, 2, 16, 16) == -1
     assert capi.gather_blocks(8, 8, 8, 2, 2, 32, 16) == -2
     assert capi.multi_layer_block_transfer(0, 8, 4, 4, 4, 4, 2) == -1

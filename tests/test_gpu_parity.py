@@ -390,6 +390,88 @@ def test_staged_swap_equals_direct_swap(memory, cfg, n, pattern):
                                                   cfg.dev_blocks, cfg.host_blocks)
 
 
+@pytest.mark.parametrize("cfg", [
+    W.C2_LLAMA8B_SWAP_OUT.scaled(layers=4, dev_blocks=256, host_blocks=256, n_blocks=96),
+    W.C4_MLA_ROUNDTRIP.scaled(layers=5, dev_blocks=96, host_blocks=96, n_blocks=40),       # 72 KiB blocks: 4.5 chunks
+    W.C5_FP8_FRAGMENTED.scaled(layers=2, dev_blocks=512, host_blocks=512, n_blocks=200),
+], ids=lambda c: c.name)
+def test_swap_beside_compute_moves_the_same_bytes(memory, cfg):
+    """HFK_SWAP_BESIDE_COMPUTE only changes the launch shape (8-16 workgroups, paced toward the host):
+    swap-out then swap-in with the flags == index_select / index_copy_, untouched blocks included."""
+    announce("swap beside compute %s: %d planes, %d pairs, %d B blocks, link %d MB/s"
+             % (cfg.name, cfg.planes, cfg.n_blocks, cfg.block_bytes, capi.get_tuning(capi.KNOB_LINK_MBPS)))
+    bb = cfg.block_bytes
+    cpu = [W.as_bytes(p).clone() for p in _cpu_planes(cfg, cfg.dev_blocks)]
+    dev = [p.to(DEV) for p in cpu]
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0x33)
+    src_ids, dst_ids = W.block_table(cfg, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    dtab, htab = ptr_table(dev), host_ptr_table(host)
+    out_pairs = W.pairs_tensor(src_ids, dst_ids).to(DEV)
+    capi.check(capi.swap_blocks(htab.data_ptr(), dtab.data_ptr(), out_pairs.data_ptr(), cfg.planes, src_ids.numel(), bb, bb, bb,
+                                cfg.dev_blocks, cfg.host_blocks, 0, stream_handle(),
+                                capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE), "hfk_swap_blocks(out, beside compute)")
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.host_blocks, bb), 0x33, dtype=torch.uint8)
+        O.torch_swap_blocks(want, cpu[p], src_ids, dst_ids)
+        assert torch.equal(host[p], want), "plane %d host side" % p
+    back = torch.roll(src_ids, 5)
+    fresh = [torch.full((cfg.dev_blocks, bb), 0x77, dtype=torch.uint8, device=DEV) for _ in range(cfg.planes)]
+    in_pairs = W.pairs_tensor(dst_ids, back).to(DEV)
+    capi.check(capi.swap_blocks(ptr_table(fresh).data_ptr(), htab.data_ptr(), in_pairs.data_ptr(), cfg.planes, back.numel(), bb, bb,
+                                bb, cfg.host_blocks, cfg.dev_blocks, 0, stream_handle(),
+                                capi.SWAP_SRC_HOST | capi.SWAP_BESIDE_COMPUTE), "hfk_swap_blocks(in, beside compute)")
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.dev_blocks, bb), 0x77, dtype=torch.uint8)
+        O.torch_swap_blocks(want, host[p], dst_ids, back)
+        assert torch.equal(fresh[p].cpu(), want), "plane %d device side" % p
+    # and through the torch op
+    for p in range(cfg.planes):
+        host[p].fill_(0x33)
+    torch.ops.pcie_through.swap_blocks(htab, dtab, out_pairs, bb, bb, bb, cfg.dev_blocks, cfg.host_blocks, None,
+                                       capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE)
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.host_blocks, bb), 0x33, dtype=torch.uint8)
+        O.torch_swap_blocks(want, cpu[p], src_ids, dst_ids)
+        assert torch.equal(host[p], want), "plane %d host side (op)" % p
+    with pytest.raises(RuntimeError, match="flag"):
+        torch.ops.pcie_through.swap_blocks(htab, dtab, out_pairs, bb, bb, bb, cfg.dev_blocks, cfg.host_blocks, None, 64)
+
+
+def test_paced_swap_ends_when_its_rate_is_unreachably_low(memory):
+    """The pacing wait is bounded: at an offered rate of 1 MB/s every chunk's wait runs into its spin limit
+    (a few milliseconds) and the swap still completes with the right bytes; an unknown link rate
+    (0) simply runs unpaced."""
+    cfg = W.C2_LLAMA8B_SWAP_OUT.scaled(layers=1, dev_blocks=16, host_blocks=16, n_blocks=8)
+    bb = cfg.block_bytes
+    cpu = [W.as_bytes(p).clone() for p in _cpu_planes(cfg, cfg.dev_blocks)]
+    dev = [p.to(DEV) for p in cpu]
+    src_ids, dst_ids = W.block_table(cfg, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    pairs = W.pairs_tensor(src_ids, dst_ids).to(DEV)
+    dtab = ptr_table(dev)
+    try:
+        for what, knob, value in (("1 MB/s", capi.KNOB_SWAP_PACE_MBPS, 1), ("unknown link", capi.KNOB_LINK_MBPS, 0)):
+            announce("paced swap, %s: %d planes x %d blocks" % (what, cfg.planes, src_ids.numel()))
+            assert capi.set_tuning(knob, value) == 0
+            pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0x11)
+            capi.check(capi.swap_blocks(host_ptr_table(host).data_ptr(), dtab.data_ptr(), pairs.data_ptr(), cfg.planes,
+                                        src_ids.numel(), bb, bb, bb, cfg.dev_blocks, cfg.host_blocks, 0, stream_handle(),
+                                        capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE))
+            torch.cuda.synchronize()
+            for p in range(cfg.planes):
+                want = torch.full((cfg.host_blocks, bb), 0x11, dtype=torch.uint8)
+                O.torch_swap_blocks(want, cpu[p], src_ids, dst_ids)
+                assert torch.equal(host[p], want), "%s plane %d" % (what, p)
+            assert capi.set_tuning(capi.KNOB_SWAP_PACE_MBPS, 0) == 0
+            assert capi.set_tuning(capi.KNOB_LINK_MBPS, -1) == 0
+    finally:
+        capi.set_tuning(capi.KNOB_SWAP_PACE_MBPS, 0)
+        capi.set_tuning(capi.KNOB_LINK_MBPS, -1)
+    assert capi.get_tuning(capi.KNOB_LINK_MBPS) > 0, "the PCIe link of the device should be readable from sysfs here"
+
+
 # ---------------------------------------------------------------------------
 # edge cases
 # ---------------------------------------------------------------------------

@@ -97,10 +97,13 @@ def test_random_swap_blocks(seed):
         n = int(rng.integers(0, dst_blocks + 1))
         with_bad = bool(rng.integers(0, 2))
         wg = int(rng.choice([0, 0, 1, 3, 1000]))
+        # the flags only choose the launch shape (grid, pacing): any value gives the same bytes
+        flags = int(rng.choice([0, capi.SWAP_BESIDE_COMPUTE, capi.SWAP_BESIDE_COMPUTE | capi.SWAP_DST_HOST,
+                                capi.SWAP_BESIDE_COMPUTE | capi.SWAP_SRC_HOST, capi.SWAP_DST_HOST, capi.SWAP_SRC_HOST]))
         announce("random swap seed %d case %d: planes %d, blocks %d->%d, %d B (strides %d/%d, offsets %d/%d), "
-                 "src_host %s dst_host %s, %d pairs, bad %s, workgroups %d"
+                 "src_host %s dst_host %s, %d pairs, bad %s, workgroups %d, flags %d"
                  % (seed, case, n_planes, src_blocks, dst_blocks, bb, sstride, dstride, soff, doff, src_host, dst_host,
-                    n, with_bad, wg))
+                    n, with_bad, wg, flags))
         src = Arena(soff + n_planes * src_blocks * sstride, src_host, rng)
         dst = Arena(doff + n_planes * dst_blocks * dstride, dst_host, rng)
         pairs, valid = _pairs(rng, n, src_blocks, dst_blocks, with_bad)
@@ -109,7 +112,7 @@ def test_random_swap_blocks(seed):
         dtab = _table(_planes(dst.addr, doff, n_planes, dst_blocks, dstride))
         capi.check(capi.swap_blocks(dtab.data_ptr(), stab.data_ptr(), pairs_d.data_ptr() if pairs.shape[0] else None,
                                     n_planes, pairs.shape[0], bb, sstride, dstride, src_blocks, dst_blocks, wg,
-                                    stream_handle()), "hfk_swap_blocks")
+                                    stream_handle(), flags), "hfk_swap_blocks")
         torch.cuda.synchronize()
         want = _expect_swap(dst.before, src.before, doff, soff, n_planes, dst_blocks, src_blocks, dstride, sstride, bb, valid)
         assert np.array_equal(dst.now(), want)
