@@ -43,7 +43,7 @@ def main():
                     help="comma list of the GPU sections to run; swap_out is the timed step and always runs unless "
                          "a profile of one other kernel alone is wanted")
     ap.add_argument("--tune", default="", help="comma list of library knobs for experiments, e.g. unroll=4,nt=0 "
-                    "(unroll, nt, wg_per_cu, swap_wgs, duplex_unroll); defaults are the shipped ones")
+                    "(unroll, nt, wg_per_cu, swap_wgs, swap_unroll, duplex_unroll, pace_mbps, link_mbps); defaults are the shipped ones")
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--skip-memcpy-loop", action="store_true")
     args = ap.parse_args()
@@ -63,7 +63,8 @@ def main():
     from heterofusedkernels_amd import workloads as W
 
     knobs = {"unroll": capi.KNOB_UNROLL, "nt": capi.KNOB_NONTEMPORAL, "wg_per_cu": capi.KNOB_WORKGROUPS_PER_CU,
-             "swap_wgs": capi.KNOB_SWAP_WORKGROUPS, "duplex_unroll": capi.KNOB_DUPLEX_UNROLL}
+             "swap_wgs": capi.KNOB_SWAP_WORKGROUPS, "duplex_unroll": capi.KNOB_DUPLEX_UNROLL,
+             "swap_unroll": capi.KNOB_SWAP_UNROLL, "pace_mbps": capi.KNOB_SWAP_PACE_MBPS, "link_mbps": capi.KNOB_LINK_MBPS}
     tuned = {}
     for item in filter(None, args.tune.split(",")):
         key, val = item.split("=")
@@ -338,7 +339,7 @@ def main():
             (duplex_kernel_gbps, total / dt / 1e9, duplex["memcpy_both_directions_GBps"]))
 
     # ---- staged swap (gather kernel on HBM + DMA copies) and what each path costs a kernel beside it ----
-    staged = None
+    staged = beside = None
     if "staged" in sections:
         run_start = 0          # the earlier sections' results are verified by now: their host slots may be reused
         host_run = torch.arange(run_start, run_start + n)
@@ -385,48 +386,96 @@ def main():
         torch.cuda.synchronize()
         staged_duplex_gbps = args.steps * 2 * payload / (time.perf_counter() - t0) / 1e9
         del staging_b
-        # a compute kernel on another stream: alone, beside the direct swap-out, beside the staged swap-out
+        # kernels on another stream: alone, and beside each way of swapping. Three neighbours: a compute-bound
+        # GEMM, an HBM-bound 1 GiB device copy and an attention kernel (mixed).
         side, comp = stream_a, stream_b
         ga = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
         gb = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
-        for _ in range(3):
-            torch.mm(ga, gb)
+        ca = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        cb = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        qkv = torch.randn(8, 32, 2048, 128, device=dev, dtype=torch.bfloat16)
+        neighbours = {
+            "gemm_8192_bf16": (lambda: torch.mm(ga, gb), 30),
+            "device_copy_1GiB": (lambda: ca.copy_(cb), 40),
+            "sdpa_8x32x2048x128_bf16": (lambda: torch.nn.functional.scaled_dot_product_attention(qkv, qkv, qkv, is_causal=True), 30),
+        }
+        for fn, _ in neighbours.values():
+            for _ in range(3):
+                fn()
 
-        def gemm_ms(side_fn, reps):
+        def neighbour_ms(fn, reps, side_fn=None, side_reps=0):
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            if side_fn is not None:
-                for _ in range(reps):
-                    side_fn(side.cuda_stream)
+            for _ in range(side_reps):
+                side_fn(side.cuda_stream)
             with torch.cuda.stream(comp):
                 e0.record()
-                for _ in range(40):
-                    torch.mm(ga, gb)
+                for _ in range(reps):
+                    fn()
                 e1.record()
+            e1.synchronize()
+            covered = side_fn is None or not side.query()      # the swaps must outlast the neighbour
             torch.cuda.synchronize()
-            return e0.elapsed_time(e1) / 40
+            return e0.elapsed_time(e1) / reps, covered
 
-        def direct_out(st):
-            capi.check(capi.swap_blocks(host_tab.data_ptr(), dev_tab.data_ptr(), pairs_out.data_ptr(), planes, n, bb, bb,
-                                        bb, cfg.dev_blocks, cfg.host_blocks, 0, st), "hfk_swap_blocks(out)")
+        beside_out_flags = capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE
+        beside_in_flags = capi.SWAP_SRC_HOST | capi.SWAP_BESIDE_COMPUTE
 
-        gemm_alone = gemm_ms(None, 0)
-        reps = max(1, int(round(40 * gemm_alone / (payload / 55e6))))      # side work lasting about as long as the GEMMs
-        gemm_direct = gemm_ms(direct_out, reps)
-        gemm_staged = gemm_ms(staged_out, reps)
-        del ga, gb, staging_buf
+        def direct(direction, flags):
+            def call(st):
+                if direction == "out":
+                    capi.check(capi.swap_blocks(host_tab.data_ptr(), dev_tab.data_ptr(), pairs_out.data_ptr(), planes, n, bb,
+                                                bb, bb, cfg.dev_blocks, cfg.host_blocks, 0, st, flags), "hfk_swap_blocks(out)")
+                else:
+                    capi.check(capi.swap_blocks(dev_tab.data_ptr(), host_tab.data_ptr(), pairs_in.data_ptr(), planes, n, bb,
+                                                bb, bb, cfg.host_blocks, cfg.dev_blocks, 0, st, flags), "hfk_swap_blocks(in)")
+            return call
+
+        def staged_in_on(st):
+            capi.check(capi.swap_blocks_staged(dev_tab.data_ptr(), host_addrs.data_ptr(), back_dev.data_ptr(),
+                                               host_run.data_ptr(), planes, n, bb, bb, bb, cfg.dev_blocks,
+                                               cfg.host_blocks, staging_buf.data_ptr(), False, 0, st),
+                       "hfk_swap_blocks_staged(in)")
+
+        ways = {"throughput_out": direct("out", 0), "throughput_in": direct("in", 0),
+                "beside_compute_out": direct("out", beside_out_flags), "beside_compute_in": direct("in", beside_in_flags),
+                "staged_out": staged_out, "staged_in": staged_in_on}
+        # own rate of the beside-compute launch shape, GPU otherwise idle; result checked like the plain swap-out's
+        for p_ in range(planes):
+            host_planes[p_][dst_ids] = 0
+        _, ms_bo = timed(lambda: ways["beside_compute_out"](stream), args.steps, args.warmup)
+        for p_ in range(planes):
+            assert torch.equal(host_planes[p_].index_select(0, dst_ids), dev_bytes[p_].index_select(0, ids_dev).cpu()), \
+                "beside-compute swap-out mismatch in plane %d" % p_
+        _, ms_bi = timed(lambda: ways["beside_compute_in"](stream), args.steps, args.warmup)
+        for p_ in range(planes):
+            assert torch.equal(dev_bytes[p_].index_select(0, back_dev).cpu(), host_planes[p_].index_select(0, dst_ids)), \
+                "beside-compute swap-in mismatch in plane %d" % p_
+        alone = {k: neighbour_ms(fn, reps)[0] for k, (fn, reps) in neighbours.items()}
+        side_reps = max(2, int(round(0.09 / (payload / 55e9))))          # about 90 ms of swapping
+        slowdown = {}
+        for way, side_fn in ways.items():
+            slowdown[way] = {}
+            for k, (fn, reps) in neighbours.items():
+                ms, covered = neighbour_ms(fn, reps, side_fn, side_reps)
+                slowdown[way][k] = round(ms / alone[k], 3) if covered else None
+        del ga, gb, ca, cb, qkv, staging_buf
         staged = {"swap_out_GBps": payload / (ms_so * 1e6), "swap_in_GBps": payload / (ms_si * 1e6),
                   "out_and_in_on_two_streams_GBps": staged_duplex_gbps,
                   "host_slots": "one run of %d consecutive slots per plane (%.1f MiB per plane, 2-D DMA copies over "
-                                "evenly spaced planes)" % (n, n * bb / 2**20),
-                  "gemm_8192_bf16_ms_alone": gemm_alone, "gemm_ms_beside_direct_swap_out": gemm_direct,
-                  "gemm_ms_beside_staged_swap_out": gemm_staged,
-                  "gemm_slowdown_pct_direct": 100 * (gemm_direct / gemm_alone - 1),
-                  "gemm_slowdown_pct_staged": 100 * (gemm_staged / gemm_alone - 1)}
-        log("staged swap, verified: out %.2f GB/s, in %.2f GB/s, both on two streams %.2f GB/s summed; a bf16 8192^3 GEMM on another stream takes %.3f ms "
-            "alone, %.3f ms (%+.0f %%) beside the direct swap-out, %.3f ms (%+.0f %%) beside the staged one" %
-            (staged["swap_out_GBps"], staged["swap_in_GBps"], staged_duplex_gbps, gemm_alone, gemm_direct,
-             staged["gemm_slowdown_pct_direct"], gemm_staged, staged["gemm_slowdown_pct_staged"]))
+                                "evenly spaced planes)" % (n, n * bb / 2**20)}
+        beside = {"swap_out_GBps": payload / (ms_bo * 1e6), "swap_in_GBps": payload / (ms_bi * 1e6),
+                  "link_MBps_from_sysfs": capi.get_tuning(capi.KNOB_LINK_MBPS),
+                  "neighbour_ms_alone": alone,
+                  "neighbour_slowdown": slowdown,
+                  "how": "each neighbour runs %s times on one stream while %d swaps of %d MiB are queued on another; "
+                         "x = its time per call / its time alone; null = the swaps ended first" %
+                         ("/".join(str(r) for _, r in neighbours.values()), side_reps, payload >> 20)}
+        log("staged swap, verified: out %.2f GB/s, in %.2f GB/s, both on two streams %.2f GB/s summed" %
+            (staged["swap_out_GBps"], staged["swap_in_GBps"], staged_duplex_gbps))
+        log("swap with HFK_SWAP_BESIDE_COMPUTE, verified: out %.2f GB/s, in %.2f GB/s" % (beside["swap_out_GBps"], beside["swap_in_GBps"]))
+        for way in ways:
+            log("  neighbours beside %-19s %s" % (way + ":", ", ".join("%s x%s" % (k.split("_")[0], v) for k, v in slowdown[way].items())))
 
     # ---- plain device copy of known size: yardstick for reachable HBM bandwidth, and the
     # calibration row for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters -----------------
@@ -573,6 +622,7 @@ def main():
                                "how": "mean of 5 back-to-back hipMemcpyAsync of %d MiB pinned" % (big >> 20)},
         "duplex": duplex,
         "staged": staged,
+        "beside_compute": beside,
         "memcpy_block_loop": memcpy_loop,
         "cpu_baseline": cpu_baseline,
         "verified": "bit-exact on every plane: " + ", ".join(sorted(sections)),

@@ -7,10 +7,12 @@
 // to XCDs round-robin, and a work item's neighbours bid+-1 sit on other XCDs while
 // the item itself streams one contiguous span, so no XCD's L2 sees another's lines
 // -- and lets a caller bound the grid (the `workgroups` argument). PCIe-bound
-// launches default to a small grid: the link needs no more. A small grid does NOT
-// make a swap cheap for kernels running beside it, though: any kernel that touches
-// host memory slows its neighbours by 1.8-2.1x on MI355X whatever its size, which
-// is what hfk_swap_blocks_staged (HBM-only kernel + DMA copies) is for.
+// launches default to a small grid: the link needs no more, and whatever a grid
+// keeps in flight beyond the link's bandwidth-delay product queues in the memory
+// fabric in front of every other kernel's traffic (a memory-bound kernel on another
+// stream runs up to 5x slower beside an oversized swap). A swap that must share the
+// GPU says so (HFK_SWAP_BESIDE_COMPUTE: 8-16 workgroups, paced toward the host) or
+// goes through hfk_swap_blocks_staged (HBM-only kernel + DMA copies).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -86,15 +88,21 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
 //  * HBM-bound launches want one workgroup per chunk (a grid-stride loop over fewer
 //    workgroups lost 5-10 %), so the bound is set high enough to be inactive up to
 //    256 Ki chunks; beyond that the loop takes over.
-//  * PCIe-bound swaps peak at 32-128 workgroups (more only adds queueing on the
-//    link), so a swap defaults to 64 workgroups.
+//  * PCIe-bound swaps are flat from 16 to 128 workgroups (55.4-55.7 GB/s out, 57.0-57.4 in);
+//    what grows with the grid is the harm to kernels on other streams (a memory-bound
+//    neighbour runs 2.3-3x slower beside 16 workgroups, 4-5.7x beside 64), so a swap
+//    defaults to 16. For the same reason the duplex swap defaults to 32 workgroups (98.2 GB/s
+//    summed against 99.1 at 128, neighbours 1.1-1.6x slower instead of 2.8-2.9x) and the
+//    host-facing transfers to 48 (-1 %, neighbours 1.8-2.5x instead of 4.9-5.3x).
 std::atomic<int> g_unroll{8};
 std::atomic<int> g_nontemporal{3};
 std::atomic<int> g_wg_per_cu{1024};
-std::atomic<int> g_swap_workgroups{64};
-// The duplex swap wants little in flight per workgroup and a few more workgroups:
-// one vector per lane and direction on 96-192 workgroups is a flat 97.5-99 GB/s summed
-// for 16, 32 and 72 KiB blocks (unroll 8 loses 6 %); its grid defaults to twice the swap's.
+std::atomic<int> g_swap_workgroups{16};
+constexpr uint32_t kDuplexWorkgroups = 32;
+constexpr uint32_t kTransferWorkgroups = 48;
+// The duplex swap wants little in flight per workgroup: one vector per lane and direction
+// (unroll 8 loses 6 %). 32 workgroups reach 98.1-98.4 GB/s summed for 16, 32 and 72 KiB
+// blocks; 40-64 dip to 89-94, 96-192 are a flat 98-99.
 std::atomic<int> g_duplex_unroll{1};
 std::atomic<int> g_swap_unroll{8};
 // Explicit offered rate of a swap that runs beside compute, MB/s; 0 = derive it from the link.
@@ -114,9 +122,11 @@ std::atomic<int> g_link_mbps_override{-1};
 constexpr uint32_t kBesideWorkgroups = 8;
 constexpr int kBesideUnroll = 4;
 // Share of the link's raw rate offered to host writes when pacing. 256-byte transaction payloads
-// cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured); from 0.92 on throughput collapses to
-// 0.84 and the neighbours' slowdown doubles, so stay clear of the edge.
-constexpr double kPaceShareOfLink = 0.86;
+// cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured, reached only by a paced grid); from 0.92
+// on throughput collapses to 0.84 and the neighbours' slowdown doubles. The closer to the cap, the
+// longer the fabric's queues: a GEMM beside the swap runs 1.56x slower at 0.83, 1.65x at 0.86,
+// 1.9x at 0.87, 2.5x at 0.90 (1.5x is what any resident kernel costs this GEMM).
+constexpr double kPaceShareOfLink = 0.84;
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
@@ -325,10 +335,9 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
                      uint64_t packed_stride, uint64_t layered_stride, uint64_t packed_blocks,
                      uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
                      bool to_packed, bool packed_is_host, uint32_t workgroups, hipStream_t s) {
-    // With the packed side in host memory the PCIe link is the bound and a small grid is
-    // best (measured optimum 64-256 workgroups, both directions); twice the swap default.
+    // With the packed side in host memory the PCIe link is the bound and a small grid does.
     if (workgroups == 0 && packed_is_host) {
-        workgroups = 2u * (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
+        workgroups = kTransferWorkgroups;
     }
     TransposeArgs a;
     uint32_t unit = 16;
@@ -458,7 +467,7 @@ int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move*
                               g_duplex_unroll.load(std::memory_order_relaxed), &unroll);
     if (rc != 0) return rc;
     if (a.n_work == 0) return HFK_OK;
-    if (workgroups == 0) workgroups = 2u * (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
+    if (workgroups == 0) workgroups = kDuplexWorkgroups;
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;

@@ -176,7 +176,7 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *                   while such a swap is in flight (measured on MI355X);
  *                 - with HFK_SWAP_BESIDE_COMPUTE and a host side named, the swap runs 8-16
  *                   workgroups and, toward the host, offers a fixed rate just under the link's
- *                   capacity (HFK_KNOB_LINK_MBPS). Same throughput (-2 % out, +1 % in), the
+ *                   capacity (HFK_KNOB_LINK_MBPS). Same throughput (-4 % out, +1 % in), the
  *                   neighbour's slowdown drops to 3-30 %.
  *   workgroups    0 = the default of the mode chosen by flags; otherwise an upper bound on the
  *                 grid. The throughput default is sized for the PCIe link: pass a large bound
@@ -298,7 +298,7 @@ enum hfk_knob {
     HFK_KNOB_DUPLEX_UNROLL = 4,     /* like HFK_KNOB_UNROLL, for hfk_swap_blocks_duplex */
     HFK_KNOB_SWAP_UNROLL = 5,       /* like HFK_KNOB_UNROLL, for hfk_swap_blocks (throughput mode) */
     HFK_KNOB_SWAP_PACE_MBPS = 6,    /* rate a HFK_SWAP_BESIDE_COMPUTE swap offers toward the host, MB/s;
-                                       0 (default) = 86 % of HFK_KNOB_LINK_MBPS               */
+                                       0 (default) = 84 % of HFK_KNOB_LINK_MBPS               */
     HFK_KNOB_LINK_MBPS = 7          /* raw rate of the current device's PCIe link, MB/s. Default: lanes x
                                        GT/s x line encoding read from sysfs (0 if unreadable: such swaps
                                        then run unpaced). Setting it overrides every device; -1 restores
