@@ -129,8 +129,15 @@ void gather(const at::Tensor& gmEmbed, const at::Tensor& gmEmbedDst, const at::T
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(gmEmbedDst));
     const void* table = device_visible(gmEmbed, "gmEmbed");
     const void* ids = device_visible(gmIds, "gmIds");
+    // A table in host memory (the reference's embedding case) is read over the PCIe link: 64
+    // workgroups already run it at the link's rate (55-57 GB/s for 1 KiB rows), and every further one
+    // only slows kernels on other streams. Gathers of a few MiB keep one workgroup per chunk (they are
+    // over in tens of microseconds and a cap would only add a partly filled second round); a device
+    // table gets the library's HBM-sized grid.
+    const bool longHostGather = !gmEmbed.is_cuda() && numIds * rowBytes > (4ull << 20);
+    const uint32_t workgroups = longHostGather ? 64u : 0u;
     check_status(hfk_gather_rows(table, gmEmbedDst.data_ptr(), ids, gmIds.scalar_type() == at::kLong, numIds,
-                                 rowBytes, tableRows, 0, current_stream()),
+                                 rowBytes, tableRows, workgroups, current_stream()),
                  "hfk_gather_rows");
 }
 

@@ -64,7 +64,10 @@ HFK_API const char* hfk_status_string(int status);
  *   ids         device-visible, int64 (ids_are_i64 != 0) or int32 indices
  *   table_rows  number of rows in table; an id outside [0, table_rows) leaves its
  *               dst row untouched. 0 disables the check (the reference never checks).
- *   workgroups  upper bound on workgroups launched, 0 = library default.
+ *   workgroups  upper bound on workgroups launched, 0 = library default (sized for a table in
+ *               device memory). For a long gather (more than a few MiB) out of a table in host
+ *               memory pass 64: the PCIe link is saturated (55-57 GB/s for 1 KiB rows) and kernels
+ *               on other streams are slowed 2x instead of 5x.
  *
  * n_ids == 0 is a successful no-op. Rows of any byte size and alignment are
  * accepted; 16-byte aligned rows take the vectorised path.
