@@ -177,10 +177,11 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *                   idle, and the excess queues in the memory fabric in front of every other
  *                   kernel's traffic: a memory-bound kernel on another stream runs 4-5x slower
  *                   while such a swap is in flight (measured on MI355X);
- *                 - with HFK_SWAP_BESIDE_COMPUTE and a host side named, the swap runs 8-16
- *                   workgroups and, toward the host, offers a fixed rate just under the link's
+ *                 - with HFK_SWAP_BESIDE_COMPUTE the swap runs 8-16 workgroups and, when
+ *                   HFK_SWAP_DST_HOST says so, offers the host a fixed rate just under the link's
  *                   capacity (HFK_KNOB_LINK_MBPS). Same throughput (-4 % out, +1 % in), the
- *                   neighbour's slowdown drops to 3-30 %.
+ *                   neighbour's slowdown drops to 3-30 %. Name the host side: without it the
+ *                   launch cannot pace (-10 % toward the host).
  *   workgroups    0 = the default of the mode chosen by flags; otherwise an upper bound on the
  *                 grid. The throughput default is sized for the PCIe link: pass a large bound
  *                 (e.g. 64 per CU) when both sides are device memory.
