@@ -44,6 +44,8 @@ def main():
                          "a profile of one other kernel alone is wanted")
     ap.add_argument("--tune", default="", help="comma list of library knobs for experiments, e.g. unroll=4,nt=0 "
                     "(unroll, nt, wg_per_cu, swap_wgs, swap_unroll, duplex_unroll, pace_mbps, link_mbps); defaults are the shipped ones")
+    ap.add_argument("--out-flags", type=int, default=1, help="flags of the timed swap-out (default HFK_SWAP_DST_HOST = 1: "
+                    "the caller knows its destination is host memory; 0 = say nothing)")
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--skip-memcpy-loop", action="store_true")
     args = ap.parse_args()
@@ -136,7 +138,7 @@ def main():
 
     def swap_out():
         capi.check(capi.swap_blocks(host_tab.data_ptr(), dev_tab.data_ptr(), pairs_out.data_ptr(), planes, n, bb, bb,
-                                    bb, cfg.dev_blocks, cfg.host_blocks, 0, stream), "hfk_swap_blocks(out)")
+                                    bb, cfg.dev_blocks, cfg.host_blocks, 0, stream, args.out_flags), "hfk_swap_blocks(out)")
 
     def gather():
         capi.check(capi.gather_blocks(prefill_tab.data_ptr(), dev_tab.data_ptr(), ids_dev.data_ptr(), planes, n, bb, bb,
@@ -223,7 +225,7 @@ def main():
 
     def swap_in():
         capi.check(capi.swap_blocks(dev_tab.data_ptr(), host_tab.data_ptr(), pairs_in.data_ptr(), planes, n, bb, bb, bb,
-                                    cfg.host_blocks, cfg.dev_blocks, 0, stream), "hfk_swap_blocks(in)")
+                                    cfg.host_blocks, cfg.dev_blocks, 0, stream, capi.SWAP_SRC_HOST), "hfk_swap_blocks(in)")
 
     swap_in_gbps = kernel_ms_in = None
     if "swap_in" in sections:
@@ -437,7 +439,7 @@ def main():
                                                cfg.host_blocks, staging_buf.data_ptr(), False, 0, st),
                        "hfk_swap_blocks_staged(in)")
 
-        ways = {"throughput_out": direct("out", 0), "throughput_in": direct("in", 0),
+        ways = {"throughput_out": direct("out", args.out_flags), "throughput_in": direct("in", capi.SWAP_SRC_HOST),
                 "beside_compute_out": direct("out", beside_out_flags), "beside_compute_in": direct("in", beside_in_flags),
                 "staged_out": staged_out, "staged_in": staged_in_on}
         # own rate of the beside-compute launch shape, GPU otherwise idle; result checked like the plain swap-out's
@@ -596,7 +598,8 @@ def main():
         # PCIe Gen5 x16 link, so that is the roofline it is priced against (theoretical link rate as
         # `peak`, the rate one large pinned hipMemcpyAsync reaches in this run as `peak_measured`).
         "roofline": {
-            "kernel": "swap_blocks_kernel<8, 3> via hfk_swap_blocks (swap-out, HBM -> pinned host)", "bound": "pcie",
+            "kernel": ("swap_blocks_kernel<4, 3>, paced" if (args.out_flags & capi.SWAP_DST_HOST) and capi.get_tuning(capi.KNOB_LINK_MBPS) > 0
+                       else "swap_blocks_kernel<8, 3>") + " via hfk_swap_blocks (swap-out, HBM -> pinned host)", "bound": "pcie",
             "achieved": out_kernel_gbps, "peak": PCIE5_X16_GBPS, "unit": "GB/s",
             "frac": frac(out_kernel_gbps, PCIE5_X16_GBPS),
             "traffic": traffic.get("swap_out_hbm_bytes_per_launch"),

@@ -127,6 +127,8 @@ constexpr int kBesideUnroll = 4;
 // longer the fabric's queues: a GEMM beside the swap runs 1.56x slower at 0.83, 1.65x at 0.86,
 // 1.9x at 0.87, 2.5x at 0.90 (1.5x is what any resident kernel costs this GEMM).
 constexpr double kPaceShareOfLink = 0.84;
+// Share offered by a throughput-mode swap-out: the cap itself.
+constexpr double kThroughputShareOfLink = 0.90;
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
@@ -455,8 +457,23 @@ int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, cons
     // Throughput mode. A swap is bound by the PCIe link, which a small grid saturates; more
     // workgroups only queue on the link.
     if (workgroups == 0) workgroups = (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
-    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s,
-                                                         g_swap_unroll.load(std::memory_order_relaxed));
+    if ((flags & HFK_SWAP_DST_HOST) != 0) {
+        // Toward the host the link accepts the most when it is offered exactly what it can take:
+        // paced at its payload-efficiency cap the same grid sustains 56.8 GB/s where it reaches 55.4
+        // unpaced, and should the cap be lower than assumed the launch degrades to the unpaced rate.
+        const uint32_t pace_mbps = (uint32_t)(kThroughputShareOfLink * current_link_mbps());
+        if (pace_mbps != 0) {
+            return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, kBesideUnroll, pace_mbps);
+        }
+    }
+    int unroll = g_swap_unroll.load(std::memory_order_relaxed);
+    if ((flags & HFK_SWAP_SRC_HOST) != 0 && block_bytes % ((uint64_t)kWorkgroupLanes * 16u * kBesideUnroll) == 0 &&
+        unroll > kBesideUnroll) {
+        // From the host, blocks that are whole 16 KiB chunks reach the link rate with half as much in
+        // flight (57.6 GB/s either way; a memory-bound neighbour 1.3-1.7x slower instead of 2.3-2.4x).
+        unroll = kBesideUnroll;
+    }
+    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, unroll);
 }
 
 int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move* in_move, uint32_t n_planes,
