@@ -170,18 +170,21 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *                   HFK_SWAP_DST_HOST        the destination planes are host memory (swap-out)
  *                   HFK_SWAP_SRC_HOST        the source planes are host memory (swap-in)
  *                   HFK_SWAP_BESIDE_COMPUTE  other kernels run at the same time and matter
- *                 0 is always valid and means "move the blocks as fast as possible". The result
- *                 never depends on flags; they select the launch shape:
- *                 - without HFK_SWAP_BESIDE_COMPUTE the grid keeps far more in flight than the
- *                   link needs. That is the fastest way to drain a swap when the GPU is otherwise
- *                   idle, and the excess queues in the memory fabric in front of every other
- *                   kernel's traffic: a memory-bound kernel on another stream runs 4-5x slower
- *                   while such a swap is in flight (measured on MI355X);
+ *                 0 is always valid. The result never depends on flags; they select the launch
+ *                 shape (grid, vectors in flight per lane, pacing). Measured on MI355X:
+ *                 - without HFK_SWAP_BESIDE_COMPUTE the swap is drained as fast as the link allows
+ *                   on 16 workgroups. Naming the host side makes it both faster and less of a
+ *                   burden: toward the host the launch is paced at 0.90 of the link's raw rate
+ *                   (HFK_KNOB_LINK_MBPS), which the link accepts better than an unbounded offer
+ *                   (55.9-56.7 against 54.9-55.7 GB/s), from the host it keeps half as much in
+ *                   flight (57.6 GB/s either way). A memory-bound kernel on another stream still
+ *                   runs 1.2-1.8x slower meanwhile (2.3-3.1x with no side named; 4-5x beside a
+ *                   64-workgroup grid: what a swap holds in flight beyond the link's
+ *                   bandwidth-delay product queues in front of every other kernel's traffic);
  *                 - with HFK_SWAP_BESIDE_COMPUTE the swap runs 8-16 workgroups and, when
- *                   HFK_SWAP_DST_HOST says so, offers the host a fixed rate just under the link's
- *                   capacity (HFK_KNOB_LINK_MBPS). Same throughput (-4 % out, +1 % in), the
- *                   neighbour's slowdown drops to 3-30 %. Name the host side: without it the
- *                   launch cannot pace (-10 % toward the host).
+ *                   HFK_SWAP_DST_HOST says so, offers the host 0.84 of the link's raw rate:
+ *                   52.8 GB/s out, 57.6 in, the neighbour's slowdown drops to 3-30 %. Name the
+ *                   host side: without it the launch cannot pace (49.8 GB/s toward the host).
  *   workgroups    0 = the default of the mode chosen by flags; otherwise an upper bound on the
  *                 grid. The throughput default is sized for the PCIe link: pass a large bound
  *                 (e.g. 64 per CU) when both sides are device memory.
