@@ -249,11 +249,13 @@ HFK_API int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_blo
  * Result: identical to hfk_swap_blocks with the same table; staging holds the moved
  * blocks afterwards.
  *
- * Why it exists: a kernel that reads or writes host memory slows every other kernel
- * running beside it (measured 1.8-2.1x on MI355X for GEMM, attention, softmax and
- * elementwise kernels alike, even for a single swap workgroup), while DMA copies do
- * not (1-7 %). Use hfk_swap_blocks / hfk_swap_blocks_duplex when the GPU is otherwise
- * idle or the swap is on the critical path, this entry point when it overlaps compute.
+ * Why it exists: kernels on other streams run within a few per cent of their time alone beside
+ * it (GEMM, device copy and attention kernels: 0.98-1.04x on MI355X), because the PCIe leg is
+ * DMA and the kernel is short. A swap whose compute units touch host memory costs its neighbours
+ * 1.06-1.3x at best (hfk_swap_blocks with HFK_SWAP_BESIDE_COMPUTE) and any long-resident kernel
+ * costs a GEMM that exactly fills the CUs a whole extra round of tiles (1.5x). Use this entry
+ * point when the swap overlaps compute and its host slots are mostly consecutive; hfk_swap_blocks
+ * when they are scattered, when no staging buffer can be spared, or when the GPU is otherwise idle.
  *
  * Block-table generalisation of the reference's staged variant
  * (pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:82-106: memcpy into a
