@@ -50,6 +50,35 @@ constexpr uint32_t kWorkgroupLanes = 256;
 
 typedef uint32_t vec16 __attribute__((ext_vector_type(4)));
 
+// Pacing of a host-facing copy. Offering the PCIe link more than it drains fills the queues
+// that every other kernel's memory traffic shares (and, toward the host, even lowers what the
+// link accepts); offering it a fixed rate just under its capacity keeps them empty at the same
+// throughput. Workgroup `bid` of `nb` starts its k-th work item no earlier than
+// (k + bid / nb) * pace_q8 / 256 ticks of the 100 MHz counter after it began, so the launch as a
+// whole offers one item per pace_q8 / 256 / nb ticks. pace_q8 == 0: no pacing.
+struct Pacer {
+    uint64_t t0;
+    uint64_t due_q8;
+    uint32_t pace_q8;
+
+    HFK_HD Pacer(uint32_t pace, uint32_t bid, uint32_t nb)
+        : t0(0), due_q8(0), pace_q8(HFK_CAN_PACE ? pace : 0) {
+        if (pace_q8 != 0) {
+            t0 = HFK_TICKS_100MHZ();
+            due_q8 = (uint64_t)pace_q8 * bid / nb;  // workgroups take turns within an interval
+        }
+    }
+
+    // Call before each work item. The counter always advances; the spin limit ends the wait regardless.
+    HFK_HD void wait_turn() {
+        if (pace_q8 == 0) return;
+        for (uint32_t spin = 0; spin < (1u << 16) && ((HFK_TICKS_100MHZ() - t0) << 8) < due_q8; ++spin) {
+            HFK_NAP();
+        }
+        due_q8 += pace_q8;
+    }
+};
+
 // NT bit0: non-temporal loads, bit1: non-temporal stores.
 template <typename V>
 HFK_HD const HFK_GLOBAL V* global_in(uint64_t addr) {
@@ -113,9 +142,7 @@ struct BlockCopyArgs {
     uint64_t src_limit;          // block indices must be < limit (unsigned compare,
     uint64_t dst_limit;          // so negative ids are rejected as well)
     uint32_t n_work;             // n_planes * n_pairs * chunks_per_block
-    uint32_t pace_q8;            // != 0: workgroup b starts its k-th chunk no earlier than
-                                 //       (k + b / workgroups) * pace_q8 / 256 ticks of the 100 MHz counter
-                                 //       after it began, i.e. the launch offers a fixed byte rate
+    uint32_t pace_q8;            // see Pacer; 0 = unpaced
 };
 
 // Where work item w of a block copy reads and writes. Everything here is uniform
@@ -197,20 +224,9 @@ HFK_HD void copy_chunk(uint64_t s_addr, uint64_t d_addr, uint64_t block_bytes, u
 
 template <typename IdT, int UNROLL, int NT>
 HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
-    // Pacing (swaps that run beside other kernels): offering the PCIe link more than it drains
-    // fills the queues that every other kernel's memory traffic shares; offering it a fixed rate
-    // just under its capacity keeps them empty at the same throughput.
-    const bool paced = HFK_CAN_PACE && a.pace_q8 != 0;
-    const uint64_t t0 = paced ? HFK_TICKS_100MHZ() : 0;
-    uint64_t due_q8 = paced ? (uint64_t)a.pace_q8 * bid / nb : 0;  // workgroups take turns within an interval
+    Pacer pacer(a.pace_q8, bid, nb);
     for (uint32_t w = bid; w < a.n_work; w += nb) {
-        if (paced) {
-            // The counter always advances; the spin limit ends the wait regardless.
-            for (uint32_t spin = 0; spin < (1u << 16) && ((HFK_TICKS_100MHZ() - t0) << 8) < due_q8; ++spin) {
-                HFK_NAP();
-            }
-            due_q8 += a.pace_q8;
-        }
+        pacer.wait_turn();
         uint64_t s_addr = 0, d_addr = 0;
         uint32_t chunk = 0;
         if (!resolve_chunk(a, w, s_addr, d_addr, chunk)) {

@@ -93,13 +93,14 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
 //    neighbour runs 2.3-3x slower beside 16 workgroups, 4-5.7x beside 64), so a swap
 //    defaults to 16. For the same reason the duplex swap defaults to 32 workgroups (98.2 GB/s
 //    summed against 99.1 at 128, neighbours 1.1-1.6x slower instead of 2.8-2.9x) and the
-//    host-facing transfers to 48 (-1 %, neighbours 1.8-2.5x instead of 4.9-5.3x).
+//    block-table transfers to 48 (-1 %, neighbours 1.8-2.5x instead of 4.9-5.3x).
 std::atomic<int> g_unroll{8};
 std::atomic<int> g_nontemporal{3};
 std::atomic<int> g_wg_per_cu{1024};
 std::atomic<int> g_swap_workgroups{16};
 constexpr uint32_t kDuplexWorkgroups = 32;
 constexpr uint32_t kTransferWorkgroups = 48;
+constexpr uint32_t kSingleBlockTransferWorkgroups = 128;
 // The duplex swap wants little in flight per workgroup: one vector per lane and direction
 // (unroll 8 loses 6 %). 32 workgroups reach 98.1-98.4 GB/s summed for 16, 32 and 72 KiB
 // blocks; 40-64 dip to 89-94, 96-192 are a flat 98-99.
@@ -129,6 +130,7 @@ constexpr int kBesideUnroll = 4;
 constexpr double kPaceShareOfLink = 0.84;
 // Share offered by a throughput-mode swap-out: the cap itself.
 constexpr double kThroughputShareOfLink = 0.90;
+constexpr uint64_t kPaceFromBytes = 256ull << 20;
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
@@ -333,20 +335,41 @@ void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, bool to_p
     }
 }
 
+// Where an address lives: 1 = host memory (pinned, device-mapped), 0 = device memory, -1 = the
+// runtime does not know the pointer.
+int memory_side(const void* p) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    if (attr.type == hipMemoryTypeHost) return 1;
+    if (attr.type == hipMemoryTypeDevice) return 0;
+    return -1;
+}
+
+// `packed_in_device` is what the caller knows for certain (the staged variant); otherwise the
+// runtime is asked where the packed pool lives.
 int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64_t* pairs, uint64_t n_pairs,
                      uint64_t packed_stride, uint64_t layered_stride, uint64_t packed_blocks,
                      uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
-                     bool to_packed, bool packed_is_host, uint32_t workgroups, hipStream_t s) {
-    // With the packed side in host memory the PCIe link is the bound and a small grid does.
-    if (workgroups == 0 && packed_is_host) {
-        workgroups = kTransferWorkgroups;
-    }
+                     bool to_packed, bool packed_in_device, uint32_t workgroups, hipStream_t s) {
     TransposeArgs a;
     uint32_t unit = 16;
     int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, packed, pairs, n_pairs, packed_stride, layered_stride,
                                  packed_blocks, layered_blocks, T, L, H, D, elem_bytes);
     if (rc != 0) return rc;
     if (a.n_work == 0) return HFK_OK;  // nothing to move
+    // With the packed side in host memory the PCIe link is the bound and a small grid does; an
+    // unknown pointer gets the small grid too. (Pacing, which gains a swap-out 1-2 %, does not pay
+    // here: the per-item address arithmetic makes a workgroup's service time shape-dependent, and
+    // one-head 128-byte-row shapes fall behind any schedule that helps the others.)
+    const int side = packed_in_device ? 0 : memory_side(packed);
+    if (workgroups == 0 && side != 0) {
+        // One block (the reference's op: 4-64 MiB, over in 0.1-1.2 ms) is sized for speed alone; a
+        // block table may run for many milliseconds beside other kernels and gets the smaller grid.
+        workgroups = pairs == nullptr ? kSingleBlockTransferWorkgroups : kTransferWorkgroups;
+    }
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
@@ -395,7 +418,7 @@ int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i
 int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* src_block, uint32_t T,
                                    uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
                                    uint32_t workgroups, hfk_stream_t stream) {
-    return launch_transpose(dev_layer_ptrs, src_block, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, true,
+    return launch_transpose(dev_layer_ptrs, src_block, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, false,
                             workgroups, static_cast<hipStream_t>(stream));
 }
 
@@ -410,7 +433,7 @@ int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs, cons
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipMemcpyAsync(staging, host_block, bytes, hipMemcpyHostToDevice, s);
     if (e != hipSuccess) return (int)e;
-    return launch_transpose(dev_layer_ptrs, staging, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, false,
+    return launch_transpose(dev_layer_ptrs, staging, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, true,
                             workgroups, s);
 }
 
@@ -424,7 +447,7 @@ int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t de
     if (block_pairs == nullptr) return HFK_ERR_NULL_POINTER;
     return launch_transpose(dev_layer_ptrs, packed_blocks, block_pairs, n_pairs, packed_block_stride,
                             dev_block_stride, n_packed_blocks, n_dev_blocks, T, L, H, D, elem_bytes, to_packed != 0,
-                            true, workgroups, static_cast<hipStream_t>(stream));
+                            false, workgroups, static_cast<hipStream_t>(stream));
 }
 
 int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* block_pairs,
@@ -457,10 +480,12 @@ int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, cons
     // Throughput mode. A swap is bound by the PCIe link, which a small grid saturates; more
     // workgroups only queue on the link.
     if (workgroups == 0) workgroups = (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
-    if ((flags & HFK_SWAP_DST_HOST) != 0) {
+    if ((flags & HFK_SWAP_DST_HOST) != 0 && (uint64_t)n_planes * n_pairs * block_bytes >= kPaceFromBytes) {
         // Toward the host the link accepts the most when it is offered exactly what it can take:
         // paced at its payload-efficiency cap the same grid sustains 56.8 GB/s where it reaches 55.4
         // unpaced, and should the cap be lower than assumed the launch degrades to the unpaced rate.
+        // A paced launch ends about 0.1 ms later than its schedule says, which only a long one amortises
+        // (32 MiB: 49 GB/s paced, 54.6 unpaced; 256 MiB: 56.0 against 55.6).
         const uint32_t pace_mbps = (uint32_t)(kThroughputShareOfLink * current_link_mbps());
         if (pace_mbps != 0) {
             return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, kBesideUnroll, pace_mbps);

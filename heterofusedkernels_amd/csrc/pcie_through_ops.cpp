@@ -201,11 +201,7 @@ void multi_layer_block_table_transfer(const at::Tensor& deviceLayerCachePtrs, co
     TORCH_CHECK(deviceBlocks >= 0, "deviceBlocks must be non-negative");
     if (blockPairs.size(0) == 0 || blockBytes == 0) return;
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(deviceLayerCachePtrs));
-    // The library's default grid is sized for a pool in host memory (the PCIe link saturates with
-    // few workgroups). A pool in device memory - the staging buffer of a DMA-staged transfer - is
-    // HBM-bound and wants one workgroup per chunk.
-    uint32_t cap = workgroup_cap(workgroups);
-    if (cap == 0 && hostBlockPool.is_cuda()) cap = 0x7fffffffu;
+    const uint32_t cap = workgroup_cap(workgroups);   // 0: the library sizes the grid for where the pool lives
     check_status(hfk_multi_layer_block_table_transfer(
                      deviceLayerCachePtrs.data_ptr(), static_cast<uint64_t>(deviceBlockStride),
                      device_visible(hostBlockPool, "hostBlockPool"), blockBytes,
