@@ -288,6 +288,9 @@ HFK_API int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host
  * i.e. hfk_gather_rows applied to every plane with a shared id list
  * (per plane: dst = src.index_select(0, ids)).
  * Same reference anchors as hfk_gather_rows; the plane loop is additive.
+ * The default grid (workgroups 0) is sized for planes in device memory; when the source planes
+ * are host memory this is a swap-in with consecutive destinations: pass workgroups 16, or use
+ * hfk_swap_blocks, whose flags pick the launch shape.
  */
 HFK_API int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs,
                       const int64_t* ids, uint32_t n_planes, uint64_t n_ids,
