@@ -3,6 +3,7 @@ strides larger than a block, bases off every alignment, planes on either side of
 link, int32 and int64 ids, out-of-range entries, random grid bounds. Each case checks the
 whole destination buffer, gaps between strided blocks included."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -22,6 +23,8 @@ BLOCK_BYTES = [1, 3, 16, 48, 100, 528, 4096, 4112, 12288, 32768, 33001]
 PADS = [0, 0, 16, 5, 4096]
 OFFSETS = [0, 0, 16, 4, 1, 7]
 CASES = 40
+# HFK_SWEEP_SEED_OFFSET=k shifts every seed by k: other cases of the same sweep, for longer one-off runs.
+SEED_OFFSET = int(os.environ.get("HFK_SWEEP_SEED_OFFSET", "0"))
 
 
 class Arena:
@@ -86,7 +89,7 @@ def _expect_swap(dst_buf, src_buf, doff, soff, n_planes, dst_blocks, src_blocks,
 
 @pytest.mark.parametrize("seed", range(4))
 def test_random_swap_blocks(seed):
-    rng = np.random.default_rng(1000 + seed)
+    rng = np.random.default_rng(1000 + seed + 17 * SEED_OFFSET)
     for case in range(CASES):
         n_planes = int(rng.integers(1, 9))
         src_blocks, dst_blocks = int(rng.integers(1, 40)), int(rng.integers(1, 40))
@@ -121,7 +124,7 @@ def test_random_swap_blocks(seed):
 
 @pytest.mark.parametrize("seed", range(4))
 def test_random_gather_rows_and_blocks(seed):
-    rng = np.random.default_rng(2000 + seed)
+    rng = np.random.default_rng(2000 + seed + 17 * SEED_OFFSET)
     for case in range(CASES):
         rows = int(rng.integers(1, 200))
         rb = int(rng.choice(BLOCK_BYTES + [7, 1000, 8212]))
@@ -170,7 +173,7 @@ def test_random_gather_rows_and_blocks(seed):
 
 @pytest.mark.parametrize("seed", range(4))
 def test_random_block_table_transfer(seed):
-    rng = np.random.default_rng(3000 + seed)
+    rng = np.random.default_rng(3000 + seed + 17 * SEED_OFFSET)
     for case in range(CASES):
         T, L, H = int(rng.integers(1, 40)), int(rng.integers(1, 6)), int(rng.integers(1, 5))
         D, e = int(rng.choice([1, 3, 8, 16, 24, 64, 128])), int(rng.choice([1, 2, 4]))
@@ -212,7 +215,7 @@ def test_random_block_table_transfer(seed):
 
 @pytest.mark.parametrize("seed", range(3))
 def test_random_duplex_and_staged(seed):
-    rng = np.random.default_rng(4000 + seed)
+    rng = np.random.default_rng(4000 + seed + 17 * SEED_OFFSET)
     for case in range(CASES):
         n_planes = int(rng.integers(1, 7))
         dev_blocks, host_blocks = int(rng.integers(4, 40)), int(rng.integers(4, 40))
