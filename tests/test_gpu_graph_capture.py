@@ -34,8 +34,9 @@ def test_swap_and_gather_replay_in_a_hip_graph():
     ids = torch.zeros(cfg.n_blocks, dtype=torch.int64, device=DEV)
 
     def run():
-        torch.ops.pcie_through.swap_blocks(htab, dtab, pairs_out, bb, bb, bb, cfg.dev_blocks, cfg.host_blocks)
-        torch.ops.pcie_through.swap_blocks(btab, htab, pairs_in, bb, bb, bb, cfg.host_blocks, cfg.dev_blocks)
+        # swap-out in the paced beside-compute shape (its schedule restarts with every replay), swap-in with its side named
+        torch.ops.pcie_through.swap_blocks(htab, dtab, pairs_out, bb, bb, bb, cfg.dev_blocks, cfg.host_blocks, None, 1 | 4)
+        torch.ops.pcie_through.swap_blocks(btab, htab, pairs_in, bb, bb, bb, cfg.host_blocks, cfg.dev_blocks, None, 2)
         torch.ops.pcie_through.gather_blocks(ptab, dtab, ids, bb, bb, cfg.dev_blocks)
 
     def set_inputs(seed):
