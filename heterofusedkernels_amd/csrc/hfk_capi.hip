@@ -122,6 +122,9 @@ std::atomic<int> g_link_mbps_override{-1};
 //    blocks that are whole 16 KiB chunks; other block sizes need 16.
 constexpr uint32_t kBesideWorkgroups = 8;
 constexpr int kBesideUnroll = 4;
+constexpr bool whole_beside_chunks(uint64_t block_bytes) {
+    return block_bytes % ((uint64_t)kWorkgroupLanes * 16u * kBesideUnroll) == 0;
+}
 // Share of the link's raw rate offered to host writes when pacing. 256-byte transaction payloads
 // cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured, reached only by a paced grid); from 0.92
 // on throughput collapses to 0.84 and the neighbours' slowdown doubles. The closer to the cap, the
@@ -472,8 +475,8 @@ int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, cons
             if (pace_mbps == 0) pace_mbps = (uint32_t)(kPaceShareOfLink * current_link_mbps());
         }
         if (workgroups == 0) {
-            const bool whole_chunks = block_bytes % ((uint64_t)kWorkgroupLanes * 16u * kBesideUnroll) == 0;
-            workgroups = ((flags & HFK_SWAP_SRC_HOST) != 0 && !whole_chunks) ? 2 * kBesideWorkgroups : kBesideWorkgroups;
+            workgroups = ((flags & HFK_SWAP_SRC_HOST) != 0 && !whole_beside_chunks(block_bytes)) ? 2 * kBesideWorkgroups
+                                                                                                : kBesideWorkgroups;
         }
         return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, kBesideUnroll, pace_mbps);
     }
@@ -492,8 +495,7 @@ int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, cons
         }
     }
     int unroll = g_swap_unroll.load(std::memory_order_relaxed);
-    if ((flags & HFK_SWAP_SRC_HOST) != 0 && block_bytes % ((uint64_t)kWorkgroupLanes * 16u * kBesideUnroll) == 0 &&
-        unroll > kBesideUnroll) {
+    if ((flags & HFK_SWAP_SRC_HOST) != 0 && whole_beside_chunks(block_bytes) && unroll > kBesideUnroll) {
         // From the host, blocks that are whole 16 KiB chunks reach the link rate with half as much in
         // flight (57.6 GB/s either way; a memory-bound neighbour 1.3-1.7x slower instead of 2.3-2.4x).
         unroll = kBesideUnroll;
