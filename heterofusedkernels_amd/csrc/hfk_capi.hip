@@ -249,7 +249,8 @@ int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, 
                       uint32_t pace_mbps = 0) {
     int unroll = 1;
     if (preferred_unroll == 0) preferred_unroll = g_unroll.load(std::memory_order_relaxed);
-    int rc = hfk::plan_block_copy<IdT>(a, preferred_unroll, &unroll);
+    // Everything but the swap runs one workgroup per chunk and wants whole chunks.
+    int rc = hfk::plan_block_copy<IdT>(a, preferred_unroll, &unroll, ROLE != Role::kSwapBlocks);
     if (rc != 0) return rc;
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);

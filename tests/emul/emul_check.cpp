@@ -74,9 +74,9 @@ void walk(const Args& a, uint32_t grid, Body body) {
 }
 
 template <typename IdT, int NT>
-void run_block_copy(BlockCopyArgs<IdT> a, int preferred_unroll, uint32_t grid_cap) {
-    int unroll = 1;
-    if (plan_block_copy<IdT>(a, preferred_unroll, &unroll) != HFK_OK) { std::printf("plan failed\n"); ++g_failures; return; }
+void run_block_copy(BlockCopyArgs<IdT> a, int preferred_unroll, uint32_t grid_cap, bool whole_chunks = false) {
+    int unroll = 1;   // whole_chunks: as the launcher plans every role but the swap
+    if (plan_block_copy<IdT>(a, preferred_unroll, &unroll, whole_chunks) != HFK_OK) { std::printf("plan failed\n"); ++g_failures; return; }
     const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
     switch (unroll) {
         case 1: walk(a, grid, block_copy_body<IdT, 1, NT>); break;
@@ -300,7 +300,7 @@ void case_gather_blocks(uint32_t n_planes, uint32_t n_ids, uint64_t block_bytes,
     int rc = plan_gather_blocks(a, dp.data(), sp.data(), ids.data(), n_planes, n_ids, block_bytes, block_bytes, src_blocks);
     if (rc != HFK_OK) { ++g_failures; std::printf("plan_gather_blocks rc=%d\n", rc); }
     else {
-        run_block_copy<int64_t, 0>(a, unroll, grid_cap);
+        run_block_copy<int64_t, 0>(a, unroll, grid_cap, true);
         char what[128];
         std::snprintf(what, sizeof what, "gather_blocks planes=%u ids=%u bytes=%llu unroll=%d grid=%u", n_planes, n_ids,
                       (unsigned long long)block_bytes, unroll, grid_cap);
@@ -331,7 +331,7 @@ void case_gather_rows(uint64_t table_rows, uint64_t n_ids, uint64_t row_bytes, s
     if (row_bytes >= kWideRowBytes) {
         BlockCopyArgs<IdT> a;
         if (plan_wide_gather<IdT>(a, table.p, dst.p, ids.data(), n_ids, row_bytes, table_rows) != HFK_OK) { ++g_failures; return; }
-        run_block_copy<IdT, 3>(a, unroll, grid_cap);
+        run_block_copy<IdT, 3>(a, unroll, grid_cap, true);
     } else {
         run_flat_gather<IdT>((uint64_t)(uintptr_t)table.p, (uint64_t)(uintptr_t)dst.p, ids.data(), n_ids, row_bytes,
                              table_rows, grid_cap, force64);
