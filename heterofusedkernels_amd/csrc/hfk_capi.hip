@@ -258,8 +258,8 @@ int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, 
     if (pace_mbps != 0) {
         // bytes per work item (average over a block) * workgroups / rate, in 1/256 ticks of 10 ns
         const double item_bytes = (double)a.block_bytes / a.chunks_per_block;
-        const double ticks = item_bytes * grid / ((double)pace_mbps * 1e6) * 1e8;
-        a.pace_q8 = (uint32_t)(ticks * 256.0 + 0.5);
+        const double q8 = item_bytes * grid / ((double)pace_mbps * 1e6) * 1e8 * 256.0 + 0.5;
+        a.pace_q8 = q8 < 4294967295.0 ? (uint32_t)q8 : 0xffffffffu;   // absurdly low rates: the wait's spin limit rules
     }
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
     switch (unroll) {
