@@ -253,7 +253,7 @@ HFK_API int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_blo
  * it (GEMM, device copy and attention kernels: 0.98-1.04x on MI355X), because the PCIe leg is
  * DMA and the kernel is short. A swap whose compute units touch host memory costs its neighbours
  * 1.06-1.3x at best (hfk_swap_blocks with HFK_SWAP_BESIDE_COMPUTE) and any long-resident kernel
- * costs a GEMM that exactly fills the CUs a whole extra round of tiles (1.5x). Use this entry
+ * costs a large GEMM about 1.5x whatever it does (the GEMM's workgroups want whole CUs). Use this entry
  * point when the swap overlaps compute and its host slots are mostly consecutive; hfk_swap_blocks
  * when they are scattered, when no staging buffer can be spared, or when the GPU is otherwise idle.
  *
