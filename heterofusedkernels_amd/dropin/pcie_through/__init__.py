@@ -2,6 +2,11 @@ from ._load import _load_opextension_so
 
 _load_opextension_so()
 
+# flags of torch.ops.pcie_through.swap_blocks (hfk.h: HFK_SWAP_*)
+SWAP_DST_HOST = 1        # the destination planes are host memory (swap-out)
+SWAP_SRC_HOST = 2        # the source planes are host memory (swap-in)
+SWAP_BESIDE_COMPUTE = 4  # other kernels run at the same time: small, paced launch
+
 
 def plane_pointer_table(planes, device):
     """int64 device tensor of kernel-usable base addresses, one per plane.

@@ -117,6 +117,14 @@ def test_op_schemas_match_reference():
     assert hasattr(torch.ops.pcie_through, "swap_blocks") and hasattr(torch.ops.pcie_through, "gather_blocks")
 
 
+def test_flag_constants_match_the_header():
+    import pcie_through
+    text = open(os.path.join(ROOT, "include", "hfk.h")).read()
+    for name in ("SWAP_DST_HOST", "SWAP_SRC_HOST", "SWAP_BESIDE_COMPUTE"):
+        value = int(re.search(r"#define HFK_%s (\d+)u" % name, text).group(1))
+        assert getattr(pcie_through, name) == value == getattr(capi, name)
+
+
 def test_ops_have_no_cpu_fallback():
     import pcie_through  # noqa: F401
 
