@@ -4,11 +4,12 @@ Artefacts (all in-tree, git-ignored):
 
     dropin/pcie_through/lib/libhfk_hip.so        gfx950 kernels + C-ABI (hipcc)
     dropin/pcie_through/lib/libpcie_through.so   torch dispatcher ops
-    dropin/pcie_through/lib/libhfk_bench.so      benchmark-only comparison paths
     dropin/heterofusedkernels/libmanaged_memory.so   host-memory registry + allocator
     dropin/heterofusedkernels/memory*.so         Python module heterofusedkernels.memory
     dropin/heterofusedkernels/include/*.h        headers shipped for native users
     bin/hfk_c_client                             plain-C99 client of the C-ABI (csrc/examples)
+    bin/libhfk_bench.so                          benchmark-only comparison paths and yardstick kernels
+                                                 (outside the packages: never installed)
 
 Run as ``python -m heterofusedkernels_amd._build`` or through ``build_all()``.
 """
@@ -31,7 +32,7 @@ GPU_ARCH = "gfx950"
 
 HFK_HIP_SO = os.path.join(PCIE_LIB, "libhfk_hip.so")
 PCIE_THROUGH_SO = os.path.join(PCIE_LIB, "libpcie_through.so")
-HFK_BENCH_SO = os.path.join(PCIE_LIB, "libhfk_bench.so")
+HFK_BENCH_SO = os.path.join(PKG, "bin", "libhfk_bench.so")
 MANAGED_MEMORY_SO = os.path.join(COMMON, "libmanaged_memory.so")
 MEMORY_EXT_SO = os.path.join(COMMON, "memory" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 C_CLIENT = os.path.join(PKG, "bin", "hfk_c_client")
@@ -65,14 +66,17 @@ def build_hfk_hip():
 
 
 def build_bench_support():
-    """Comparison paths used by bench.py only (per-block hipMemcpyAsync loop)."""
-    os.makedirs(PCIE_LIB, exist_ok=True)
+    """Comparison paths used by bench.py only (per-block hipMemcpyAsync loop, HBM read / write / copy
+    yardstick kernels of the gather's shape). Built beside the C client, not into a package."""
+    os.makedirs(os.path.dirname(HFK_BENCH_SO), exist_ok=True)
     _run(
         [
-            "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-D__HIP_PLATFORM_AMD__=1",
-            "-I" + os.path.join(ROCM, "include"), os.path.join(CSRC, "bench_support.cpp"), "-o", HFK_BENCH_SO,
-            "-L" + os.path.join(ROCM, "lib"), "-lamdhip64",
-        ]
+            os.path.join(ROCM, "bin", "hipcc"), "--offload-arch=" + GPU_ARCH, "-O3", "-std=c++17", "-fPIC",
+            "-shared", "-fvisibility=hidden", "-Wall",
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+            "-I" + INCLUDE, "-I" + CSRC, os.path.join(CSRC, "bench_support.hip"), "-o", HFK_BENCH_SO,
+        ],
+        quiet_patterns=("packed-fp32-ops' is not a recognized feature",),
     )
 
 

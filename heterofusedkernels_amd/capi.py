@@ -19,6 +19,11 @@ KNOB_DUPLEX_UNROLL = 4
 KNOB_SWAP_UNROLL = 5
 KNOB_SWAP_PACE_MBPS = 6
 KNOB_LINK_MBPS = 7
+KNOB_DUPLEX_WORKGROUPS = 8
+KNOB_THROUGHPUT_PACE_PERMILLE = 9
+KNOB_HBM_LDS_BYTES = 10
+KNOB_PACED_UNROLL = 11
+KNOB_PACED_WORKGROUPS = 12
 SWAP_DST_HOST = 1
 SWAP_SRC_HOST = 2
 SWAP_BESIDE_COMPUTE = 4
@@ -41,6 +46,7 @@ ENTRY_POINTS = (
     "hfk_swap_blocks",
     "hfk_swap_blocks_duplex",
     "hfk_swap_blocks_staged",
+    "hfk_swap_blocks_auto",
     "hfk_gather_blocks",
     "hfk_set_tuning",
     "hfk_get_tuning",
@@ -87,15 +93,17 @@ def load():
     L.hfk_fused_memcpy_multi_layer_block_transfer.argtypes = [vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
     L.hfk_fused_memcpy_multi_layer_block_transfer.restype = ci
     L.hfk_multi_layer_block_table_transfer.argtypes = [vp, u64, vp, u64, vp, u64, u64, u64, u32, u32, u32, u32, u32, ci,
-                                                       u32, vp]
+                                                       u32, u32, vp]
     L.hfk_multi_layer_block_table_transfer.restype = ci
     L.hfk_swap_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, u32, u32, vp]
     L.hfk_swap_blocks.restype = ci
-    L.hfk_swap_blocks_duplex.argtypes = [ctypes.POINTER(BlockMove), ctypes.POINTER(BlockMove), u32, u64, u32, vp]
+    L.hfk_swap_blocks_duplex.argtypes = [ctypes.POINTER(BlockMove), ctypes.POINTER(BlockMove), u32, u64, u32, u32, vp]
     L.hfk_swap_blocks_duplex.restype = ci
     L.hfk_swap_blocks_staged.argtypes = [vp, vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, vp, ci, u32, vp]
     L.hfk_swap_blocks_staged.restype = ci
-    L.hfk_gather_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u32, vp]
+    L.hfk_swap_blocks_auto.argtypes = [vp, vp, vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, vp, u64, ci, u32, u32, vp]
+    L.hfk_swap_blocks_auto.restype = ci
+    L.hfk_gather_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u32, u32, vp]
     L.hfk_gather_blocks.restype = ci
     L.hfk_set_tuning.argtypes = [ci, i64]
     L.hfk_set_tuning.restype = ci
@@ -131,11 +139,11 @@ def fused_memcpy_multi_layer_block_transfer(layer_ptrs, host_block, staging, T, 
 
 def multi_layer_block_table_transfer(layer_ptrs, dev_block_stride, packed_blocks, packed_block_stride, pairs, n_pairs,
                                      n_packed_blocks, n_dev_blocks, T, L, H, D, elem_bytes, to_packed, workgroups=0,
-                                     stream=0):
+                                     stream=0, flags=0):
     return load().hfk_multi_layer_block_table_transfer(layer_ptrs, dev_block_stride, packed_blocks,
                                                        packed_block_stride, pairs, n_pairs, n_packed_blocks,
                                                        n_dev_blocks, T, L, H, D, elem_bytes, int(bool(to_packed)),
-                                                       workgroups, stream)
+                                                       flags, workgroups, stream)
 
 
 def swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, src_stride, dst_stride,
@@ -144,11 +152,11 @@ def swap_blocks(dst_planes, src_planes, pairs, n_planes, n_pairs, block_bytes, s
                                   dst_stride, src_blocks, dst_blocks, flags, workgroups, stream)
 
 
-def swap_blocks_duplex(out_move, in_move, n_planes, block_bytes, workgroups=0, stream=0):
+def swap_blocks_duplex(out_move, in_move, n_planes, block_bytes, workgroups=0, stream=0, flags=0):
     """out_move / in_move: BlockMove instances or None."""
     return load().hfk_swap_blocks_duplex(ctypes.byref(out_move) if out_move is not None else None,
                                          ctypes.byref(in_move) if in_move is not None else None, n_planes, block_bytes,
-                                         workgroups, stream)
+                                         flags, workgroups, stream)
 
 
 def swap_blocks_staged(dev_planes, host_plane_addrs, dev_ids, host_ids, n_planes, n_blocks, block_bytes, dev_stride,
@@ -159,10 +167,19 @@ def swap_blocks_staged(dev_planes, host_plane_addrs, dev_ids, host_ids, n_planes
                                          int(bool(to_host)), workgroups, stream)
 
 
+def swap_blocks_auto(dev_planes, host_planes_mapped, host_plane_addrs, pairs, host_ids, n_planes, n_pairs, block_bytes,
+                     dev_stride, host_stride, dev_blocks, host_blocks, staging, staging_bytes, to_host,
+                     min_run_blocks=0, flags=0, stream=0):
+    """host_plane_addrs / host_ids: addresses of HOST arrays or None; pairs: device [n, 2] (src, dst)."""
+    return load().hfk_swap_blocks_auto(dev_planes, host_planes_mapped, host_plane_addrs, pairs, host_ids, n_planes,
+                                       n_pairs, block_bytes, dev_stride, host_stride, dev_blocks, host_blocks, staging,
+                                       staging_bytes, int(bool(to_host)), min_run_blocks, flags, stream)
+
+
 def gather_blocks(dst_planes, src_planes, ids, n_planes, n_ids, block_bytes, src_stride, src_blocks=0,
-                  workgroups=0, stream=0):
+                  workgroups=0, stream=0, flags=0):
     return load().hfk_gather_blocks(dst_planes, src_planes, ids, n_planes, n_ids, block_bytes, src_stride,
-                                    src_blocks, workgroups, stream)
+                                    src_blocks, flags, workgroups, stream)
 
 
 def set_tuning(knob, value):

@@ -79,6 +79,23 @@ struct Pacer {
     }
 };
 
+// Block tables and plane-address tables are read, never written, by the kernel that uses them, and
+// every lane of a workgroup reads the same entry. Reading them through the constant address space
+// tells the compiler both facts, so it uses scalar loads: they are counted apart from the vector
+// loads and stores, and a table lookup no longer waits for the workgroup's outstanding stores to
+// drain (which, toward host memory, takes microseconds and sits on the critical path of a
+// workgroup that keeps little in flight).
+#if defined(__HIP_DEVICE_COMPILE__)
+#define HFK_CONSTANT __attribute__((address_space(4)))
+#else
+#define HFK_CONSTANT
+#endif
+
+template <typename T>
+HFK_HD T table_entry(const T* table, uint64_t index) {
+    return reinterpret_cast<const HFK_CONSTANT T*>(reinterpret_cast<uint64_t>(table))[index];
+}
+
 // NT bit0: non-temporal loads, bit1: non-temporal stores.
 template <typename V>
 HFK_HD const HFK_GLOBAL V* global_in(uint64_t addr) {
@@ -143,28 +160,127 @@ struct BlockCopyArgs {
     uint64_t dst_limit;          // so negative ids are rejected as well)
     uint32_t n_work;             // n_planes * n_pairs * chunks_per_block
     uint32_t pace_q8;            // see Pacer; 0 = unpaced
+    uint32_t zero_skipped;       // != 0: a pair whose source index is out of range but whose destination is
+                                 // valid gets zeros written instead of being left alone (a staging buffer
+                                 // must never hand an earlier transfer's bytes on to the host)
+    // Run filter (RunFilter below): lets one block table be split between two movers, by the length
+    // of the run of consecutive `run_ids` a pair belongs to. run_mode 0 = every pair.
+    uint32_t run_mode;
+    uint32_t run_min;            // a run is "long" from this many consecutive ids on
+    const int64_t* run_ids;      // entry j at run_ids[j * id_stride]
 };
 
+// Which pairs of a block table a launch moves, when the table is split by run length: pair j belongs to
+// the maximal run of entries whose run_ids are consecutive (ids[i + 1] == ids[i] + 1) around it.
+enum RunFilter : uint32_t { kAllPairs = 0, kLongRunsOnly = 1, kShortRunsOnly = 2 };
+
+// Length of the maximal run of consecutive ids around entry j, counted no further than `cap`: the
+// result is min(cap, run length). The host uses the same function to decide which runs it copies,
+// so the two sides of a split table agree by construction.
+HFK_HD uint32_t run_length_capped(const int64_t* ids, uint32_t stride, uint32_t n, uint32_t j, uint32_t cap) {
+    uint32_t len = 1;
+    for (uint32_t i = j; i > 0 && len < cap &&
+                         table_entry(ids, (uint64_t)(i - 1) * stride) + 1 == table_entry(ids, (uint64_t)i * stride); --i) {
+        ++len;
+    }
+    for (uint32_t i = j; i + 1 < n && len < cap &&
+                         table_entry(ids, (uint64_t)(i + 1) * stride) == table_entry(ids, (uint64_t)i * stride) + 1; ++i) {
+        ++len;
+    }
+    return len;
+}
+
 // Where work item w of a block copy reads and writes. Everything here is uniform
-// over the workgroup, so the compiler keeps it in scalar registers. Returns false
-// when the item's block indices are out of range (the item is skipped).
-template <typename IdT>
-HFK_HD bool resolve_chunk(const BlockCopyArgs<IdT>& a, uint32_t w, uint64_t& s_addr, uint64_t& d_addr,
-                          uint32_t& chunk) {
+// over the workgroup, so the compiler keeps it in scalar registers. Returns kSkip
+// when the item's block indices are out of range or the run filter leaves the pair
+// to another mover, kZeroFill when only the source index is out of range and the
+// launch asked for zeros in that case (d_addr is then valid), kCopy otherwise.
+enum ChunkAction : uint32_t { kSkip = 0, kCopy = 1, kZeroFill = 2 };
+
+// SPLIT selects, at compile time, the variant that honours the run filter; kernels that move whole
+// tables (the hot ones) are built without it and carry none of its code.
+template <typename IdT, bool SPLIT = false>
+HFK_HD ChunkAction resolve_chunk(const BlockCopyArgs<IdT>& a, uint32_t w, uint64_t& s_addr, uint64_t& d_addr,
+                                 uint32_t& chunk) {
     chunk = w % a.chunks_per_block;
     const uint32_t tile = w / a.chunks_per_block;
-    const uint32_t pair = tile % a.n_pairs;
-    const uint32_t plane = tile / a.n_pairs;
-    const uint64_t sb = a.src_ids ? (uint64_t)(int64_t)a.src_ids[(uint64_t)pair * a.id_stride] : (uint64_t)pair;
-    const uint64_t db = a.dst_ids ? (uint64_t)(int64_t)a.dst_ids[(uint64_t)pair * a.id_stride] : (uint64_t)pair;
-    if (sb >= a.src_limit || db >= a.dst_limit) {
-        return false;
+    uint32_t pair, plane;
+    if constexpr (!SPLIT) {             // plane-major: neighbouring workgroups stream neighbouring pairs of one plane
+        pair = tile % a.n_pairs;
+        plane = tile / a.n_pairs;
+    } else {                            // pair-major: all items of a pair are adjacent, so a filtered-out
+        pair = tile / a.n_planes;       // pair is stepped over at once (next_pair_item); the filter itself
+        plane = tile % a.n_planes;      // is the caller's business (pair_selected), once per pair
     }
-    s_addr = (a.src_planes ? a.src_planes[plane] : a.src_base + (uint64_t)plane * a.src_plane_stride) +
-             sb * a.src_stride;
-    d_addr = (a.dst_planes ? a.dst_planes[plane] : a.dst_base + (uint64_t)plane * a.dst_plane_stride) +
-             db * a.dst_stride;
-    return true;
+    // The four table reads (two block indices, two plane addresses) do not depend on one another and
+    // none can fault (pair < n_pairs, plane < n_planes): they are all issued before the first
+    // comparison, so a work item pays one scalar-load latency, not a chain of them. A workgroup that
+    // keeps little in flight (the duplex swap: one vector per lane and direction) is as fast as its
+    // iterations are short.
+    const uint64_t sb = a.src_ids ? (uint64_t)(int64_t)table_entry(a.src_ids, (uint64_t)pair * a.id_stride) : (uint64_t)pair;
+    const uint64_t db = a.dst_ids ? (uint64_t)(int64_t)table_entry(a.dst_ids, (uint64_t)pair * a.id_stride) : (uint64_t)pair;
+    const uint64_t s_plane = a.src_planes ? table_entry(a.src_planes, plane) : a.src_base + (uint64_t)plane * a.src_plane_stride;
+    const uint64_t d_plane = a.dst_planes ? table_entry(a.dst_planes, plane) : a.dst_base + (uint64_t)plane * a.dst_plane_stride;
+    s_addr = s_plane + sb * a.src_stride;
+    d_addr = d_plane + db * a.dst_stride;
+    if (db >= a.dst_limit) {
+        return kSkip;
+    }
+    if (sb >= a.src_limit) {
+        return a.zero_skipped != 0 ? kZeroFill : kSkip;
+    }
+    return kCopy;
+}
+
+// Whether the launch's run filter leaves pair `pair` to this launch.
+template <typename IdT>
+HFK_HD bool pair_selected(const BlockCopyArgs<IdT>& a, uint32_t pair) {
+    const bool is_long = run_length_capped(a.run_ids, a.id_stride, a.n_pairs, pair, a.run_min) >= a.run_min;
+    return is_long == (a.run_mode == kLongRunsOnly);
+}
+
+// In pair-major order (run filter on), the first work item after w that belongs to workgroup `bid`
+// of `nb` (items bid, bid + nb, ...) and to a later pair than w does.
+template <typename IdT>
+HFK_HD uint64_t next_pair_item(const BlockCopyArgs<IdT>& a, uint64_t w, uint32_t bid, uint32_t nb) {
+    const uint64_t per_pair = (uint64_t)a.n_planes * a.chunks_per_block;
+    const uint64_t first = (w / per_pair + 1) * per_pair;             // first item of the next pair
+    return first + ((uint64_t)bid + nb - first % nb) % nb;            // >= first, congruent to bid mod nb
+}
+
+// U loads, then U stores, 256 vectors apart: the straight-line core of every copy.
+template <int U, int NT>
+HFK_HD void copy_steps(const HFK_GLOBAL vec16* sv, HFK_GLOBAL vec16* dv) {
+    vec16 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
+    }
+}
+
+// The last, short chunk of a block: `remaining` (< 2 * U * 256, uniform over the workgroup) vectors
+// from sv/dv on (which already include the lane's offset). Cut into pieces of U, U/2, ... 1 full
+// steps and one guarded step, each piece straight-line code with its loads ahead of its stores, so a
+// tail needs no more registers than a full chunk and all branches but the last are uniform.
+template <int U, int NT>
+HFK_HD void copy_tail(const HFK_GLOBAL vec16* sv, HFK_GLOBAL vec16* dv, uint64_t remaining, uint32_t tid) {
+    if (remaining >= (uint64_t)U * kWorkgroupLanes) {
+        copy_steps<U, NT>(sv, dv);
+        sv += U * kWorkgroupLanes;
+        dv += U * kWorkgroupLanes;
+        remaining -= (uint64_t)U * kWorkgroupLanes;
+    }
+    if constexpr (U > 1) {
+        copy_tail<U / 2, NT>(sv, dv, remaining, tid);
+    } else {
+        if (tid < remaining) {
+            store_unit<NT>(dv, load_unit<NT>(sv));
+        }
+    }
 }
 
 // Copies chunk `chunk` (256 * UNROLL vectors) of one block of block_bytes bytes.
@@ -177,30 +293,10 @@ HFK_HD void copy_chunk(uint64_t s_addr, uint64_t d_addr, uint64_t block_bytes, u
         const uint64_t first = (uint64_t)chunk * kChunkVecs;
         const HFK_GLOBAL vec16* sv = global_in<vec16>(s_addr) + first + tid;
         HFK_GLOBAL vec16* dv = global_out<vec16>(d_addr) + first + tid;
-        vec16 v[UNROLL];
         if (first + kChunkVecs <= block_vecs) {
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
-            }
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
-            }
-        } else {
-            const uint64_t lane_first = first + tid;
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
-                    v[u] = load_unit<NT>(sv + u * kWorkgroupLanes);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
-                    store_unit<NT>(dv + u * kWorkgroupLanes, v[u]);
-                }
-            }
+            copy_steps<UNROLL, NT>(sv, dv);
+        } else if (first < block_vecs) {
+            copy_tail<(UNROLL > 1 ? UNROLL / 2 : 1), NT>(sv, dv, block_vecs - first, tid);
         }
     } else {
         // Blocks that are not 16-byte aligned/sized: same chunk, narrower units.
@@ -222,17 +318,66 @@ HFK_HD void copy_chunk(uint64_t s_addr, uint64_t d_addr, uint64_t block_bytes, u
     }
 }
 
-template <typename IdT, int UNROLL, int NT>
+// Writes zeros over chunk `chunk` of one block (same chunking as copy_chunk).
+template <int UNROLL, int NT>
+HFK_HD void zero_chunk(uint64_t d_addr, uint64_t block_bytes, uint32_t chunk, uint32_t tid) {
+    constexpr uint32_t kChunkVecs = kWorkgroupLanes * UNROLL;
+    constexpr uint64_t kChunkBytes = (uint64_t)kChunkVecs * 16u;
+    if (((d_addr | block_bytes) & 15u) == 0) {
+        const uint64_t block_vecs = block_bytes >> 4;
+        const uint64_t lane_first = (uint64_t)chunk * kChunkVecs + tid;
+        HFK_GLOBAL vec16* dv = global_out<vec16>(d_addr) + lane_first;
+        const vec16 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (lane_first + (uint64_t)u * kWorkgroupLanes < block_vecs) {
+                store_unit<NT>(dv + u * kWorkgroupLanes, zero);
+            }
+        }
+    } else {
+        const uint64_t lo = (uint64_t)chunk * kChunkBytes;
+        const uint64_t hi = (lo + kChunkBytes < block_bytes) ? lo + kChunkBytes : block_bytes;
+        HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(d_addr);
+        for (uint64_t o = lo + tid; o < hi; o += kWorkgroupLanes) {
+            d1[o] = 0;
+        }
+    }
+}
+
+// SPLIT: the launch moves only the pairs its run filter selects (a.run_mode must then be
+// kLongRunsOnly or kShortRunsOnly); without it a.run_mode must be kAllPairs.
+template <typename IdT, int UNROLL, int NT, bool SPLIT = false>
 HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
     Pacer pacer(a.pace_q8, bid, nb);
-    for (uint32_t w = bid; w < a.n_work; w += nb) {
-        pacer.wait_turn();
+    uint64_t w = bid;                   // 64-bit so that w + nb cannot wrap
+    uint32_t judged_pair = 0xffffffffu; // SPLIT: the pair the filter was last evaluated for, and its verdict
+    bool judged_selected = false;       // (a workgroup's consecutive items mostly belong to one pair)
+    while (w < a.n_work) {
         uint64_t s_addr = 0, d_addr = 0;
         uint32_t chunk = 0;
-        if (!resolve_chunk(a, w, s_addr, d_addr, chunk)) {
+        if constexpr (SPLIT) {
+            const uint32_t pair = (uint32_t)(w / ((uint64_t)a.n_planes * a.chunks_per_block));
+            if (pair != judged_pair) {
+                judged_pair = pair;
+                judged_selected = pair_selected(a, pair);
+            }
+            if (!judged_selected) {
+                w = next_pair_item(a, w, bid, nb);
+                continue;
+            }
+        }
+        const ChunkAction what = resolve_chunk<IdT, SPLIT>(a, (uint32_t)w, s_addr, d_addr, chunk);
+        if (what == kSkip) {            // moves nothing, so it takes no turn on the link either
+            w = SPLIT ? next_pair_item(a, w, bid, nb) : w + nb;
             continue;
         }
-        copy_chunk<UNROLL, NT>(s_addr, d_addr, a.block_bytes, chunk, tid);
+        pacer.wait_turn();
+        if (what == kCopy) {
+            copy_chunk<UNROLL, NT>(s_addr, d_addr, a.block_bytes, chunk, tid);
+        } else {
+            zero_chunk<UNROLL, NT>(d_addr, a.block_bytes, chunk, tid);
+        }
+        w += nb;
     }
 }
 
@@ -250,16 +395,20 @@ struct DuplexCopyArgs {
     BlockCopyArgs<int64_t> first;
     BlockCopyArgs<int64_t> second;
     uint32_t n_work;  // max(first.n_work, second.n_work)
+    uint32_t pace_q8; // see Pacer: one turn per iteration (one chunk of each copy); 0 = unpaced
 };
 
 template <int UNROLL, int NT>
 HFK_HD void duplex_copy_body(const DuplexCopyArgs& a, uint32_t bid, uint32_t nb, uint32_t tid) {
     constexpr uint32_t kChunkVecs = kWorkgroupLanes * UNROLL;
-    for (uint32_t w = bid; w < a.n_work; w += nb) {
+    Pacer pacer(a.pace_q8, bid, nb);
+    for (uint64_t w64 = bid; w64 < a.n_work; w64 += nb) {   // 64-bit counter: w + nb cannot wrap
+        const uint32_t w = (uint32_t)w64;
+        pacer.wait_turn();
         uint64_t s0 = 0, d0 = 0, s1 = 0, d1 = 0;
         uint32_t c0 = 0, c1 = 0;
-        const bool v0 = w < a.first.n_work && resolve_chunk(a.first, w, s0, d0, c0);
-        const bool v1 = w < a.second.n_work && resolve_chunk(a.second, w, s1, d1, c1);
+        const bool v0 = w < a.first.n_work && resolve_chunk(a.first, w, s0, d0, c0) == kCopy;
+        const bool v1 = w < a.second.n_work && resolve_chunk(a.second, w, s1, d1, c1) == kCopy;
         const bool fast0 = v0 && ((s0 | d0 | a.first.block_bytes) & 15u) == 0 &&
                            ((uint64_t)c0 + 1) * kChunkVecs <= (a.first.block_bytes >> 4);
         const bool fast1 = v1 && ((s1 | d1 | a.second.block_bytes) & 15u) == 0 &&
@@ -320,7 +469,8 @@ HFK_HD void flat_gather_body(const FlatGatherArgs<IdT>& a, uint32_t bid, uint32_
     const IndexT total = (IndexT)a.total_units;
     const IndexT row_units = (IndexT)a.row_units;
 
-    for (uint32_t w = bid; w < a.n_work; w += nb) {
+    for (uint64_t w64 = bid; w64 < a.n_work; w64 += nb) {
+        const uint32_t w = (uint32_t)w64;
         const IndexT g0 = (IndexT)w * kChunkUnits + tid;
         V v[UNROLL];
         bool ok[UNROLL];
@@ -393,11 +543,12 @@ HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, ui
     constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
     const uint32_t LH = a.L * a.H;
 
-    for (uint32_t w = bid; w < a.n_work; w += nb) {
+    for (uint64_t w64 = bid; w64 < a.n_work; w64 += nb) {
+        const uint32_t w = (uint32_t)w64;
         const uint32_t chunk = w % a.chunks_per_block;
         const uint32_t pair = w / a.chunks_per_block;
-        const uint64_t pb = a.pairs ? (uint64_t)a.pairs[2 * (uint64_t)pair] : 0;
-        const uint64_t db = a.pairs ? (uint64_t)a.pairs[2 * (uint64_t)pair + 1] : 0;
+        const uint64_t pb = a.pairs ? (uint64_t)table_entry(a.pairs, 2 * (uint64_t)pair) : 0;
+        const uint64_t db = a.pairs ? (uint64_t)table_entry(a.pairs, 2 * (uint64_t)pair + 1) : 0;
         if (pb >= a.packed_limit || db >= a.layered_limit) {
             continue;
         }

@@ -20,6 +20,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <type_traits>
 
 #include "hfk.h"
 #include "hfk_bodies.h"
@@ -38,6 +39,23 @@ using hfk::vec16;
 // block gather, the scatter out of a staging buffer and wide-row gathers, and a
 // profile should say which one ran.
 enum class Role { kSwapBlocks, kGatherBlocks, kGatherRows, kScatterBlocks };
+
+// The same three, restricted by the run filter to one share of a table that is split between the
+// copy engines and the compute units (hfk_swap_blocks_auto).
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void swap_short_runs_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void gather_long_runs_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void scatter_long_runs_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
 
 template <int UNROLL, int NT>
 __global__ __launch_bounds__(256) void swap_blocks_kernel(const BlockCopyArgs<int64_t> a) {
@@ -83,56 +101,80 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
 
 // ---- tuning state ---------------------------------------------------------
 // Defaults are the measured best on MI355X:
-//  * 8 x 16 B in flight per lane and non-temporal loads + stores: +15-20 % HBM copy
-//    bandwidth over plain accesses (5.1 -> 6.1 TB/s; the data is touched once).
-//  * HBM-bound launches want one workgroup per chunk (a grid-stride loop over fewer
-//    workgroups lost 5-10 %), so the bound is set high enough to be inactive up to
-//    256 Ki chunks; beyond that the loop takes over.
+//  * HBM-bound launches (gathers, the staged swap's kernel): ONE 16-byte vector per lane, i.e. 4 KiB
+//    per workgroup, one workgroup per chunk, non-temporal loads and stores. A compute unit holds 8
+//    such workgroups (32 KiB in flight per unit, 8 MiB on the chip), and the finer the chunks, the
+//    more evenly the traffic spreads: 6.28-6.36 TB/s on 32 KiB blocks where 8 vectors per lane
+//    reach 5.5-6.0, 6.5-6.6 TB/s on 72 KiB and 16 KiB blocks (with more in flight per lane the best
+//    rate needs the resident workgroups bounded to about 48 KiB per unit, HFK_KNOB_HBM_LDS_BYTES,
+//    and stays below this one). A grid-stride loop over fewer workgroups loses 5-10 %, so the grid
+//    bound is high enough to stay inactive (CUs x 65536 workgroups).
+//  * non-temporal accesses: +15-20 % over plain ones (the data is touched once).
 //  * PCIe-bound swaps are flat from 16 to 128 workgroups (55.4-55.7 GB/s out, 57.0-57.4 in);
 //    what grows with the grid is the harm to kernels on other streams (a memory-bound
 //    neighbour runs 2.3-3x slower beside 16 workgroups, 4-5.7x beside 64), so a swap
 //    defaults to 16. For the same reason the duplex swap defaults to 32 workgroups (98.2 GB/s
 //    summed against 99.1 at 128, neighbours 1.1-1.6x slower instead of 2.8-2.9x) and the
 //    block-table transfers to 48 (-1 %, neighbours 1.8-2.5x instead of 4.9-5.3x).
-std::atomic<int> g_unroll{8};
+std::atomic<int> g_unroll{1};
 std::atomic<int> g_nontemporal{3};
-std::atomic<int> g_wg_per_cu{1024};
+std::atomic<int> g_wg_per_cu{65536};
 std::atomic<int> g_swap_workgroups{16};
 constexpr uint32_t kDuplexWorkgroups = 32;
+constexpr uint32_t kBesideDuplexWorkgroups = 16;
+constexpr int kBesideDuplexUnroll = 2;
+constexpr uint32_t kBesideTransferWorkgroups = 16;
 constexpr uint32_t kTransferWorkgroups = 48;
 constexpr uint32_t kSingleBlockTransferWorkgroups = 128;
+constexpr uint32_t kHostGatherWorkgroups = 64;
+constexpr uint64_t kLongHostGatherBytes = 4ull << 20;
 // The duplex swap wants little in flight per workgroup: one vector per lane and direction
 // (unroll 8 loses 6 %). 32 workgroups reach 98.1-98.4 GB/s summed for 16, 32 and 72 KiB
 // blocks; 40-64 dip to 89-94, 96-192 are a flat 98-99.
 std::atomic<int> g_duplex_unroll{1};
+std::atomic<int> g_duplex_workgroups{(int)kDuplexWorkgroups};
+std::atomic<int> g_hbm_lds_bytes{0};
+// Share of the link's raw rate, in thousandths, that a long throughput-mode launch offers toward the
+// host (0 = unpaced).
+std::atomic<int> g_throughput_pace_permille{900};
 std::atomic<int> g_swap_unroll{8};
 // Explicit offered rate of a swap that runs beside compute, MB/s; 0 = derive it from the link.
 std::atomic<int> g_swap_pace_mbps{0};
 // PCIe link rate override, MB/s; -1 = read each device's link from sysfs on first use.
 std::atomic<int> g_link_mbps_override{-1};
 
-// A swap that shares the GPU with other kernels (HFK_SWAP_BESIDE_COMPUTE) runs a grid this small:
-// enough workgroups to keep the link busy, few enough that what they hold in flight stays near the
-// link's bandwidth-delay product. Measured on MI355X, 16-72 KiB blocks:
-//  * writes to host: 8 workgroups x 4 vectors per lane, paced, sustain 56.8 GB/s (more than any
-//    unpaced grid: 55.5) and slow a memory-bound neighbour by 3-30 % where the 64-workgroup
-//    grid slows it 4-5x;
-//  * reads from host: pacing changes nothing, the neighbour's slowdown grows with the number of
-//    resident workgroups (8: 1.15-1.3x, 16: 1.3-1.8x, 64: 4-5x) while 8 already reach 57.5 GB/s on
-//    blocks that are whole 16 KiB chunks; other block sizes need 16.
-constexpr uint32_t kBesideWorkgroups = 8;
-constexpr int kBesideUnroll = 4;
-constexpr bool whole_beside_chunks(uint64_t block_bytes) {
-    return block_bytes % ((uint64_t)kWorkgroupLanes * 16u * kBesideUnroll) == 0;
-}
+// Launch shapes of a swap whose host side the caller has named. What a host-facing launch keeps in
+// flight beyond the link's bandwidth-delay product (about 64 KiB toward the host, 128 KiB from it)
+// does not make it faster; it queues in the memory fabric in front of every other kernel's traffic.
+// The gentlest shape that still fills the link is the finest one: ONE 16-byte vector per lane (4 KiB
+// per workgroup iteration) and just enough workgroups. Measured on MI355X with 32 KiB blocks, as
+// own rate / slowdown of a 1 GiB device copy / of a bf16 8192^3 GEMM on another stream:
+//  * toward the host, paced (workgroups x vectors per lane):
+//      12 x 1 at 0.90 of the link: 56.4 GB/s / 1.05x / 2.2x      16 x 4 at 0.90: 56.5 / 2.7x / 4.1x
+//      16 x 1 at 0.90:             56.6 GB/s / 1.08x / 2.7x
+//      12 x 1 at 0.84:             52.8 GB/s / 1.05x / 1.64x     8 x 4 at 0.84: 52.2 / 1.64x / 1.75x
+//    (8 x 1 cannot hold the pace: 42.9 GB/s; unpaced, small grids are erratic: 38-48 GB/s);
+//  * from the host, unpaced (pacing changes nothing there):
+//      24 x 1: 55.9 GB/s / 1.30x / 1.58x     40 x 1: 57.4 / 1.95x / 1.59x     16 x 4: 57.4 / 3.4x / 1.58x
+//    the copy's slowdown follows what is in flight, the GEMM's (1.55-1.6x) is what any resident kernel
+//    costs it.
+std::atomic<int> g_paced_workgroups{16};         // toward the host, throughput mode (HFK_KNOB_PACED_WORKGROUPS): 12 hold
+                                                 // the pace on an idle GPU, 16 also after a long run of other work
+constexpr uint32_t kBesidePacedWorkgroups = 12;  // toward the host, beside compute (the lower pace leaves the margin)
+constexpr uint32_t kFromHostWorkgroups = 40;     // from the host, throughput mode
+constexpr uint32_t kBesideFromHostWorkgroups = 24;
+constexpr uint32_t kBesideWorkgroups = 8;        // HFK_SWAP_BESIDE_COMPUTE with no host side named: 8 x 4, unpaced
+constexpr int kBesideUnnamedUnroll = 4;
+std::atomic<int> g_paced_unroll{1};              // vectors per lane of the named-side shapes (HFK_KNOB_PACED_UNROLL)
+int named_side_unroll() { return g_paced_unroll.load(std::memory_order_relaxed); }
 // Share of the link's raw rate offered to host writes when pacing. 256-byte transaction payloads
 // cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured, reached only by a paced grid); from 0.92
 // on throughput collapses to 0.84 and the neighbours' slowdown doubles. The closer to the cap, the
-// longer the fabric's queues: a GEMM beside the swap runs 1.56x slower at 0.83, 1.65x at 0.86,
-// 1.9x at 0.87, 2.5x at 0.90 (1.5x is what any resident kernel costs this GEMM).
+// longer the fabric's queues: a GEMM beside the 12 x 1 swap runs 1.64x slower at 0.84, 1.93x at 0.88,
+// 2.2x at 0.90 (1.55-1.6x is what any resident kernel costs this GEMM).
 constexpr double kPaceShareOfLink = 0.84;
-// Share offered by a throughput-mode swap-out: the cap itself.
-constexpr double kThroughputShareOfLink = 0.90;
+// Share offered by a throughput-mode swap-out: the cap itself (HFK_KNOB_THROUGHPUT_PACE_PERMILLE, default 0.90).
+double throughput_share_of_link() { return g_throughput_pace_permille.load(std::memory_order_relaxed) / 1000.0; }
 constexpr uint64_t kPaceFromBytes = 256ull << 20;
 
 constexpr int kMaxDevices = 64;
@@ -222,25 +264,38 @@ int current_link_mbps() {
 
 // ---- block copy -----------------------------------------------------------
 template <Role ROLE, typename IdT, int UNROLL, int NT>
-void launch_block_copy_one(const BlockCopyArgs<IdT>& a, uint32_t grid, hipStream_t s) {
+void launch_block_copy_one(const BlockCopyArgs<IdT>& a, uint32_t grid, uint32_t lds, hipStream_t s) {
+    if constexpr (std::is_same<IdT, int64_t>::value && ROLE != Role::kGatherRows) {
+        if (a.run_mode != hfk::kAllPairs) {   // a split table: non-temporal or plain, nothing in between
+            constexpr int SNT = NT != 0 ? 3 : 0;
+            if constexpr (ROLE == Role::kSwapBlocks) {
+                hipLaunchKernelGGL((swap_short_runs_kernel<UNROLL, SNT>), dim3(grid), dim3(256), lds, s, a);
+            } else if constexpr (ROLE == Role::kGatherBlocks) {
+                hipLaunchKernelGGL((gather_long_runs_kernel<UNROLL, SNT>), dim3(grid), dim3(256), lds, s, a);
+            } else {
+                hipLaunchKernelGGL((scatter_long_runs_kernel<UNROLL, SNT>), dim3(grid), dim3(256), lds, s, a);
+            }
+            return;
+        }
+    }
     if constexpr (ROLE == Role::kSwapBlocks) {
-        hipLaunchKernelGGL((swap_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((swap_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), lds, s, a);
     } else if constexpr (ROLE == Role::kGatherBlocks) {
-        hipLaunchKernelGGL((gather_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((gather_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), lds, s, a);
     } else if constexpr (ROLE == Role::kScatterBlocks) {
-        hipLaunchKernelGGL((scatter_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((scatter_blocks_kernel<UNROLL, NT>), dim3(grid), dim3(256), lds, s, a);
     } else {
-        hipLaunchKernelGGL((gather_rows_wide_kernel<IdT, UNROLL, NT>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((gather_rows_wide_kernel<IdT, UNROLL, NT>), dim3(grid), dim3(256), lds, s, a);
     }
 }
 
 template <Role ROLE, typename IdT, int UNROLL>
-void launch_block_copy_nt(const BlockCopyArgs<IdT>& a, uint32_t grid, int nt, hipStream_t s) {
+void launch_block_copy_nt(const BlockCopyArgs<IdT>& a, uint32_t grid, int nt, uint32_t lds, hipStream_t s) {
     switch (nt & 3) {
-        case 0: launch_block_copy_one<ROLE, IdT, UNROLL, 0>(a, grid, s); break;
-        case 1: launch_block_copy_one<ROLE, IdT, UNROLL, 1>(a, grid, s); break;
-        case 2: launch_block_copy_one<ROLE, IdT, UNROLL, 2>(a, grid, s); break;
-        default: launch_block_copy_one<ROLE, IdT, UNROLL, 3>(a, grid, s); break;
+        case 0: launch_block_copy_one<ROLE, IdT, UNROLL, 0>(a, grid, lds, s); break;
+        case 1: launch_block_copy_one<ROLE, IdT, UNROLL, 1>(a, grid, lds, s); break;
+        case 2: launch_block_copy_one<ROLE, IdT, UNROLL, 2>(a, grid, lds, s); break;
+        default: launch_block_copy_one<ROLE, IdT, UNROLL, 3>(a, grid, lds, s); break;
     }
 }
 
@@ -262,12 +317,15 @@ int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, 
         a.pace_q8 = q8 < 4294967295.0 ? (uint32_t)q8 : 0xffffffffu;   // absurdly low rates: the wait's spin limit rules
     }
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
+    // HBM-bound launches may ask for LDS they never touch: it bounds how many workgroups a compute
+    // unit holds at a time (HFK_KNOB_HBM_LDS_BYTES).
+    const uint32_t lds = ROLE == Role::kSwapBlocks ? 0u : (uint32_t)g_hbm_lds_bytes.load(std::memory_order_relaxed);
     switch (unroll) {
-        case 1: launch_block_copy_nt<ROLE, IdT, 1>(a, grid, nt, s); break;
-        case 2: launch_block_copy_nt<ROLE, IdT, 2>(a, grid, nt, s); break;
-        case 4: launch_block_copy_nt<ROLE, IdT, 4>(a, grid, nt, s); break;
-        case 8: launch_block_copy_nt<ROLE, IdT, 8>(a, grid, nt, s); break;
-        default: launch_block_copy_nt<ROLE, IdT, 16>(a, grid, nt, s); break;
+        case 1: launch_block_copy_nt<ROLE, IdT, 1>(a, grid, nt, lds, s); break;
+        case 2: launch_block_copy_nt<ROLE, IdT, 2>(a, grid, nt, lds, s); break;
+        case 4: launch_block_copy_nt<ROLE, IdT, 4>(a, grid, nt, lds, s); break;
+        case 8: launch_block_copy_nt<ROLE, IdT, 8>(a, grid, nt, lds, s); break;
+        default: launch_block_copy_nt<ROLE, IdT, 16>(a, grid, nt, lds, s); break;
     }
     return finish_launch();
 }
@@ -357,7 +415,8 @@ int memory_side(const void* p) {
 int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64_t* pairs, uint64_t n_pairs,
                      uint64_t packed_stride, uint64_t layered_stride, uint64_t packed_blocks,
                      uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
-                     bool to_packed, bool packed_in_device, uint32_t workgroups, hipStream_t s) {
+                     bool to_packed, bool packed_in_device, uint32_t workgroups, hipStream_t s,
+                     bool beside_compute = false) {
     TransposeArgs a;
     uint32_t unit = 16;
     int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, packed, pairs, n_pairs, packed_stride, layered_stride,
@@ -372,7 +431,9 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     if (workgroups == 0 && side != 0) {
         // One block (the reference's op: 4-64 MiB, over in 0.1-1.2 ms) is sized for speed alone; a
         // block table may run for many milliseconds beside other kernels and gets the smaller grid.
-        workgroups = pairs == nullptr ? kSingleBlockTransferWorkgroups : kTransferWorkgroups;
+        workgroups = pairs == nullptr ? kSingleBlockTransferWorkgroups
+                     : beside_compute ? kBesideTransferWorkgroups
+                                      : kTransferWorkgroups;
     }
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
@@ -382,6 +443,184 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, to_packed, s);
     else launch_transpose_v<uint8_t>(a, grid, nt, to_packed, s);
     return finish_launch();
+}
+
+// Launch shape of a block-table swap, from what the caller says about it (`flags`) and how many bytes
+// it moves (`bytes`; for a table split by run length, the share this launch moves).
+constexpr uint32_t kSwapFlagMask = HFK_SWAP_DST_HOST | HFK_SWAP_SRC_HOST | HFK_SWAP_BESIDE_COMPUTE;
+
+int launch_swap(const BlockCopyArgs<int64_t>& a, uint32_t flags, uint32_t workgroups, uint64_t bytes, hipStream_t s) {
+    const bool beside = (flags & HFK_SWAP_BESIDE_COMPUTE) != 0;
+    if ((flags & HFK_SWAP_DST_HOST) != 0 && (beside || bytes >= kPaceFromBytes)) {
+        // Toward the host the link accepts the most when it is offered exactly what it can take
+        // (offering 1.5-2x its rate lowers what it accepts to 47-49 GB/s). A swap that shares the GPU
+        // offers 0.84 of the raw rate, one that owns it the payload-efficiency cap, 0.90; should the
+        // cap be lower than assumed the launch degrades to an unpaced one. A paced launch ends about
+        // 0.1 ms behind its schedule, which only a long one amortises (32 MiB: 49 GB/s paced, 54.6
+        // unpaced), so a short throughput-mode swap stays unpaced.
+        uint32_t pace_mbps = 0;
+        if (beside) {
+            pace_mbps = (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed);
+            if (pace_mbps == 0) pace_mbps = (uint32_t)(kPaceShareOfLink * current_link_mbps());
+        } else {
+            pace_mbps = (uint32_t)(throughput_share_of_link() * current_link_mbps());
+        }
+        if (pace_mbps != 0) {
+            if (workgroups == 0) {
+                workgroups = beside ? kBesidePacedWorkgroups : (uint32_t)g_paced_workgroups.load(std::memory_order_relaxed);
+            }
+            return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, named_side_unroll(), pace_mbps);
+        }
+    }
+    if ((flags & HFK_SWAP_SRC_HOST) != 0) {
+        const uint32_t grid = beside ? kBesideFromHostWorkgroups : kFromHostWorkgroups;
+        return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups ? workgroups : grid, s, named_side_unroll());
+    }
+    if (beside) {
+        // No usable pace (no host side named, or the link's rate is unknown): the small unpaced grid
+        // (49.8 GB/s toward the host: between the link rate and twice it, offering more gets less accepted).
+        return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups ? workgroups : kBesideWorkgroups, s,
+                                                             kBesideUnnamedUnroll);
+    }
+    // Nothing known about the sides: sized for the PCIe link, which a small grid saturates
+    // (16 workgroups x 8 vectors per lane: 55.4-55.7 GB/s out, 57.0-57.4 in).
+    if (workgroups == 0) workgroups = (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
+    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, g_swap_unroll.load(std::memory_order_relaxed));
+}
+
+// ---- staged swap: HBM-only kernel + DMA copies ----------------------------
+// What the PCIe leg of a staged (or split) swap needs to know.
+struct HostLeg {
+    void* const* host_plane_addrs;   // host array of n_planes host addresses
+    const int64_t* host_block_ids;   // host array of n_blocks slots
+    uint32_t n_planes;
+    uint64_t n_blocks;
+    uint64_t block_bytes;
+    uint64_t host_block_stride;
+    void* staging;                   // [n_planes][n_blocks][block_bytes] in device memory
+    bool to_host;
+};
+
+int check_host_leg(const HostLeg& h, uint64_t host_blocks) {
+    if (h.host_plane_addrs == nullptr || h.host_block_ids == nullptr) return HFK_ERR_NULL_POINTER;
+    if (h.host_block_stride < h.block_bytes) return HFK_ERR_BAD_SIZE;
+    for (uint32_t p = 0; p < h.n_planes; ++p) {
+        if (h.host_plane_addrs[p] == nullptr) return HFK_ERR_NULL_POINTER;
+    }
+    for (uint64_t i = 0; i < h.n_blocks; ++i) {  // nothing is enqueued unless every host slot is valid
+        if (h.host_block_ids[i] < 0 || (host_blocks != 0 && (uint64_t)h.host_block_ids[i] >= host_blocks)) {
+            return HFK_ERR_OUT_OF_RANGE;
+        }
+    }
+    return HFK_OK;
+}
+
+// The PCIe leg: one copy per run of at least `min_run` consecutive host slots. A run of k slots is
+// k * block_bytes contiguous bytes in every plane. Planes that are evenly spaced on the host (a
+// pool [planes][blocks][...], the usual case) are moved together by ONE 2-D copy per run (rows =
+// planes), which the DMA engines execute at their full rate (57 GB/s measured, against 53 for one
+// copy per plane); a plane that does not line up gets its own copy. Host blocks with a padded
+// stride use a 2-D copy per plane (rows = blocks). All copies go to `s`: dealing the runs to two
+// streams gains nothing (same-direction copies are executed one after the other: 45.1 GB/s either
+// way for 111 runs of 2-14 MiB; a copy costs its engine about 9.5 us before the first byte moves).
+int copy_host_runs(const HostLeg& h, uint64_t min_run, hipStream_t s) {
+    const uint64_t stage_pitch = h.n_blocks * h.block_bytes;
+    hipError_t e = hipSuccess;
+    // Copies `run_bytes` at host_off / stage_off for planes [p0, p0 + count), which are evenly spaced
+    // by `pitch` bytes on the host (count == 1: a plain copy).
+    auto copy_plane_group = [&](uint32_t p0, uint32_t count, int64_t pitch, uint64_t host_off, uint64_t stage_off,
+                                uint64_t run_bytes) -> hipError_t {
+        hipStream_t cs = s;
+        char* hp = static_cast<char*>(h.host_plane_addrs[p0]) + host_off;
+        char* d = static_cast<char*>(h.staging) + (uint64_t)p0 * stage_pitch + stage_off;
+        if (count == 1) {
+            return h.to_host ? hipMemcpyAsync(hp, d, run_bytes, hipMemcpyDeviceToHost, cs)
+                             : hipMemcpyAsync(d, hp, run_bytes, hipMemcpyHostToDevice, cs);
+        }
+        return h.to_host
+                   ? hipMemcpy2DAsync(hp, (size_t)pitch, d, stage_pitch, run_bytes, count, hipMemcpyDeviceToHost, cs)
+                   : hipMemcpy2DAsync(d, stage_pitch, hp, (size_t)pitch, run_bytes, count, hipMemcpyHostToDevice, cs);
+    };
+    hfk::for_each_host_run(h.host_block_ids, h.n_blocks, [&](uint64_t first, uint64_t len) {
+        if (len < min_run || e != hipSuccess) return;
+        hipStream_t cs = s;
+        const uint64_t host_off = (uint64_t)h.host_block_ids[first] * h.host_block_stride;
+        const uint64_t stage_off = first * h.block_bytes;
+        const uint64_t run_bytes = len * h.block_bytes;
+        if (h.host_block_stride == h.block_bytes) {
+            // maximal groups of evenly spaced planes: one 2-D copy each
+            uint32_t p0 = 0;
+            while (p0 < h.n_planes && e == hipSuccess) {
+                uint32_t count = 1;
+                int64_t pitch = 0;
+                if (p0 + 1 < h.n_planes) {
+                    pitch = static_cast<char*>(h.host_plane_addrs[p0 + 1]) - static_cast<char*>(h.host_plane_addrs[p0]);
+                    if (pitch >= (int64_t)run_bytes) {
+                        count = 2;
+                        while (p0 + count < h.n_planes &&
+                               static_cast<char*>(h.host_plane_addrs[p0 + count]) -
+                                       static_cast<char*>(h.host_plane_addrs[p0 + count - 1]) == pitch) {
+                            ++count;
+                        }
+                    }
+                }
+                e = copy_plane_group(p0, count, pitch, host_off, stage_off, run_bytes);
+                p0 += count;
+            }
+        } else {
+            for (uint32_t p = 0; p < h.n_planes && e == hipSuccess; ++p) {
+                char* hp = static_cast<char*>(h.host_plane_addrs[p]) + host_off;
+                char* d = static_cast<char*>(h.staging) + (uint64_t)p * stage_pitch + stage_off;
+                e = h.to_host ? hipMemcpy2DAsync(hp, h.host_block_stride, d, h.block_bytes, h.block_bytes, len,
+                                                 hipMemcpyDeviceToHost, cs)
+                              : hipMemcpy2DAsync(d, h.block_bytes, hp, h.host_block_stride, h.block_bytes, len,
+                                                 hipMemcpyHostToDevice, cs);
+            }
+        }
+    });
+    return e == hipSuccess ? HFK_OK : (int)e;
+}
+
+int staged_swap(const void* dev_plane_ptrs, void* const* host_plane_addrs, const int64_t* dev_block_ids,
+                const int64_t* host_block_ids, uint32_t n_planes, uint64_t n_blocks, uint64_t block_bytes,
+                uint64_t dev_block_stride, uint64_t host_block_stride, uint64_t dev_blocks, uint64_t host_blocks,
+                void* staging, int to_host, uint32_t workgroups, hipStream_t s) {
+    const HostLeg leg{host_plane_addrs, host_block_ids, n_planes, n_blocks, block_bytes, host_block_stride, staging,
+                      to_host != 0};
+    BlockCopyArgs<int64_t> a;
+    int rc = hfk::plan_stage_blocks(a, dev_plane_ptrs, staging, dev_block_ids, n_planes, n_blocks, block_bytes,
+                                    dev_block_stride, dev_blocks, to_host != 0);
+    if (rc != 0) return rc;
+    rc = check_host_leg(leg, host_blocks);
+    if (rc != 0) return rc;
+    if (to_host) {
+        rc = launch_block_copy<Role::kGatherBlocks, int64_t>(a, workgroups, s);
+        if (rc != 0) return rc;
+        return copy_host_runs(leg, 1, s);
+    }
+    rc = copy_host_runs(leg, 1, s);
+    if (rc != 0) return rc;
+    return launch_block_copy<Role::kScatterBlocks, int64_t>(a, workgroups, s);
+}
+
+// A run of host slots is worth a DMA copy when one copy of it moves at least this much.
+constexpr uint64_t kDmaRunBytes = 16ull << 20;
+constexpr uint64_t kDmaRunBytesBesideCompute = 4ull << 20;
+// Longest run threshold the kernels' run filter is asked to evaluate (it reads up to twice as many
+// table entries per pair); a larger threshold means "never stage".
+constexpr uint64_t kMaxRunFilter = 1024;
+
+// Number of leading planes that one 2-D copy covers (planes evenly spaced on the host).
+uint64_t evenly_spaced_planes(const HostLeg& h) {
+    if (h.n_planes < 2) return 1;
+    const int64_t pitch = static_cast<char*>(h.host_plane_addrs[1]) - static_cast<char*>(h.host_plane_addrs[0]);
+    if (pitch < (int64_t)h.block_bytes) return 1;
+    uint64_t count = 2;
+    while (count < h.n_planes && static_cast<char*>(h.host_plane_addrs[count]) -
+                                         static_cast<char*>(h.host_plane_addrs[count - 1]) == pitch) {
+        ++count;
+    }
+    return count;
 }
 
 }  // namespace
@@ -411,6 +650,13 @@ int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i
     if (table == nullptr || dst == nullptr || ids == nullptr) return HFK_ERR_NULL_POINTER;
     if (row_bytes == 0) return HFK_ERR_BAD_SIZE;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (workgroups == 0 && n_ids * row_bytes > kLongHostGatherBytes && memory_side(table) == 1) {
+        // A table in host memory (the reference's embedding case) is read over the PCIe link: 64
+        // workgroups already run it at the link's rate (55-57 GB/s for 1 KiB rows), and every further
+        // one only slows kernels on other streams. Gathers of a few MiB keep one workgroup per chunk
+        // (they are over in tens of microseconds and a cap would only add a partly filled second round).
+        workgroups = kHostGatherWorkgroups;
+    }
     if (ids_are_i64) {
         return gather_rows_typed<int64_t>(table, dst, static_cast<const int64_t*>(ids), n_ids, row_bytes,
                                           table_rows, workgroups, s);
@@ -445,78 +691,66 @@ int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t de
                                          void* packed_blocks, uint64_t packed_block_stride,
                                          const int64_t* block_pairs, uint64_t n_pairs, uint64_t n_packed_blocks,
                                          uint64_t n_dev_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D,
-                                         uint32_t elem_bytes, int to_packed, uint32_t workgroups,
+                                         uint32_t elem_bytes, int to_packed, uint32_t flags, uint32_t workgroups,
                                          hfk_stream_t stream) {
+    if ((flags & ~(uint32_t)HFK_SWAP_BESIDE_COMPUTE) != 0) return HFK_ERR_BAD_FLAGS;
     if (n_pairs == 0) return HFK_OK;
     if (block_pairs == nullptr) return HFK_ERR_NULL_POINTER;
     return launch_transpose(dev_layer_ptrs, packed_blocks, block_pairs, n_pairs, packed_block_stride,
                             dev_block_stride, n_packed_blocks, n_dev_blocks, T, L, H, D, elem_bytes, to_packed != 0,
-                            false, workgroups, static_cast<hipStream_t>(stream));
+                            false, workgroups, static_cast<hipStream_t>(stream), (flags & HFK_SWAP_BESIDE_COMPUTE) != 0);
 }
 
 int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* block_pairs,
                     uint32_t n_planes, uint64_t n_pairs, uint64_t block_bytes, uint64_t src_block_stride,
                     uint64_t dst_block_stride, uint64_t src_blocks, uint64_t dst_blocks, uint32_t flags,
                     uint32_t workgroups, hfk_stream_t stream) {
-    if ((flags & ~(uint32_t)(HFK_SWAP_DST_HOST | HFK_SWAP_SRC_HOST | HFK_SWAP_BESIDE_COMPUTE)) != 0) {
-        return HFK_ERR_BAD_FLAGS;
-    }
+    if ((flags & ~kSwapFlagMask) != 0) return HFK_ERR_BAD_FLAGS;
     if (n_planes == 0 || n_pairs == 0) return HFK_OK;
     BlockCopyArgs<int64_t> a;
     int rc = hfk::plan_swap_blocks(a, dst_plane_ptrs, src_plane_ptrs, block_pairs, n_planes, n_pairs, block_bytes,
                                    src_block_stride, dst_block_stride, src_blocks, dst_blocks);
     if (rc != 0) return rc;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if ((flags & HFK_SWAP_BESIDE_COMPUTE) != 0) {
-        // Without a named host side the grid is still the small one, only unpaced (49.8 GB/s toward
-        // the host on MI355X: between the link rate and twice it, offering more gets less accepted).
-        uint32_t pace_mbps = 0;
-        if ((flags & HFK_SWAP_DST_HOST) != 0) {
-            pace_mbps = (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed);
-            if (pace_mbps == 0) pace_mbps = (uint32_t)(kPaceShareOfLink * current_link_mbps());
-        }
-        if (workgroups == 0) {
-            workgroups = ((flags & HFK_SWAP_SRC_HOST) != 0 && !whole_beside_chunks(block_bytes)) ? 2 * kBesideWorkgroups
-                                                                                                : kBesideWorkgroups;
-        }
-        return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, kBesideUnroll, pace_mbps);
-    }
-    // Throughput mode. A swap is bound by the PCIe link, which a small grid saturates; more
-    // workgroups only queue on the link.
-    if (workgroups == 0) workgroups = (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
-    if ((flags & HFK_SWAP_DST_HOST) != 0 && (uint64_t)n_planes * n_pairs * block_bytes >= kPaceFromBytes) {
-        // Toward the host the link accepts the most when it is offered exactly what it can take:
-        // paced at its payload-efficiency cap the same grid sustains 56.8 GB/s where it reaches 55.4
-        // unpaced, and should the cap be lower than assumed the launch degrades to the unpaced rate.
-        // A paced launch ends about 0.1 ms later than its schedule says, which only a long one amortises
-        // (32 MiB: 49 GB/s paced, 54.6 unpaced; 256 MiB: 56.0 against 55.6).
-        const uint32_t pace_mbps = (uint32_t)(kThroughputShareOfLink * current_link_mbps());
-        if (pace_mbps != 0) {
-            return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, kBesideUnroll, pace_mbps);
-        }
-    }
-    int unroll = g_swap_unroll.load(std::memory_order_relaxed);
-    if ((flags & HFK_SWAP_SRC_HOST) != 0 && whole_beside_chunks(block_bytes) && unroll > kBesideUnroll) {
-        // From the host, blocks that are whole 16 KiB chunks reach the link rate with half as much in
-        // flight (57.6 GB/s either way; a memory-bound neighbour 1.3-1.7x slower instead of 2.3-2.4x).
-        unroll = kBesideUnroll;
-    }
-    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, unroll);
+    return launch_swap(a, flags, workgroups, (uint64_t)n_planes * n_pairs * block_bytes,
+                       static_cast<hipStream_t>(stream));
 }
 
 int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move* in_move, uint32_t n_planes,
-                           uint64_t block_bytes, uint32_t workgroups, hfk_stream_t stream) {
+                           uint64_t block_bytes, uint32_t flags, uint32_t workgroups, hfk_stream_t stream) {
+    if ((flags & ~(uint32_t)HFK_SWAP_BESIDE_COMPUTE) != 0) return HFK_ERR_BAD_FLAGS;
     DuplexCopyArgs a;
     int unroll = 1;
     if (block_bytes == 0) return HFK_ERR_BAD_SIZE;
+    const bool beside = (flags & HFK_SWAP_BESIDE_COMPUTE) != 0;
+    // Beside compute: half the workgroups, two vectors per lane and direction, paced (97-98 GB/s summed
+    // on 16 workgroups where one vector per lane leaves them latency-bound at 64).
     int rc = hfk::plan_duplex(a, out_move, in_move, n_planes, block_bytes,
-                              g_duplex_unroll.load(std::memory_order_relaxed), &unroll);
+                              beside ? kBesideDuplexUnroll : g_duplex_unroll.load(std::memory_order_relaxed), &unroll);
     if (rc != 0) return rc;
     if (a.n_work == 0) return HFK_OK;
-    if (workgroups == 0) workgroups = kDuplexWorkgroups;
+    if (workgroups == 0) {
+        workgroups = beside ? kBesideDuplexWorkgroups : (uint32_t)g_duplex_workgroups.load(std::memory_order_relaxed);
+    }
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
+    const uint64_t out_bytes = out_move ? (uint64_t)n_planes * out_move->n_pairs * block_bytes : 0;
+    if (a.first.n_work != 0 && (beside || out_bytes >= kPaceFromBytes)) {
+        // Every iteration moves one chunk toward the host (and one from it): offer the link what the
+        // paced one-way swap offers it in the same mode.
+        uint32_t pace_mbps = 0;
+        if (beside) {
+            pace_mbps = (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed);
+            if (pace_mbps == 0) pace_mbps = (uint32_t)(kPaceShareOfLink * current_link_mbps());
+        } else {
+            pace_mbps = (uint32_t)(throughput_share_of_link() * current_link_mbps());
+        }
+        if (pace_mbps != 0) {
+            const double item_bytes = (double)block_bytes / a.first.chunks_per_block;
+            const double q8 = item_bytes * grid / ((double)pace_mbps * 1e6) * 1e8 * 256.0 + 0.5;
+            a.pace_q8 = q8 < 4294967295.0 ? (uint32_t)q8 : 0xffffffffu;
+        }
+    }
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (unroll) {
@@ -535,103 +769,95 @@ int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host_plane_a
                            uint64_t host_blocks, void* staging, int to_host, uint32_t workgroups,
                            hfk_stream_t stream) {
     if (n_planes == 0 || n_blocks == 0) return HFK_OK;
-    if (host_plane_addrs == nullptr || host_block_ids == nullptr) return HFK_ERR_NULL_POINTER;
-    if (host_block_stride < block_bytes) return HFK_ERR_BAD_SIZE;
-    BlockCopyArgs<int64_t> a;
-    int rc = hfk::plan_stage_blocks(a, dev_plane_ptrs, staging, dev_block_ids, n_planes, n_blocks, block_bytes,
-                                    dev_block_stride, dev_blocks, to_host != 0);
-    if (rc != 0) return rc;
-    for (uint32_t p = 0; p < n_planes; ++p) {
-        if (host_plane_addrs[p] == nullptr) return HFK_ERR_NULL_POINTER;
-    }
-    for (uint64_t i = 0; i < n_blocks; ++i) {  // nothing is enqueued unless every host slot is valid
-        if (host_block_ids[i] < 0 || (host_blocks != 0 && (uint64_t)host_block_ids[i] >= host_blocks)) {
-            return HFK_ERR_OUT_OF_RANGE;
-        }
-    }
+    return staged_swap(dev_plane_ptrs, host_plane_addrs, dev_block_ids, host_block_ids, n_planes, n_blocks, block_bytes,
+                       dev_block_stride, host_block_stride, dev_blocks, host_blocks, staging, to_host, workgroups,
+                       static_cast<hipStream_t>(stream));
+}
+
+int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs, void* const* host_plane_addrs,
+                         const int64_t* block_pairs, const int64_t* host_block_ids, uint32_t n_planes,
+                         uint64_t n_pairs, uint64_t block_bytes, uint64_t dev_block_stride,
+                         uint64_t host_block_stride, uint64_t dev_blocks, uint64_t host_blocks, void* staging,
+                         uint64_t staging_bytes, int to_host, uint32_t min_run_blocks, uint32_t flags,
+                         hfk_stream_t stream) {
+    if ((flags & ~(uint32_t)HFK_SWAP_BESIDE_COMPUTE) != 0) return HFK_ERR_BAD_FLAGS;
+    if (n_planes == 0 || n_pairs == 0) return HFK_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // The PCIe leg. A run of k consecutive host slots is k * block_bytes contiguous bytes in every
-    // plane. Planes that are evenly spaced on the host (a pool [planes][blocks][...], the usual case)
-    // are moved together by ONE 2-D copy per run (rows = planes), which the DMA engines execute at
-    // their full rate (57 GB/s measured, against 53 for one copy per plane); a plane that does not
-    // line up gets its own copy. Host blocks with a padded stride use a 2-D copy per plane (rows = blocks).
-    const uint64_t stage_pitch = n_blocks * block_bytes;
-    // Copies `run_bytes` at host_off / stage_off for planes [p0, p0 + count), which are evenly spaced
-    // by `pitch` bytes on the host (count == 1: a plain copy).
-    auto copy_plane_group = [&](uint32_t p0, uint32_t count, int64_t pitch, uint64_t host_off, uint64_t stage_off,
-                                uint64_t run_bytes) -> hipError_t {
-        char* h = static_cast<char*>(host_plane_addrs[p0]) + host_off;
-        char* d = static_cast<char*>(staging) + (uint64_t)p0 * stage_pitch + stage_off;
-        if (count == 1) {
-            return to_host ? hipMemcpyAsync(h, d, run_bytes, hipMemcpyDeviceToHost, s)
-                           : hipMemcpyAsync(d, h, run_bytes, hipMemcpyHostToDevice, s);
-        }
-        return to_host ? hipMemcpy2DAsync(h, (size_t)pitch, d, stage_pitch, run_bytes, count, hipMemcpyDeviceToHost, s)
-                       : hipMemcpy2DAsync(d, stage_pitch, h, (size_t)pitch, run_bytes, count, hipMemcpyHostToDevice, s);
-    };
-    auto copy_runs = [&]() -> int {
-        uint64_t first = 0;
-        while (first < n_blocks) {
-            uint64_t len = 1;
-            while (first + len < n_blocks && host_block_ids[first + len] == host_block_ids[first] + (int64_t)len) ++len;
-            const uint64_t host_off = (uint64_t)host_block_ids[first] * host_block_stride;
-            const uint64_t stage_off = first * block_bytes;
-            const uint64_t run_bytes = len * block_bytes;
-            hipError_t e = hipSuccess;
-            if (host_block_stride == block_bytes) {
-                // maximal groups of evenly spaced planes: one 2-D copy each
-                uint32_t p0 = 0;
-                while (p0 < n_planes && e == hipSuccess) {
-                    uint32_t count = 1;
-                    int64_t pitch = 0;
-                    if (p0 + 1 < n_planes) {
-                        pitch = static_cast<char*>(host_plane_addrs[p0 + 1]) - static_cast<char*>(host_plane_addrs[p0]);
-                        if (pitch >= (int64_t)run_bytes) {
-                            count = 2;
-                            while (p0 + count < n_planes &&
-                                   static_cast<char*>(host_plane_addrs[p0 + count]) -
-                                           static_cast<char*>(host_plane_addrs[p0 + count - 1]) == pitch) {
-                                ++count;
-                            }
-                        }
-                    }
-                    e = copy_plane_group(p0, count, pitch, host_off, stage_off, run_bytes);
-                    p0 += count;
-                }
-            } else {
-                for (uint32_t p = 0; p < n_planes && e == hipSuccess; ++p) {
-                    char* h = static_cast<char*>(host_plane_addrs[p]) + host_off;
-                    char* d = static_cast<char*>(staging) + (uint64_t)p * stage_pitch + stage_off;
-                    e = to_host ? hipMemcpy2DAsync(h, host_block_stride, d, block_bytes, block_bytes, len,
-                                                   hipMemcpyDeviceToHost, s)
-                                : hipMemcpy2DAsync(d, block_bytes, h, host_block_stride, block_bytes, len,
-                                                   hipMemcpyHostToDevice, s);
-                }
-            }
-            if (e != hipSuccess) return (int)e;
-            first += len;
-        }
-        return HFK_OK;
-    };
-    if (to_host) {
-        rc = launch_block_copy<Role::kGatherBlocks, int64_t>(a, workgroups, s);
-        if (rc != 0) return rc;
-        return copy_runs();
-    }
-    rc = copy_runs();
+    const bool out = to_host != 0;
+    const uint32_t side_flags = flags | (out ? HFK_SWAP_DST_HOST : HFK_SWAP_SRC_HOST);
+    // The direct mover over the whole table: (src, dst) = (device, host) on the way out, (host, device) back.
+    BlockCopyArgs<int64_t> direct;
+    int rc = out ? hfk::plan_swap_blocks(direct, host_plane_ptrs, dev_plane_ptrs, block_pairs, n_planes, n_pairs,
+                                         block_bytes, dev_block_stride, host_block_stride, dev_blocks, host_blocks)
+                 : hfk::plan_swap_blocks(direct, dev_plane_ptrs, host_plane_ptrs, block_pairs, n_planes, n_pairs,
+                                         block_bytes, host_block_stride, dev_block_stride, host_blocks, dev_blocks);
     if (rc != 0) return rc;
-    return launch_block_copy<Role::kScatterBlocks, int64_t>(a, workgroups, s);
+    direct.zero_skipped = out ? 1u : 0u;   // one rule for the whole table, whichever mover takes a pair
+    const uint64_t total_bytes = (uint64_t)n_planes * n_pairs * block_bytes;
+    const bool can_stage = staging != nullptr && host_plane_addrs != nullptr && host_block_ids != nullptr &&
+                           staging_bytes / block_bytes / n_pairs >= n_planes;
+    uint64_t min_run = min_run_blocks;
+    uint64_t long_blocks = 0;
+    if (can_stage) {
+        const HostLeg probe{host_plane_addrs, host_block_ids, n_planes, n_pairs, block_bytes, host_block_stride, staging,
+                            out};
+        rc = check_host_leg(probe, host_blocks);
+        if (rc != 0) return rc;
+        if (min_run == 0) {
+            // A copy costs the DMA engines about 9.5 us before its first byte, 0.5 MiB of link time. A swap
+            // that has the GPU to itself hands them only runs they move at 97 % of the link rate or better
+            // (16 MiB per copy); one that shares it gives up to 12 % of its own rate (4 MiB per copy) so
+            // that more of the table bypasses the compute units.
+            const uint64_t run_bytes = (flags & HFK_SWAP_BESIDE_COMPUTE) != 0 ? kDmaRunBytesBesideCompute : kDmaRunBytes;
+            const uint64_t planes_per_copy = host_block_stride == block_bytes ? evenly_spaced_planes(probe) : 1;
+            const uint64_t per_block = block_bytes * planes_per_copy;
+            min_run = (run_bytes + per_block - 1) / per_block;
+        }
+        if (min_run <= kMaxRunFilter) long_blocks = hfk::blocks_in_long_runs(host_block_ids, n_pairs, min_run);
+    }
+    if (long_blocks == 0) {   // nothing for the copy engines (or no staging to give them): one direct launch
+        return launch_swap(direct, side_flags, 0, total_bytes, s);
+    }
+    const HostLeg leg{host_plane_addrs, host_block_ids, n_planes, n_pairs, block_bytes, host_block_stride, staging, out};
+    const int64_t* host_column = block_pairs + (out ? 1 : 0);
+    const int64_t* dev_column = block_pairs + (out ? 0 : 1);
+    BlockCopyArgs<int64_t> hbm;   // long runs: device planes <-> staging, the copy engines do the rest
+    rc = hfk::plan_stage_blocks(hbm, dev_plane_ptrs, staging, dev_column, n_planes, n_pairs, block_bytes,
+                                dev_block_stride, dev_blocks, out);
+    if (rc != 0) return rc;
+    hbm.id_stride = 2;
+    const bool split = long_blocks < n_pairs;
+    if (split) {
+        hfk::filter_runs(hbm, hfk::kLongRunsOnly, host_column, (uint32_t)min_run);
+        hfk::filter_runs(direct, hfk::kShortRunsOnly, host_column, (uint32_t)min_run);
+    }
+    if (out) {
+        rc = launch_block_copy<Role::kGatherBlocks, int64_t>(hbm, 0, s);
+        if (rc == 0) rc = copy_host_runs(leg, min_run, s);
+    } else {
+        rc = copy_host_runs(leg, min_run, s);
+        if (rc == 0) rc = launch_block_copy<Role::kScatterBlocks, int64_t>(hbm, 0, s);
+    }
+    if (rc != 0 || !split) return rc;
+    return launch_swap(direct, side_flags, 0, (n_pairs - long_blocks) * n_planes * block_bytes, s);
 }
 
 int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* ids,
                       uint32_t n_planes, uint64_t n_ids, uint64_t block_bytes, uint64_t src_block_stride,
-                      uint64_t src_blocks, uint32_t workgroups, hfk_stream_t stream) {
+                      uint64_t src_blocks, uint32_t flags, uint32_t workgroups, hfk_stream_t stream) {
+    if ((flags & ~(uint32_t)(HFK_SWAP_SRC_HOST | HFK_SWAP_BESIDE_COMPUTE)) != 0) return HFK_ERR_BAD_FLAGS;
     if (n_planes == 0 || n_ids == 0) return HFK_OK;
     BlockCopyArgs<int64_t> a;
     int rc = hfk::plan_gather_blocks(a, dst_plane_ptrs, src_plane_ptrs, ids, n_planes, n_ids, block_bytes,
                                      src_block_stride, src_blocks);
     if (rc != 0) return rc;
-    return launch_block_copy<Role::kGatherBlocks, int64_t>(a, workgroups, static_cast<hipStream_t>(stream));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if ((flags & HFK_SWAP_SRC_HOST) != 0) {
+        // Source planes in host memory: this is a swap-in whose destinations are consecutive, and the
+        // PCIe link, not HBM, sizes the launch.
+        return launch_swap(a, flags, workgroups, (uint64_t)n_planes * n_ids * block_bytes, s);
+    }
+    return launch_block_copy<Role::kGatherBlocks, int64_t>(a, workgroups, s);
 }
 
 int hfk_set_tuning(int knob, int64_t value) {
@@ -645,7 +871,7 @@ int hfk_set_tuning(int knob, int64_t value) {
             g_nontemporal.store((int)value);
             return HFK_OK;
         case HFK_KNOB_WORKGROUPS_PER_CU:
-            if (value < 1 || value > 1024) return HFK_ERR_BAD_KNOB;
+            if (value < 1 || value > 65536) return HFK_ERR_BAD_KNOB;
             g_wg_per_cu.store((int)value);
             return HFK_OK;
         case HFK_KNOB_SWAP_WORKGROUPS:
@@ -668,6 +894,26 @@ int hfk_set_tuning(int knob, int64_t value) {
             if (value < -1 || value > 1000000) return HFK_ERR_BAD_KNOB;
             g_link_mbps_override.store((int)value);
             return HFK_OK;
+        case HFK_KNOB_DUPLEX_WORKGROUPS:
+            if (value < 1 || value > (1 << 20)) return HFK_ERR_BAD_KNOB;
+            g_duplex_workgroups.store((int)value);
+            return HFK_OK;
+        case HFK_KNOB_THROUGHPUT_PACE_PERMILLE:
+            if (value < 0 || value > 2000) return HFK_ERR_BAD_KNOB;
+            g_throughput_pace_permille.store((int)value);
+            return HFK_OK;
+        case HFK_KNOB_PACED_UNROLL:
+            if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return HFK_ERR_BAD_KNOB;
+            g_paced_unroll.store((int)value);
+            return HFK_OK;
+        case HFK_KNOB_PACED_WORKGROUPS:
+            if (value < 1 || value > (1 << 20)) return HFK_ERR_BAD_KNOB;
+            g_paced_workgroups.store((int)value);
+            return HFK_OK;
+        case HFK_KNOB_HBM_LDS_BYTES:
+            if (value < 0 || value > 65536) return HFK_ERR_BAD_KNOB;
+            g_hbm_lds_bytes.store((int)value);
+            return HFK_OK;
         default:
             return HFK_ERR_BAD_KNOB;
     }
@@ -683,6 +929,11 @@ int64_t hfk_get_tuning(int knob) {
         case HFK_KNOB_SWAP_UNROLL: return g_swap_unroll.load();
         case HFK_KNOB_SWAP_PACE_MBPS: return g_swap_pace_mbps.load();
         case HFK_KNOB_LINK_MBPS: return current_link_mbps();
+        case HFK_KNOB_DUPLEX_WORKGROUPS: return g_duplex_workgroups.load();
+        case HFK_KNOB_THROUGHPUT_PACE_PERMILLE: return g_throughput_pace_permille.load();
+        case HFK_KNOB_HBM_LDS_BYTES: return g_hbm_lds_bytes.load();
+        case HFK_KNOB_PACED_UNROLL: return g_paced_unroll.load();
+        case HFK_KNOB_PACED_WORKGROUPS: return g_paced_workgroups.load();
         default: return HFK_ERR_BAD_KNOB;
     }
 }

@@ -225,6 +225,10 @@ inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_pt
         a.dst_plane_stride = n_blocks * block_bytes;
         a.dst_stride = block_bytes;
         a.dst_limit = kUnchecked;
+        // The copies that follow move staging[p][i] to the host whatever ids[i] was (the ids live on the
+        // device), so an entry the kernel cannot fill is zeroed rather than left holding an earlier
+        // transfer's bytes.
+        a.zero_skipped = 1;
     } else {
         a.dst_planes = static_cast<const uint64_t*>(dev_plane_ptrs);
         a.dst_ids = dev_block_ids;
@@ -236,6 +240,40 @@ inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_pt
         a.src_limit = kUnchecked;
     }
     return HFK_OK;
+}
+
+// Splitting one block table between two movers by the length of its runs of consecutive host slots.
+// A maximal run is entries first .. first + len - 1 with ids[i + 1] == ids[i] + 1. `f(first, len)` is
+// called for every maximal run in table order. The kernels classify a pair with run_length_capped()
+// (hfk_bodies.h), which gives min(cap, len) for the same maximal run: "long" means len >= min_run on
+// both sides.
+template <typename F>
+inline void for_each_host_run(const int64_t* ids, uint64_t n, F f) {
+    uint64_t first = 0;
+    while (first < n) {
+        uint64_t len = 1;
+        while (first + len < n && ids[first + len] == ids[first + len - 1] + 1) ++len;
+        f(first, len);
+        first += len;
+    }
+}
+
+// Blocks of the table that sit in runs of at least min_run entries.
+inline uint64_t blocks_in_long_runs(const int64_t* ids, uint64_t n, uint64_t min_run) {
+    uint64_t total = 0;
+    for_each_host_run(ids, n, [&](uint64_t, uint64_t len) {
+        if (len >= min_run) total += len;
+    });
+    return total;
+}
+
+// Restricts a planned block copy to the pairs in long (or short) runs of `run_ids`
+// (entry j at run_ids[j * a.id_stride], the table column that holds the host slots).
+template <typename IdT>
+inline void filter_runs(BlockCopyArgs<IdT>& a, RunFilter mode, const int64_t* run_ids, uint32_t min_run) {
+    a.run_mode = mode;
+    a.run_ids = run_ids;
+    a.run_min = min_run;
 }
 
 // Wide-row gather expressed as a single-plane block copy with dst block i = i.

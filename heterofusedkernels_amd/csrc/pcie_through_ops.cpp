@@ -4,7 +4,7 @@
 // (pcieThrough/csrc/host/gather_torch.cpp:60,
 //  pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:113-114);
 // multi_layer_block_table_transfer, swap_blocks, swap_blocks_duplex, swap_blocks_staged,
-// gather_blocks and gather_into are additive. Every op unpacks its tensors into
+// swap_blocks_auto, gather_blocks and gather_into are additive. Every op unpacks its tensors into
 // raw device-visible addresses, takes the current HIP stream of the device that
 // owns the device-side tensor, and calls the C-ABI of libhfk_hip.so; nothing is
 // allocated and nothing waits.
@@ -64,6 +64,11 @@ hfk_stream_t current_stream() {
 
 void check_status(int rc, const char* entry) {
     TORCH_CHECK(rc == 0, entry, " failed: ", hfk_status_string(rc), " (", rc, ")");
+}
+
+uint32_t flag_bits(int64_t flags, const char* op) {
+    TORCH_CHECK(flags >= 0 && flags <= 0xffffffffLL, op, ": flags out of range");
+    return static_cast<uint32_t>(flags);
 }
 
 uint32_t workgroup_cap(const std::optional<int64_t>& workgroups) {
@@ -129,15 +134,10 @@ void gather(const at::Tensor& gmEmbed, const at::Tensor& gmEmbedDst, const at::T
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(gmEmbedDst));
     const void* table = device_visible(gmEmbed, "gmEmbed");
     const void* ids = device_visible(gmIds, "gmIds");
-    // A table in host memory (the reference's embedding case) is read over the PCIe link: 64
-    // workgroups already run it at the link's rate (55-57 GB/s for 1 KiB rows), and every further one
-    // only slows kernels on other streams. Gathers of a few MiB keep one workgroup per chunk (they are
-    // over in tens of microseconds and a cap would only add a partly filled second round); a device
-    // table gets the library's HBM-sized grid.
-    const bool longHostGather = !gmEmbed.is_cuda() && numIds * rowBytes > (4ull << 20);
-    const uint32_t workgroups = longHostGather ? 64u : 0u;
+    // workgroups 0: the library sizes the grid for where the table lives (HBM, or host memory
+    // behind the PCIe link, the reference's embedding case).
     check_status(hfk_gather_rows(table, gmEmbedDst.data_ptr(), ids, gmIds.scalar_type() == at::kLong, numIds,
-                                 rowBytes, tableRows, workgroups, current_stream()),
+                                 rowBytes, tableRows, 0, current_stream()),
                  "hfk_gather_rows");
 }
 
@@ -181,7 +181,7 @@ void fused_memcpy_multi_layer_block_transfer(const at::Tensor& deviceBlockCacheP
 // deviceLayerCachePtrs[l] points at block 0 of layer l's cache [deviceBlocks][H, T, D].
 void multi_layer_block_table_transfer(const at::Tensor& deviceLayerCachePtrs, const at::Tensor& hostBlockPool,
                                       const at::Tensor& blockPairs, int64_t deviceBlockStride, int64_t deviceBlocks,
-                                      bool toHost, std::optional<int64_t> workgroups) {
+                                      bool toHost, std::optional<int64_t> workgroups, int64_t flags) {
     TORCH_CHECK(hostBlockPool.dim() == 5,
                 "hostBlockPool must be [blocks, blockSize, layers, heads, headDims], got ", hostBlockPool.dim(),
                 " dims");
@@ -207,7 +207,8 @@ void multi_layer_block_table_transfer(const at::Tensor& deviceLayerCachePtrs, co
                      device_visible(hostBlockPool, "hostBlockPool"), blockBytes,
                      static_cast<const int64_t*>(device_visible(blockPairs, "blockPairs")),
                      static_cast<uint64_t>(blockPairs.size(0)), static_cast<uint64_t>(hostBlockPool.size(0)),
-                     static_cast<uint64_t>(deviceBlocks), T, L, H, D, elem, toHost ? 1 : 0, cap, current_stream()),
+                     static_cast<uint64_t>(deviceBlocks), T, L, H, D, elem, toHost ? 1 : 0,
+                     flag_bits(flags, "multi_layer_block_table_transfer"), cap, current_stream()),
                  "hfk_multi_layer_block_table_transfer");
 }
 
@@ -250,7 +251,7 @@ void swap_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs,
 void swap_blocks_duplex(const at::Tensor& devicePlanePtrs, const at::Tensor& hostPlanePtrs,
                         const at::Tensor& outBlockPairs, const at::Tensor& inBlockPairs, int64_t blockBytes,
                         int64_t deviceBlockStride, int64_t hostBlockStride, int64_t deviceBlocks, int64_t hostBlocks,
-                        std::optional<int64_t> workgroups) {
+                        std::optional<int64_t> workgroups, int64_t flags) {
     check_ptr_table(devicePlanePtrs, "devicePlanePtrs");
     check_ptr_table(hostPlanePtrs, "hostPlanePtrs");
     check_ptr_table(outBlockPairs, "outBlockPairs");
@@ -287,7 +288,8 @@ void swap_blocks_duplex(const at::Tensor& devicePlanePtrs, const at::Tensor& hos
     in_move.src_blocks = static_cast<uint64_t>(hostBlocks);
     in_move.dst_blocks = static_cast<uint64_t>(deviceBlocks);
     check_status(hfk_swap_blocks_duplex(&out_move, &in_move, static_cast<uint32_t>(devicePlanePtrs.numel()),
-                                        static_cast<uint64_t>(blockBytes), workgroup_cap(workgroups), current_stream()),
+                                        static_cast<uint64_t>(blockBytes), flag_bits(flags, "swap_blocks_duplex"),
+                                        workgroup_cap(workgroups), current_stream()),
                  "hfk_swap_blocks_duplex");
 }
 
@@ -333,10 +335,63 @@ void swap_blocks_staged(const at::Tensor& devicePlanePtrs, const at::Tensor& hos
                  "hfk_swap_blocks_staged");
 }
 
+// Block-table swap that picks, per run of consecutive host slots, between the staged mover
+// (HBM kernel + DMA copies) and the direct one; see hfk_swap_blocks_auto. blockPairs rows are
+// (device_block, host_block) when toHost, (host_block, device_block) otherwise. hostPlaneAddrs
+// (CPU int64: host addresses of the planes), hostBlockIds (CPU int64: the host column of
+// blockPairs) and staging are optional; without them the whole table moves the direct way.
+void swap_blocks_auto(const at::Tensor& devicePlanePtrs, const at::Tensor& hostPlanePtrs, const at::Tensor& blockPairs,
+                      int64_t blockBytes, int64_t deviceBlockStride, int64_t hostBlockStride, bool toHost,
+                      const std::optional<at::Tensor>& hostPlaneAddrs, const std::optional<at::Tensor>& hostBlockIds,
+                      const std::optional<at::Tensor>& staging, int64_t deviceBlocks, int64_t hostBlocks,
+                      int64_t minRunBlocks, int64_t flags) {
+    check_ptr_table(devicePlanePtrs, "devicePlanePtrs");
+    check_ptr_table(hostPlanePtrs, "hostPlanePtrs");
+    check_ptr_table(blockPairs, "blockPairs");
+    TORCH_CHECK(devicePlanePtrs.is_cuda(), "devicePlanePtrs must be a device tensor");
+    TORCH_CHECK(devicePlanePtrs.numel() == hostPlanePtrs.numel(), "plane tables differ in length");
+    TORCH_CHECK(devicePlanePtrs.numel() <= 0xffffffffLL, "too many planes");
+    TORCH_CHECK(blockPairs.dim() == 2 && blockPairs.size(1) == 2, "blockPairs must be [n, 2]");
+    TORCH_CHECK(blockBytes > 0 && deviceBlockStride >= blockBytes && hostBlockStride >= blockBytes,
+                "swap_blocks_auto: strides must be at least blockBytes, blockBytes positive");
+    TORCH_CHECK(deviceBlocks >= 0 && hostBlocks >= 0, "swap_blocks_auto: block counts must be non-negative");
+    TORCH_CHECK(minRunBlocks >= 0 && minRunBlocks <= 0xffffffffLL, "swap_blocks_auto: minRunBlocks out of range");
+    const uint64_t planes = static_cast<uint64_t>(devicePlanePtrs.numel());
+    const uint64_t n = static_cast<uint64_t>(blockPairs.size(0));
+    void* const* host_addrs = nullptr;
+    const int64_t* host_ids = nullptr;
+    void* staging_ptr = nullptr;
+    uint64_t staging_bytes = 0;
+    if (hostPlaneAddrs.has_value() && hostBlockIds.has_value() && staging.has_value()) {
+        check_ptr_table(*hostPlaneAddrs, "hostPlaneAddrs");
+        check_ptr_table(*hostBlockIds, "hostBlockIds");
+        TORCH_CHECK(hostPlaneAddrs->device().is_cpu() && hostBlockIds->device().is_cpu(),
+                    "hostPlaneAddrs and hostBlockIds must be CPU tensors");
+        TORCH_CHECK(static_cast<uint64_t>(hostPlaneAddrs->numel()) == planes, "hostPlaneAddrs must hold one address per plane");
+        TORCH_CHECK(hostBlockIds->dim() == 1 && static_cast<uint64_t>(hostBlockIds->numel()) == n,
+                    "hostBlockIds must hold one slot per row of blockPairs");
+        TORCH_CHECK(staging->is_cuda() && staging->is_contiguous(), "staging must be a contiguous device tensor");
+        host_addrs = reinterpret_cast<void* const*>(hostPlaneAddrs->data_ptr<int64_t>());
+        host_ids = hostBlockIds->data_ptr<int64_t>();
+        staging_ptr = staging->data_ptr();
+        staging_bytes = static_cast<uint64_t>(staging->nbytes());
+    }
+    if (planes == 0 || n == 0) return;
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(devicePlanePtrs));
+    check_status(hfk_swap_blocks_auto(devicePlanePtrs.data_ptr(), device_visible(hostPlanePtrs, "hostPlanePtrs"),
+                                      host_addrs, static_cast<const int64_t*>(device_visible(blockPairs, "blockPairs")),
+                                      host_ids, static_cast<uint32_t>(planes), n, static_cast<uint64_t>(blockBytes),
+                                      static_cast<uint64_t>(deviceBlockStride), static_cast<uint64_t>(hostBlockStride),
+                                      static_cast<uint64_t>(deviceBlocks), static_cast<uint64_t>(hostBlocks),
+                                      staging_ptr, staging_bytes, toHost ? 1 : 0, static_cast<uint32_t>(minRunBlocks),
+                                      flag_bits(flags, "swap_blocks_auto"), current_stream()),
+                 "hfk_swap_blocks_auto");
+}
+
 // Shared-id block gather over planes; see hfk_gather_blocks.
 void gather_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtrs, const at::Tensor& blockIds,
                    int64_t blockBytes, int64_t srcBlockStride, int64_t srcBlocks,
-                   std::optional<int64_t> workgroups) {
+                   std::optional<int64_t> workgroups, int64_t flags) {
     check_ptr_table(dstPlanePtrs, "dstPlanePtrs");
     check_ptr_table(srcPlanePtrs, "srcPlanePtrs");
     check_ptr_table(blockIds, "blockIds");
@@ -353,7 +408,8 @@ void gather_blocks(const at::Tensor& dstPlanePtrs, const at::Tensor& srcPlanePtr
                           static_cast<const int64_t*>(device_visible(blockIds, "blockIds")),
                           static_cast<uint32_t>(dstPlanePtrs.numel()), static_cast<uint64_t>(blockIds.size(0)),
                           static_cast<uint64_t>(blockBytes), static_cast<uint64_t>(srcBlockStride),
-                          static_cast<uint64_t>(srcBlocks), workgroup_cap(workgroups), current_stream()),
+                          static_cast<uint64_t>(srcBlocks), flag_bits(flags, "gather_blocks"),
+                          workgroup_cap(workgroups), current_stream()),
         "hfk_gather_blocks");
 }
 
@@ -370,21 +426,25 @@ TORCH_LIBRARY(pcie_through, m) {
     m.def("gather_into(Tensor gmEmbed, Tensor(a!) gmEmbedDst, Tensor gmIds, int? aiv=None) -> ()");
     m.def(
         "multi_layer_block_table_transfer(Tensor deviceLayerCachePtrs, Tensor hostBlockPool, Tensor blockPairs, int "
-        "deviceBlockStride, int deviceBlocks=0, bool toHost=False, int? workgroups=None) -> ()");
+        "deviceBlockStride, int deviceBlocks=0, bool toHost=False, int? workgroups=None, int flags=0) -> ()");
     m.def(
         "swap_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockPairs, int blockBytes, int "
         "srcBlockStride, int dstBlockStride, int srcBlocks=0, int dstBlocks=0, int? workgroups=None, int flags=0) -> ()");
     m.def(
         "swap_blocks_duplex(Tensor devicePlanePtrs, Tensor hostPlanePtrs, Tensor outBlockPairs, Tensor inBlockPairs, int "
         "blockBytes, int deviceBlockStride, int hostBlockStride, int deviceBlocks=0, int hostBlocks=0, int? "
-        "workgroups=None) -> ()");
+        "workgroups=None, int flags=0) -> ()");
     m.def(
         "swap_blocks_staged(Tensor devicePlanePtrs, Tensor hostPlaneAddrs, Tensor deviceBlockIds, Tensor hostBlockIds, "
         "Tensor(a!) staging, int blockBytes, int deviceBlockStride, int hostBlockStride, bool toHost, int "
         "deviceBlocks=0, int hostBlocks=0, int? workgroups=None) -> ()");
     m.def(
         "gather_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockIds, int blockBytes, int "
-        "srcBlockStride, int srcBlocks=0, int? workgroups=None) -> ()");
+        "srcBlockStride, int srcBlocks=0, int? workgroups=None, int flags=0) -> ()");
+    m.def(
+        "swap_blocks_auto(Tensor devicePlanePtrs, Tensor hostPlanePtrs, Tensor blockPairs, int blockBytes, int "
+        "deviceBlockStride, int hostBlockStride, bool toHost, Tensor? hostPlaneAddrs=None, Tensor? hostBlockIds=None, "
+        "Tensor(a!)? staging=None, int deviceBlocks=0, int hostBlocks=0, int minRunBlocks=0, int flags=0) -> ()");
 }
 
 // PyTorch-ROCm files HIP tensors under the CUDA dispatch key. A call whose tensors
@@ -400,4 +460,5 @@ TORCH_LIBRARY_IMPL(pcie_through, CUDA, m) {
     m.impl("swap_blocks_duplex", TORCH_FN(pciethrough::swap_blocks_duplex));
     m.impl("swap_blocks_staged", TORCH_FN(pciethrough::swap_blocks_staged));
     m.impl("gather_blocks", TORCH_FN(pciethrough::gather_blocks));
+    m.impl("swap_blocks_auto", TORCH_FN(pciethrough::swap_blocks_auto));
 }

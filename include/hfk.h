@@ -29,7 +29,7 @@ extern "C" {
 #define HFK_API __attribute__((visibility("default")))
 
 #define HFK_VERSION_MAJOR 0
-#define HFK_VERSION_MINOR 1
+#define HFK_VERSION_MINOR 2
 
 /* A hipStream_t passed as an opaque pointer; NULL is the null stream. */
 typedef void* hfk_stream_t;
@@ -64,10 +64,11 @@ HFK_API const char* hfk_status_string(int status);
  *   ids         device-visible, int64 (ids_are_i64 != 0) or int32 indices
  *   table_rows  number of rows in table; an id outside [0, table_rows) leaves its
  *               dst row untouched. 0 disables the check (the reference never checks).
- *   workgroups  upper bound on workgroups launched, 0 = library default (sized for a table in
- *               device memory). For a long gather (more than a few MiB) out of a table in host
- *               memory pass 64: the PCIe link is saturated (55-57 GB/s for 1 KiB rows) and kernels
- *               on other streams are slowed 2x instead of 5x.
+ *   workgroups  upper bound on workgroups launched, 0 = library default: one workgroup per 16 KiB
+ *               of output for a table in device memory; for a table in host memory (the library
+ *               asks the runtime where `table` lives) a gather of more than 4 MiB runs on 64
+ *               workgroups, which saturate the PCIe link (55-57 GB/s for 1 KiB rows) and slow
+ *               kernels on other streams 2x where the device-sized grid slows them 5x.
  *
  * n_ids == 0 is a successful no-op. Rows of any byte size and alignment are
  * accepted; 16-byte aligned rows take the vectorised path.
@@ -137,6 +138,9 @@ HFK_API int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_pt
  *   block_pairs      device-visible int64 [n_pairs, 2] = (packed_block, dev_block)
  *   n_packed_blocks, n_dev_blocks  pool sizes; a pair outside them is skipped,
  *                    0 disables that side's check
+ *   flags            0, or HFK_SWAP_BESIDE_COMPUTE: other kernels run meanwhile and matter. Only the
+ *                    default grid changes (packed pool in host memory: 48 workgroups, 16 with the
+ *                    flag), never the result.
  * Strides must be at least one block of their side. Destination blocks must be distinct.
  */
 HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t dev_block_stride,
@@ -144,8 +148,8 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
                                          const int64_t* block_pairs, uint64_t n_pairs,
                                          uint64_t n_packed_blocks, uint64_t n_dev_blocks,
                                          uint32_t T, uint32_t L, uint32_t H, uint32_t D,
-                                         uint32_t elem_bytes, int to_packed, uint32_t workgroups,
-                                         hfk_stream_t stream);
+                                         uint32_t elem_bytes, int to_packed, uint32_t flags,
+                                         uint32_t workgroups, hfk_stream_t stream);
 
 /*
  * Block-table swap, all planes (layer x K/V) in one launch:
@@ -171,20 +175,21 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *                   HFK_SWAP_SRC_HOST        the source planes are host memory (swap-in)
  *                   HFK_SWAP_BESIDE_COMPUTE  other kernels run at the same time and matter
  *                 0 is always valid. The result never depends on flags; they select the launch
- *                 shape (grid, vectors in flight per lane, pacing). Measured on MI355X:
- *                 - without HFK_SWAP_BESIDE_COMPUTE the swap is drained as fast as the link allows
- *                   on 16 workgroups. Naming the host side makes it both faster and less of a
- *                   burden: toward the host the launch is paced at 0.90 of the link's raw rate
- *                   (HFK_KNOB_LINK_MBPS), which the link accepts better than an unbounded offer
- *                   (55.9-56.7 against 54.9-55.7 GB/s), from the host it keeps half as much in
- *                   flight (57.6 GB/s either way). A memory-bound kernel on another stream still
- *                   runs 1.2-1.8x slower meanwhile (2.3-3.1x with no side named; 4-5x beside a
- *                   64-workgroup grid: what a swap holds in flight beyond the link's
- *                   bandwidth-delay product queues in front of every other kernel's traffic);
- *                 - with HFK_SWAP_BESIDE_COMPUTE the swap runs 8-16 workgroups and, when
- *                   HFK_SWAP_DST_HOST says so, offers the host 0.84 of the link's raw rate:
- *                   52.8 GB/s out, 57.6 in, the neighbour's slowdown drops to 3-30 %. Name the
- *                   host side: without it the launch cannot pace (49.8 GB/s toward the host).
+ *                 shape (grid, vectors in flight per lane, pacing). Measured on MI355X, 32 KiB
+ *                 blocks, as own rate / slowdown of a 1 GiB device copy / of a bf16 8192^3 GEMM
+ *                 running on another stream meanwhile:
+ *                 - no flags: 16 workgroups x 8 vectors per lane, 55.4-55.7 GB/s out, 57.0-57.4 in;
+ *                   the copy beside it runs 6x slower, the GEMM 4.4x / 1.6x (out / in): what a swap
+ *                   holds in flight beyond the link's bandwidth-delay product queues in front of
+ *                   every other kernel's traffic.
+ *                 - HFK_SWAP_DST_HOST (swap-out): 16 workgroups x 1 vector per lane; a swap of 256 MiB
+ *                   or more is paced at 0.90 of the link's raw rate (HFK_KNOB_LINK_MBPS), which the
+ *                   link accepts better than an unbounded offer: 56.6 GB/s / 1.08x / 2.7x.
+ *                 - HFK_SWAP_SRC_HOST (swap-in): 40 x 1, unpaced: 57.4 GB/s / 1.95x / 1.6x.
+ *                 - with HFK_SWAP_BESIDE_COMPUTE as well: out on 12 x 1 paced at 0.84: 52.8 GB/s / 1.05x /
+ *                   1.64x; in on 24 x 1: 55.9 GB/s / 1.30x / 1.58x (1.55-1.6x is what any resident
+ *                   kernel costs this GEMM). Name the host side: without it the launch cannot
+ *                   pick these shapes (8 x 4 unpaced, 49.8 GB/s toward the host).
  *   workgroups    0 = the default of the mode chosen by flags; otherwise an upper bound on the
  *                 grid. The throughput default is sized for the PCIe link: pass a large bound
  *                 (e.g. 64 per CU) when both sides are device memory.
@@ -225,13 +230,16 @@ typedef struct hfk_block_move {
  * run in either order. The two moves must not touch the same bytes (no block may
  * be read by one and written by the other); either move may be empty (n_pairs 0).
  * `in_move` should be the one that reads host memory.
+ * flags: 0, or HFK_SWAP_BESIDE_COMPUTE (other kernels run meanwhile and matter): 16 workgroups
+ * instead of 32, one vector per lane and direction, and the launch offers the link 0.84 of its raw
+ * rate in each direction (see hfk_swap_blocks). The result never depends on flags.
  *
  * No counterpart in the reference (its transfer op is host -> device only and one
  * block per call, pcieThrough/tests/test_transfer_kernel.py:58-72).
  */
 HFK_API int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move* in_move,
-                                   uint32_t n_planes, uint64_t block_bytes, uint32_t workgroups,
-                                   hfk_stream_t stream);
+                                   uint32_t n_planes, uint64_t block_bytes, uint32_t flags,
+                                   uint32_t workgroups, hfk_stream_t stream);
 
 /*
  * Staged block-table swap: the compute units never touch host memory. Blocks travel
@@ -246,8 +254,8 @@ HFK_API int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_blo
  * spaced, else one copy per plane), so it is efficient when the host slots of a
  * transfer are (mostly) consecutive: 256 consecutive 32 KiB slots of 64 planes are
  * one 2-D copy of 64 rows of 8 MiB.
- * Result: identical to hfk_swap_blocks with the same table; staging holds the moved
- * blocks afterwards.
+ * Result: that of hfk_swap_blocks with the same table, with one exception on the way out (a
+ * device id out of range, below); staging holds the moved blocks afterwards.
  *
  * Why it exists: kernels on other streams run within a few per cent of their time alone beside
  * it (GEMM, device copy and attention kernels: 0.98-1.04x on MI355X), because the PCIe leg is
@@ -268,11 +276,11 @@ HFK_API int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_blo
  *   staging           device buffer of n_planes * n_blocks * block_bytes bytes
  *   dev_blocks / host_blocks  blocks per plane; 0 = unchecked. A host id out of range
  *                     rejects the call (HFK_ERR_OUT_OF_RANGE) before anything is enqueued.
- *                     A device id out of range is skipped by the kernel as everywhere
- *                     else; since the ids live on the device the copies cannot skip it
- *                     too, so on the way out its host slot receives whatever
- *                     staging[p][i] held before the call. Validate device ids upstream
- *                     if that matters.
+ *                     A device id out of range: on the way in the block is skipped, as
+ *                     everywhere else. On the way out the ids live on the device, so the
+ *                     copies cannot skip the entry; the kernel writes zeros to staging[p][i]
+ *                     instead and the host slot receives zeros (hfk_swap_blocks would leave
+ *                     the slot untouched). Bytes of an earlier transfer never reach the host.
  */
 HFK_API int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host_plane_addrs,
                                    const int64_t* dev_block_ids, const int64_t* host_block_ids,
@@ -282,39 +290,100 @@ HFK_API int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host
                                    int to_host, uint32_t workgroups, hfk_stream_t stream);
 
 /*
+ * Block-table swap that chooses the mover per run of host slots: the selection between the direct
+ * and the staged path that the reference leaves to its caller (its two ops
+ * multi_layer_block_transfer / fused_memcpy_multi_layer_block_transfer,
+ * pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:58-106, and the crossover its README
+ * measures, pcieThrough/tests/README.md:72-75), made per call and per run here.
+ *
+ *   - Runs of at least k consecutive host slots go the staged way: HBM gather/scatter kernel +
+ *     one 2-D DMA copy per run. Kernels on other streams do not notice them.
+ *   - Everything else goes the direct way, in one launch of the block-swap kernel that steps over
+ *     the pairs the copy engines took.
+ *   - With no staging buffer (NULL, or smaller than n_planes * n_pairs * block_bytes), or no host
+ *     arrays, the whole table goes the direct way: exactly hfk_swap_blocks with the host side named.
+ * k = min_run_blocks, or when that is 0 the smallest run whose single copy moves 16 MiB, with
+ * HFK_SWAP_BESIDE_COMPUTE 4 MiB. A copy costs the DMA engines about 9.5 us before its first byte, the
+ * link time of 0.5 MiB: runs of 16 MiB move at 97 % of the link rate, runs of 4 MiB at 88 %, single
+ * 2 MiB slots at 80 %. A swap that owns the GPU therefore keeps short runs on the compute units
+ * (k = 8 for 64 evenly spaced planes of 32 KiB blocks), one that shares it pays some of its own rate to
+ * keep the compute units off host memory (k = 2). min_run_blocks = 1 stages everything
+ * (hfk_swap_blocks_staged), above 1024 nothing.
+ *
+ *   dev_plane_ptrs    device-visible array of n_planes uint64 device addresses
+ *   host_plane_ptrs   device-visible array of n_planes uint64 mapped host addresses (direct mover)
+ *   host_plane_addrs  HOST array of n_planes host addresses of the same planes (copy engines); may be NULL
+ *   block_pairs       device-visible int64 [n_pairs, 2] = (src_block, dst_block):
+ *                     (device, host) when to_host != 0, (host, device) otherwise
+ *   host_block_ids    HOST int64 [n_pairs]: the host column of block_pairs, read before the call
+ *                     returns; may be NULL. It must equal that column: where the two disagree
+ *                     blocks end up unmoved or moved twice (never outside the pools: both
+ *                     copies are range-checked).
+ *   dev_blocks / host_blocks  blocks per plane; 0 = unchecked. With host arrays present, a host id
+ *                     out of range rejects the call (HFK_ERR_OUT_OF_RANGE) before anything is
+ *                     enqueued. A device id out of range: skipped on the way in; on the way out
+ *                     its host slot receives zeros, whichever mover had the pair.
+ *   staging           device buffer, or NULL; staging_bytes its size
+ *   flags             0 or HFK_SWAP_BESIDE_COMPUTE (shape of the direct launch, see hfk_swap_blocks;
+ *                     the host side is named by to_host)
+ * All work is enqueued on `stream` in order. Destination blocks must be distinct.
+ */
+HFK_API int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs,
+                                 void* const* host_plane_addrs, const int64_t* block_pairs,
+                                 const int64_t* host_block_ids, uint32_t n_planes, uint64_t n_pairs,
+                                 uint64_t block_bytes, uint64_t dev_block_stride,
+                                 uint64_t host_block_stride, uint64_t dev_blocks, uint64_t host_blocks,
+                                 void* staging, uint64_t staging_bytes, int to_host,
+                                 uint32_t min_run_blocks, uint32_t flags, hfk_stream_t stream);
+
+/*
  * Paged block gather over many planes in one launch:
  *   for p < n_planes, i < n_ids:
  *     dst_plane_ptrs[p][i*block_bytes ...] = src_plane_ptrs[p][ids[i]*src_block_stride ...]
  * i.e. hfk_gather_rows applied to every plane with a shared id list
  * (per plane: dst = src.index_select(0, ids)).
  * Same reference anchors as hfk_gather_rows; the plane loop is additive.
- * The default grid (workgroups 0) is sized for planes in device memory; when the source planes
- * are host memory this is a swap-in with consecutive destinations: pass workgroups 16, or use
- * hfk_swap_blocks, whose flags pick the launch shape.
+ *   flags  0 = source planes in device memory (grid of one workgroup per chunk, HBM-bound).
+ *          HFK_SWAP_SRC_HOST = the source planes are host memory: the gather is then a swap-in with
+ *          consecutive destinations and gets that launch shape (16 workgroups); with
+ *          HFK_SWAP_BESIDE_COMPUTE as well, the 8-16 workgroup shape. The result never depends on flags.
  */
 HFK_API int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs,
                       const int64_t* ids, uint32_t n_planes, uint64_t n_ids,
                       uint64_t block_bytes, uint64_t src_block_stride,
-                      uint64_t src_blocks, uint32_t workgroups, hfk_stream_t stream);
+                      uint64_t src_blocks, uint32_t flags, uint32_t workgroups,
+                      hfk_stream_t stream);
 
 /*
  * Benchmark/tuning knobs (process-wide, not thread-safe against concurrent
  * launches). Defaults are the measured best for MI355X.
  */
 enum hfk_knob {
-    HFK_KNOB_UNROLL = 0,        /* 16-byte accesses in flight per lane: 1, 2, 4, 8, 16  */
+    HFK_KNOB_UNROLL = 0,        /* 16-byte accesses in flight per lane of the HBM-bound launches
+                                   (gathers, staged swap's kernel): 1 (default), 2, 4, 8, 16 */
     HFK_KNOB_NONTEMPORAL = 1,   /* bit0: non-temporal loads, bit1: non-temporal stores */
     HFK_KNOB_WORKGROUPS_PER_CU = 2, /* default grid bound of the gathers and the
-                                       transfer = CUs * this, 1..1024                  */
+                                       transfer = CUs * this, 1..65536 (default 65536)  */
     HFK_KNOB_SWAP_WORKGROUPS = 3,   /* default grid bound of hfk_swap_blocks           */
     HFK_KNOB_DUPLEX_UNROLL = 4,     /* like HFK_KNOB_UNROLL, for hfk_swap_blocks_duplex */
     HFK_KNOB_SWAP_UNROLL = 5,       /* like HFK_KNOB_UNROLL, for hfk_swap_blocks (throughput mode) */
     HFK_KNOB_SWAP_PACE_MBPS = 6,    /* rate a HFK_SWAP_BESIDE_COMPUTE swap offers toward the host, MB/s;
                                        0 (default) = 84 % of HFK_KNOB_LINK_MBPS               */
-    HFK_KNOB_LINK_MBPS = 7          /* raw rate of the current device's PCIe link, MB/s. Default: lanes x
+    HFK_KNOB_LINK_MBPS = 7,         /* raw rate of the current device's PCIe link, MB/s. Default: lanes x
                                        GT/s x line encoding read from sysfs (0 if unreadable: such swaps
                                        then run unpaced). Setting it overrides every device; -1 restores
                                        the default                                                  */
+    HFK_KNOB_DUPLEX_WORKGROUPS = 8, /* default grid bound of hfk_swap_blocks_duplex                       */
+    HFK_KNOB_THROUGHPUT_PACE_PERMILLE = 9, /* share of HFK_KNOB_LINK_MBPS, in thousandths, that a swap-out or
+                                       duplex swap of 256 MiB or more offers toward the host when it is
+                                       not marked HFK_SWAP_BESIDE_COMPUTE; 0 = unpaced; default 900      */
+    HFK_KNOB_PACED_UNROLL = 11,     /* like HFK_KNOB_UNROLL, for the paced and the HFK_SWAP_BESIDE_COMPUTE launch
+                                       shapes of hfk_swap_blocks                                          */
+    HFK_KNOB_PACED_WORKGROUPS = 12, /* default grid of a paced swap toward the host (hfk_swap_blocks with
+                                       HFK_SWAP_DST_HOST)                                                  */
+    HFK_KNOB_HBM_LDS_BYTES = 10     /* dynamic LDS, 0..65536 bytes, that the HBM-bound launches (gathers, the
+                                       staged swap's kernel) request without using it: with 160 KiB of LDS
+                                       per compute unit it bounds the workgroups a unit holds at a time   */
 };
 HFK_API int hfk_set_tuning(int knob, int64_t value);
 HFK_API int64_t hfk_get_tuning(int knob);

@@ -78,6 +78,16 @@ void run_block_copy(BlockCopyArgs<IdT> a, int preferred_unroll, uint32_t grid_ca
     int unroll = 1;   // whole_chunks: as the launcher plans every role but the swap
     if (plan_block_copy<IdT>(a, preferred_unroll, &unroll, whole_chunks) != HFK_OK) { std::printf("plan failed\n"); ++g_failures; return; }
     const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+    if (a.run_mode != kAllPairs) {   // a split table runs the bodies built with the run filter, as the launcher does
+        switch (unroll) {
+            case 1: walk(a, grid, block_copy_body<IdT, 1, NT, true>); break;
+            case 2: walk(a, grid, block_copy_body<IdT, 2, NT, true>); break;
+            case 4: walk(a, grid, block_copy_body<IdT, 4, NT, true>); break;
+            case 8: walk(a, grid, block_copy_body<IdT, 8, NT, true>); break;
+            default: walk(a, grid, block_copy_body<IdT, 16, NT, true>); break;
+        }
+        return;
+    }
     switch (unroll) {
         case 1: walk(a, grid, block_copy_body<IdT, 1, NT>); break;
         case 2: walk(a, grid, block_copy_body<IdT, 2, NT>); break;
@@ -265,8 +275,11 @@ void case_stage(uint32_t n_planes, uint32_t n_blocks, uint64_t block_bytes, uint
     else run_block_copy<int64_t, 3>(a, unroll, grid_cap);
     for (uint32_t p = 0; p < n_planes; ++p)
         for (uint32_t i = 0; i < n_blocks; ++i) {
-            if (ids[i] < 0 || ids[i] >= (int64_t)dev_blocks) continue;
             uint8_t* st = staging_exp.p + ((uint64_t)p * n_blocks + i) * block_bytes;
+            if (ids[i] < 0 || ids[i] >= (int64_t)dev_blocks) {
+                if (to_staging) std::memset(st, 0, block_bytes);   // a slot the gather cannot fill is zeroed
+                continue;
+            }
             uint8_t* dv = dev_exp[p]->p + (uint64_t)ids[i] * ds;
             if (to_staging) std::memcpy(st, dv, block_bytes); else std::memcpy(dv, st, block_bytes);
         }
@@ -277,6 +290,109 @@ void case_stage(uint32_t n_planes, uint32_t n_blocks, uint64_t block_bytes, uint
     for (uint32_t p = 0; p < n_planes; ++p) expect_equal(dev[p]->p, dev_exp[p]->p, dev[p]->n, what);
     for (auto* b : dev) delete b;
     for (auto* b : dev_exp) delete b;
+}
+
+// ---- one block table split between two movers by run length (hfk_swap_blocks_auto) ----------
+// Long runs of consecutive host slots: kernel between device planes and staging + plain copies
+// (the copy engines' part, done here with memcpy per run exactly as copy_host_runs walks them);
+// everything else: the direct kernel with the complementary filter.
+void case_auto(uint32_t n_planes, uint32_t n_pairs, uint64_t block_bytes, uint32_t dev_blocks, uint32_t host_blocks,
+               bool to_host, uint32_t min_run, int unroll, uint32_t grid_cap, bool with_bad_dev) {
+    std::vector<Buf*> dev, host, dev_exp, host_exp;
+    std::vector<uint64_t> dp, hp;
+    for (uint32_t p = 0; p < n_planes; ++p) {
+        dev.push_back(new Buf(dev_blocks * block_bytes));
+        host.push_back(new Buf(host_blocks * block_bytes));
+        dev_exp.push_back(new Buf(dev_blocks * block_bytes));
+        host_exp.push_back(new Buf(host_blocks * block_bytes));
+        dev.back()->randomize();
+        host.back()->randomize();
+        std::memcpy(dev_exp.back()->p, dev.back()->p, dev.back()->n);
+        std::memcpy(host_exp.back()->p, host.back()->p, host.back()->n);
+        dp.push_back((uint64_t)(uintptr_t)dev.back()->p);
+        hp.push_back((uint64_t)(uintptr_t)host.back()->p);
+    }
+    // host slots: runs of random length at distinct places, in random order; device blocks distinct
+    std::vector<int64_t> host_ids;
+    {
+        std::vector<std::pair<int64_t, int64_t>> runs;   // (start, len) cut out of 0..host_blocks-1 left to right
+        int64_t at = 0;
+        while (at < (int64_t)host_blocks) {
+            const int64_t len = 1 + (int64_t)(rng() % 5);
+            const int64_t gap = 1 + (int64_t)(rng() % 2);        // a gap keeps neighbouring runs apart
+            if (at + len > (int64_t)host_blocks) break;
+            runs.push_back({at, len});
+            at += len + gap;
+        }
+        std::shuffle(runs.begin(), runs.end(), rng);
+        for (auto& r : runs)
+            for (int64_t i = 0; i < r.second && host_ids.size() < n_pairs; ++i) host_ids.push_back(r.first + i);
+    }
+    n_pairs = (uint32_t)host_ids.size();
+    std::vector<int64_t> dperm(dev_blocks);
+    for (uint32_t i = 0; i < dev_blocks; ++i) dperm[i] = i;
+    std::shuffle(dperm.begin(), dperm.end(), rng);
+    std::vector<int64_t> pairs(2 * (size_t)n_pairs), dev_ids(n_pairs);
+    for (uint32_t j = 0; j < n_pairs; ++j) {
+        dev_ids[j] = dperm[j % dev_blocks];
+        if (with_bad_dev && j % 4 == 1) dev_ids[j] = (j % 8 == 1) ? -2 : (int64_t)dev_blocks + 1;
+        pairs[2 * j] = to_host ? dev_ids[j] : host_ids[j];
+        pairs[2 * j + 1] = to_host ? host_ids[j] : dev_ids[j];
+    }
+    Buf staging((uint64_t)n_planes * n_pairs * block_bytes + 16);
+    staging.randomize();
+    // expected
+    for (uint32_t p = 0; p < n_planes; ++p)
+        for (uint32_t j = 0; j < n_pairs; ++j) {
+            uint8_t* h = host_exp[p]->p + (uint64_t)host_ids[j] * block_bytes;
+            const bool bad = dev_ids[j] < 0 || dev_ids[j] >= (int64_t)dev_blocks;
+            if (to_host) {
+                if (bad) std::memset(h, 0, block_bytes);
+                else std::memcpy(h, dev[p]->p + (uint64_t)dev_ids[j] * block_bytes, block_bytes);
+            } else if (!bad) {
+                std::memcpy(dev_exp[p]->p + (uint64_t)dev_ids[j] * block_bytes, h, block_bytes);
+            }
+        }
+    // the three steps, in the order the entry point enqueues them
+    const int64_t* host_column = pairs.data() + (to_host ? 1 : 0);
+    const int64_t* dev_column = pairs.data() + (to_host ? 0 : 1);
+    BlockCopyArgs<int64_t> direct, hbm;
+    int rc = to_host ? plan_swap_blocks(direct, hp.data(), dp.data(), pairs.data(), n_planes, n_pairs, block_bytes, block_bytes,
+                                        block_bytes, dev_blocks, host_blocks)
+                     : plan_swap_blocks(direct, dp.data(), hp.data(), pairs.data(), n_planes, n_pairs, block_bytes, block_bytes,
+                                        block_bytes, host_blocks, dev_blocks);
+    if (rc == HFK_OK) rc = plan_stage_blocks(hbm, dp.data(), staging.p, dev_column, n_planes, n_pairs, block_bytes, block_bytes,
+                                             dev_blocks, to_host);
+    if (rc != HFK_OK) { ++g_failures; std::printf("case_auto plan rc=%d\n", rc); return; }
+    direct.zero_skipped = to_host ? 1u : 0u;
+    hbm.id_stride = 2;
+    filter_runs(hbm, kLongRunsOnly, host_column, min_run);
+    filter_runs(direct, kShortRunsOnly, host_column, min_run);
+    auto copies = [&]() {
+        for_each_host_run(host_ids.data(), n_pairs, [&](uint64_t first, uint64_t len) {
+            if (len < min_run) return;
+            for (uint32_t p = 0; p < n_planes; ++p) {
+                uint8_t* h = host[p]->p + (uint64_t)host_ids[first] * block_bytes;
+                uint8_t* st = staging.p + ((uint64_t)p * n_pairs + first) * block_bytes;
+                if (to_host) std::memcpy(h, st, len * block_bytes); else std::memcpy(st, h, len * block_bytes);
+            }
+        });
+    };
+    if (to_host) { run_block_copy<int64_t, 3>(hbm, unroll, grid_cap, true); copies(); }
+    else { copies(); run_block_copy<int64_t, 3>(hbm, unroll, grid_cap, true); }
+    run_block_copy<int64_t, 3>(direct, unroll > 4 ? 4 : unroll, grid_cap > 16 ? 16 : grid_cap);
+    char what[192];
+    std::snprintf(what, sizeof what, "auto planes=%u pairs=%u bytes=%llu to_host=%d min_run=%u unroll=%d grid=%u bad=%d long=%llu",
+                  n_planes, n_pairs, (unsigned long long)block_bytes, (int)to_host, min_run, unroll, grid_cap, (int)with_bad_dev,
+                  (unsigned long long)blocks_in_long_runs(host_ids.data(), n_pairs, min_run));
+    for (uint32_t p = 0; p < n_planes; ++p) {
+        expect_equal(dev[p]->p, dev_exp[p]->p, dev[p]->n, what);
+        expect_equal(host[p]->p, host_exp[p]->p, host[p]->n, what);
+    }
+    for (auto* b : dev) delete b;
+    for (auto* b : host) delete b;
+    for (auto* b : dev_exp) delete b;
+    for (auto* b : host_exp) delete b;
 }
 
 // ---- gather_blocks (multi-plane, shared ids) -------------------------------
@@ -527,6 +643,16 @@ int main() {
             case_stage(2, 6, 16384, 8, 64, to_staging, unroll, 3, true);
             case_stage(1, 4, 4100, 6, 0, to_staging, unroll, 2, false);
         }
+
+    // one table split by run length between the staged and the direct mover
+    for (bool to_host : {true, false})
+        for (uint32_t min_run : {1u, 2u, 3u, 4u, 6u, 9u})
+            for (int unroll : {1, 4, 8}) {
+                case_auto(3, 20, 32768, 24, 40, to_host, min_run, unroll, 5, false);
+                case_auto(2, 30, 16384, 32, 60, to_host, min_run, unroll, 1000, true);
+                case_auto(2, 11, 73728, 12, 30, to_host, min_run, unroll, 16, true);
+                case_auto(1, 9, 4100, 10, 20, to_host, min_run, unroll, 3, false);
+            }
 
     // block-table transfer, both directions
     for (bool to_packed : {false, true}) {

@@ -40,10 +40,11 @@ def bytes_np(t):
 
 
 def swap(dst_tab, src_tab, pairs_dev, n_planes, block_bytes, src_stride=None, dst_stride=None, src_blocks=0,
-         dst_blocks=0, workgroups=0):
+         dst_blocks=0, workgroups=0, flags=0):
+    """flags: capi.SWAP_DST_HOST / SWAP_SRC_HOST / SWAP_BESIDE_COMPUTE; they pick the launch shape only."""
     rc = capi.swap_blocks(dst_tab.data_ptr(), src_tab.data_ptr(), pairs_dev.data_ptr(), n_planes,
                           pairs_dev.shape[0], block_bytes, src_stride or block_bytes, dst_stride or block_bytes,
-                          src_blocks, dst_blocks, workgroups, stream_handle())
+                          src_blocks, dst_blocks, workgroups, stream_handle(), flags)
     capi.check(rc, "hfk_swap_blocks")
 
 
@@ -54,7 +55,19 @@ def gather_rows(table, dst, ids, row_bytes, table_rows=0, workgroups=0):
     capi.check(rc, "hfk_gather_rows")
 
 
-def gather_blocks(dst_tab, src_tab, ids_dev, n_planes, block_bytes, src_stride=None, src_blocks=0, workgroups=0):
+def gather_blocks(dst_tab, src_tab, ids_dev, n_planes, block_bytes, src_stride=None, src_blocks=0, workgroups=0,
+                  flags=0):
     rc = capi.gather_blocks(dst_tab.data_ptr(), src_tab.data_ptr(), ids_dev.data_ptr(), n_planes, ids_dev.shape[0],
-                            block_bytes, src_stride or block_bytes, src_blocks, workgroups, stream_handle())
+                            block_bytes, src_stride or block_bytes, src_blocks, workgroups, stream_handle(), flags)
     capi.check(rc, "hfk_gather_blocks")
+
+
+def oracle_swap_planes(dst_before, src_planes, pairs, plane_ids):
+    """What the C oracle makes of planes `plane_ids`: dst_before / src_planes are lists of CPU uint8
+    tensors [blocks, block_bytes] (one per entry of plane_ids), pairs an int64 [n, 2] tensor.
+    Returns the expected destination planes as numpy arrays."""
+    from oracle import oracle as O
+
+    want = [d.numpy().copy() for d in dst_before]
+    O.c_swap_blocks(want, [s.numpy() for s in src_planes], pairs.cpu().numpy())
+    return want

@@ -45,7 +45,7 @@ def test_managed_memory_exports_every_declared_symbol():
 
 def test_capi_loads_and_reports():
     L = capi.load()
-    assert L.hfk_version() == 1
+    assert L.hfk_version() == 2
     assert capi.status_string(0) == "ok"
     assert "NULL" in capi.status_string(-1)
     assert capi.get_tuning(capi.KNOB_UNROLL) in (1, 2, 4, 8, 16)
@@ -95,6 +95,21 @@ def test_argument_errors_are_reported_before_any_gpu_work():
     assert capi.swap_blocks_duplex(bad, None, 4, 4096) == -1
     assert capi.multi_layer_block_table_transfer(8, 64, 8, 64, 0, 3, 0, 0, 2, 2, 2, 8, 1, False) == -1
     assert capi.multi_layer_block_table_transfer(8, 8, 8, 64, 8, 3, 0, 0, 2, 2, 2, 8, 1, False) == -2   # stride < block
+    # flags are checked first, on every entry point that takes them
+    assert capi.multi_layer_block_table_transfer(8, 64, 8, 64, 8, 3, 0, 0, 2, 2, 2, 8, 1, False, flags=1) == -6
+    assert capi.swap_blocks_duplex(None, None, 4, 4096, flags=capi.SWAP_DST_HOST) == -6
+    assert capi.swap_blocks_duplex(None, None, 4, 4096, flags=capi.SWAP_BESIDE_COMPUTE) == 0
+    assert capi.gather_blocks(8, 8, 8, 2, 2, 16, 16, flags=capi.SWAP_DST_HOST) == -6
+    assert capi.gather_blocks(0, 0, 0, 0, 0, 16, 16, flags=capi.SWAP_SRC_HOST | capi.SWAP_BESIDE_COMPUTE) == 0
+    # the run-splitting swap: flags, sizes and host slots are validated on the host
+    auto = dict(dev_planes=8, host_planes_mapped=8, host_plane_addrs=planes.ctypes.data, pairs=8,
+                host_ids=ids.ctypes.data, n_planes=2, n_pairs=3, block_bytes=64, dev_stride=64, host_stride=64,
+                dev_blocks=0, host_blocks=8, staging=8, staging_bytes=2 * 3 * 64, to_host=True)
+    assert capi.swap_blocks_auto(**auto) == -5                                      # host id 9 >= 8 host blocks
+    assert capi.swap_blocks_auto(**dict(auto, flags=capi.SWAP_SRC_HOST)) == -6
+    assert capi.swap_blocks_auto(**dict(auto, n_pairs=0)) == 0
+    assert capi.swap_blocks_auto(**dict(auto, block_bytes=0)) == -2
+    assert capi.swap_blocks_auto(**dict(auto, pairs=0)) == -1
 
 
 # ---- torch ops: schemas are the reference's ---------------------------------

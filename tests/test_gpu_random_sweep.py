@@ -160,8 +160,9 @@ def test_random_gather_rows_and_blocks(seed):
         ids64 = torch.from_numpy(ids.astype(np.int64)).to(DEV) if n else torch.zeros(1, dtype=torch.int64, device=DEV)
         stab = _table(_planes(src.addr, toff, n_planes, rows, stride))
         dtab = _table(_planes(out.addr, doff, n_planes, n, rb))
+        gflags = int(rng.choice([0, 0, capi.SWAP_SRC_HOST, capi.SWAP_SRC_HOST | capi.SWAP_BESIDE_COMPUTE]))   # launch shape only
         capi.check(capi.gather_blocks(dtab.data_ptr(), stab.data_ptr(), ids64.data_ptr(), n_planes, n, rb, stride, rows,
-                                      wg, stream_handle()), "hfk_gather_blocks")
+                                      wg, stream_handle(), gflags), "hfk_gather_blocks")
         torch.cuda.synchronize()
         want = out.before.copy()
         for p in range(n_planes):
@@ -201,8 +202,8 @@ def test_random_block_table_transfer(seed):
         lptrs = _table([layers.addr + l * dev_blocks * layer_bytes for l in range(L)])
         capi.check(capi.multi_layer_block_table_transfer(
             lptrs.data_ptr(), layer_bytes, packed.addr + poff, block_bytes, pairs_d.data_ptr() if pairs_d is not None else None,
-            pairs_all.shape[0], packed_blocks, dev_blocks, T, L, H, D, e, int(to_packed), wg, stream_handle()),
-            "hfk_multi_layer_block_table_transfer")
+            pairs_all.shape[0], packed_blocks, dev_blocks, T, L, H, D, e, int(to_packed), wg, stream_handle(),
+            int(rng.choice([0, capi.SWAP_BESIDE_COMPUTE]))), "hfk_multi_layer_block_table_transfer")
         torch.cuda.synchronize()
         want_layers = layers.before.copy().reshape(L, dev_blocks, layer_bytes)
         want_packed = packed.before.copy()
@@ -241,7 +242,8 @@ def test_random_duplex_and_staged(seed):
                             dev_blocks, host_blocks)
         im = capi.BlockMove(dtab.data_ptr(), htab.data_ptr(), pi.data_ptr() if n_in else None, n_in, hstride, dstride,
                             host_blocks, dev_blocks)
-        capi.check(capi.swap_blocks_duplex(om, im, n_planes, bb, wg, stream_handle()), "hfk_swap_blocks_duplex")
+        capi.check(capi.swap_blocks_duplex(om, im, n_planes, bb, wg, stream_handle(),
+                                           int(rng.choice([0, capi.SWAP_BESIDE_COMPUTE]))), "hfk_swap_blocks_duplex")
         torch.cuda.synchronize()
         want_host = _expect_swap(host.before, dev.before, hoff, doff, n_planes, host_blocks, dev_blocks, hstride, dstride, bb,
                                  out_pairs)
@@ -258,24 +260,120 @@ def test_random_duplex_and_staged(seed):
         if rng.integers(0, 2):
             host_ids = rng.permutation(host_blocks)[:n].astype(np.int64)          # scattered slots
         to_host = bool(rng.integers(0, 2))
-        announce("random staged seed %d case %d: %d blocks, to_host %s" % (seed, case, n, to_host))
+        bad_dev = bool(rng.integers(0, 2))
+        if bad_dev:         # a device id out of range: skipped on the way in, zeros in the host slot on the way out
+            dev_ids[rng.integers(0, n, 2)] = np.array([-1, dev_blocks], dtype=np.int64)[rng.integers(0, 2, 2)]
+        ok = (dev_ids >= 0) & (dev_ids < dev_blocks)
+        announce("random staged seed %d case %d: %d blocks, to_host %s, bad device ids %s" % (seed, case, n, to_host, bad_dev))
         dev2 = Arena(doff + n_planes * dev_blocks * dstride, False, rng)
         host2 = Arena(hoff + n_planes * host_blocks * hstride, True, rng)
-        staging = torch.zeros(n_planes * n * bb, dtype=torch.uint8, device=DEV)
+        staging = torch.full((n_planes * n * bb,), 0xC3, dtype=torch.uint8, device=DEV)
         dtab2 = _table(_planes(dev2.addr, doff, n_planes, dev_blocks, dstride))
         host_addrs = (ctypes.c_void_p * n_planes)(*_planes(host2.host_addr, hoff, n_planes, host_blocks, hstride))
         ids_d = torch.from_numpy(dev_ids).to(DEV)
-        capi.check(capi.swap_blocks_staged(dtab2.data_ptr(), host_addrs, ids_d.data_ptr(), host_ids.ctypes.data, n_planes, n,
-                                           bb, dstride, hstride, dev_blocks, host_blocks, staging.data_ptr(), int(to_host),
-                                           wg, stream_handle()), "hfk_swap_blocks_staged")
+        capi.check(capi.swap_blocks_staged(dtab2.data_ptr(), host_addrs, ids_d.data_ptr(), host_ids.ctypes.data,
+                                           n_planes, n, bb, dstride, hstride, dev_blocks, host_blocks,
+                                           staging.data_ptr(), int(to_host), wg, stream_handle()),
+                   "hfk_swap_blocks_staged")
         torch.cuda.synchronize()
         if to_host:
             want = _expect_swap(host2.before, dev2.before, hoff, doff, n_planes, host_blocks, dev_blocks, hstride, dstride,
-                                bb, np.stack([dev_ids, host_ids], 1))
+                                bb, np.stack([dev_ids, host_ids], 1)[ok])
+            for p in range(n_planes):
+                _view(want, hoff, p, host_blocks, hstride, bb)[host_ids[~ok]] = 0
             assert np.array_equal(host2.now(), want), "staged host side"
             assert np.array_equal(dev2.now(), dev2.before)
         else:
             want = _expect_swap(dev2.before, host2.before, doff, hoff, n_planes, dev_blocks, host_blocks, dstride, hstride,
-                                bb, np.stack([host_ids, dev_ids], 1))
+                                bb, np.stack([host_ids, dev_ids], 1)[ok])
             assert np.array_equal(dev2.now(), want), "staged device side"
             assert np.array_equal(host2.now(), host2.before)
+
+
+def _run_table(rng, n, blocks):
+    """n distinct slots out of `blocks`: runs of 1-6 consecutive slots, in random order."""
+    runs, at = [], 0
+    while at < blocks:
+        length = int(rng.integers(1, 7))
+        if at + length > blocks:
+            break
+        runs.append(np.arange(at, at + length, dtype=np.int64))
+        at += length + int(rng.integers(1, 3))      # a gap keeps neighbouring runs from joining up
+    order = rng.permutation(len(runs))
+    ids = np.concatenate([runs[i] for i in order]) if runs else np.zeros(0, dtype=np.int64)
+    return ids[:n]
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_swap_blocks_auto(seed):
+    """The run-splitting swap against the oracle: fragmented host slots, every threshold from "stage
+    everything" to "stage nothing", with and without a staging buffer, padded strides (2-D copies per
+    plane), planes that are not evenly spaced on the host, bad device ids."""
+    rng = np.random.default_rng(5000 + seed + 17 * SEED_OFFSET)
+    for case in range(CASES):
+        n_planes = int(rng.integers(1, 7))
+        dev_blocks, host_blocks = int(rng.integers(4, 40)), int(rng.integers(8, 60))
+        bb = int(rng.choice(BLOCK_BYTES))
+        dstride, hstride = bb + int(rng.choice(PADS)), bb + int(rng.choice(PADS))
+        doff, hoff = int(rng.choice(OFFSETS)), int(rng.choice(OFFSETS))
+        host_ids = _run_table(rng, int(rng.integers(1, min(dev_blocks, host_blocks) + 1)), host_blocks)
+        n = host_ids.shape[0]
+        dev_ids = rng.permutation(dev_blocks)[:n].astype(np.int64)
+        to_host = bool(rng.integers(0, 2))
+        bad_dev = bool(rng.integers(0, 2))
+        if bad_dev:
+            dev_ids[rng.integers(0, n, 2)] = np.array([-1, dev_blocks], dtype=np.int64)[rng.integers(0, 2, 2)]
+        ok = (dev_ids >= 0) & (dev_ids < dev_blocks)
+        min_run = int(rng.choice([0, 1, 2, 3, 4, 7, 5000]))
+        how = int(rng.integers(0, 4))       # 0: full arguments, 1: no staging, 2: staging too small, 3: no host arrays
+        flags = int(rng.choice([0, capi.SWAP_BESIDE_COMPUTE]))
+        plane_gap = int(rng.choice([0, 0, 64]))       # != 0: the last plane sits off the even spacing
+        announce("random auto seed %d case %d: %d planes, blocks %d/%d, %d B (strides %d/%d, offsets %d/%d), %d pairs, "
+                 "to_host %s, bad device ids %s, min_run %d, how %d, flags %d, plane gap %d"
+                 % (seed, case, n_planes, dev_blocks, host_blocks, bb, dstride, hstride, doff, hoff, n, to_host, bad_dev,
+                    min_run, how, flags, plane_gap))
+        dev = Arena(doff + n_planes * dev_blocks * dstride, False, rng)
+        host = Arena(hoff + n_planes * host_blocks * hstride + plane_gap, True, rng)
+        dev_addrs = _planes(dev.addr, doff, n_planes, dev_blocks, dstride)
+        host_offsets = [hoff + p * host_blocks * hstride + (plane_gap if p == n_planes - 1 and p > 0 else 0)
+                        for p in range(n_planes)]
+        dtab = _table(dev_addrs)
+        htab = _table([host.addr + o for o in host_offsets])
+        host_addrs = (ctypes.c_void_p * n_planes)(*[host.host_addr + o for o in host_offsets])
+        pairs = np.stack([dev_ids, host_ids] if to_host else [host_ids, dev_ids], 1).astype(np.int64)
+        pairs_d = torch.from_numpy(pairs).to(DEV)
+        staging = torch.full((max(n_planes * n * bb, 1),), 0xC3, dtype=torch.uint8, device=DEV)
+        staging_bytes = staging.numel() if how != 2 else max(staging.numel() - 1, 0)
+        capi.check(capi.swap_blocks_auto(dtab.data_ptr(), htab.data_ptr(), host_addrs if how != 3 else None,
+                                         pairs_d.data_ptr(), host_ids.ctypes.data if how != 3 else None, n_planes, n, bb,
+                                         dstride, hstride, dev_blocks, host_blocks,
+                                         staging.data_ptr() if how != 1 else None, staging_bytes if how != 1 else 0,
+                                         int(to_host), min_run, flags, stream_handle()), "hfk_swap_blocks_auto")
+        torch.cuda.synchronize()
+
+        def host_view(buf, p):
+            return np.lib.stride_tricks.as_strided(buf[host_offsets[p]:], shape=(host_blocks, bb), strides=(hstride, 1),
+                                                   writeable=True)
+
+        want_host, want_dev = host.before.copy(), dev.before.copy()
+        for p in range(n_planes):
+            d = _view(want_dev if not to_host else dev.before, doff, p, dev_blocks, dstride, bb)
+            h = host_view(want_host if to_host else host.before, p)
+            if to_host:
+                h[host_ids[ok]] = d[dev_ids[ok]]
+                h[host_ids[~ok]] = 0
+            else:
+                d[dev_ids[ok]] = h[host_ids[ok]]
+        # the same planes through the C oracle (contiguous copies of the strided views)
+        for p in range(n_planes):
+            if to_host:
+                chk = np.ascontiguousarray(host_view(host.before, p))
+                O.c_swap_blocks([chk], [np.ascontiguousarray(_view(dev.before, doff, p, dev_blocks, dstride, bb))], pairs[ok])
+                chk[host_ids[~ok]] = 0
+                assert np.array_equal(chk, host_view(want_host, p))
+            else:
+                chk = np.ascontiguousarray(_view(dev.before, doff, p, dev_blocks, dstride, bb))
+                O.c_swap_blocks([chk], [np.ascontiguousarray(host_view(host.before, p))], pairs[ok])
+                assert np.array_equal(chk, _view(want_dev, doff, p, dev_blocks, dstride, bb))
+        assert np.array_equal(host.now(), want_host), "host side"
+        assert np.array_equal(dev.now(), want_dev), "device side"
