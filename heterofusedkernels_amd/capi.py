@@ -27,6 +27,8 @@ KNOB_PACED_WORKGROUPS = 12
 SWAP_DST_HOST = 1
 SWAP_SRC_HOST = 2
 SWAP_BESIDE_COMPUTE = 4
+STATIC_STAGING_BYTES = 64 << 20
+ERR_STAGING_TOO_SMALL = -7
 
 
 class BlockMove(ctypes.Structure):
@@ -46,6 +48,7 @@ ENTRY_POINTS = (
     "hfk_swap_blocks",
     "hfk_swap_blocks_duplex",
     "hfk_swap_blocks_staged",
+    "hfk_swap_blocks_staged_static",
     "hfk_swap_blocks_auto",
     "hfk_gather_blocks",
     "hfk_set_tuning",
@@ -101,6 +104,8 @@ def load():
     L.hfk_swap_blocks_duplex.restype = ci
     L.hfk_swap_blocks_staged.argtypes = [vp, vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, vp, ci, u32, vp]
     L.hfk_swap_blocks_staged.restype = ci
+    L.hfk_swap_blocks_staged_static.argtypes = [vp, vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, ci, u32, vp]
+    L.hfk_swap_blocks_staged_static.restype = ci
     L.hfk_swap_blocks_auto.argtypes = [vp, vp, vp, vp, vp, u32, u64, u64, u64, u64, u64, u64, vp, u64, ci, u32, u32, vp]
     L.hfk_swap_blocks_auto.restype = ci
     L.hfk_gather_blocks.argtypes = [vp, vp, vp, u32, u64, u64, u64, u64, u32, u32, vp]
@@ -165,6 +170,14 @@ def swap_blocks_staged(dev_planes, host_plane_addrs, dev_ids, host_ids, n_planes
     return load().hfk_swap_blocks_staged(dev_planes, host_plane_addrs, dev_ids, host_ids, n_planes, n_blocks,
                                          block_bytes, dev_stride, host_stride, dev_blocks, host_blocks, staging,
                                          int(bool(to_host)), workgroups, stream)
+
+
+def swap_blocks_staged_static(dev_planes, host_plane_addrs, dev_ids, host_ids, n_planes, n_blocks, block_bytes,
+                              dev_stride, host_stride, dev_blocks, host_blocks, to_host, workgroups=0, stream=0):
+    """hfk_swap_blocks_staged through the library's own staging array (no staging argument, no allocation)."""
+    return load().hfk_swap_blocks_staged_static(dev_planes, host_plane_addrs, dev_ids, host_ids, n_planes, n_blocks,
+                                                block_bytes, dev_stride, host_stride, dev_blocks, host_blocks,
+                                                int(bool(to_host)), workgroups, stream)
 
 
 def swap_blocks_auto(dev_planes, host_planes_mapped, host_plane_addrs, pairs, host_ids, n_planes, n_pairs, block_bytes,

@@ -603,6 +603,31 @@ int staged_swap(const void* dev_plane_ptrs, void* const* host_plane_addrs, const
     return launch_block_copy<Role::kScatterBlocks, int64_t>(a, workgroups, s);
 }
 
+// ---- staging owned by the library, for callers that may not allocate ------
+// One array per device the library is loaded on, held until the process ends. In host code the
+// array's name stands for the symbol, not for device memory: the address kernels and copies use
+// is asked of the runtime once per device and kept.
+constexpr uint64_t kStaticStagingBytes = HFK_STATIC_STAGING_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticStagingBytes];
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int static_staging(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return HFK_ERR_TOO_LARGE;
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        // `dev` is current: the address returned is that of this device's copy of the array.
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // racing threads store the same address
+    }
+    *out = ptr;
+    return HFK_OK;
+}
+
 // A run of host slots is worth a DMA copy when one copy of it moves at least this much.
 constexpr uint64_t kDmaRunBytes = 16ull << 20;
 constexpr uint64_t kDmaRunBytesBesideCompute = 4ull << 20;
@@ -638,6 +663,8 @@ const char* hfk_status_string(int status) {
         case HFK_ERR_BAD_KNOB: return "hfk: unknown tuning knob or value out of range";
         case HFK_ERR_OUT_OF_RANGE: return "hfk: host-side index outside the declared range";
         case HFK_ERR_BAD_FLAGS: return "hfk: unknown flag bits";
+        case HFK_ERR_STAGING_TOO_SMALL:
+            return "hfk: transfer exceeds the library's static staging buffer (HFK_STATIC_STAGING_BYTES)";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -769,6 +796,26 @@ int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host_plane_a
                            uint64_t host_blocks, void* staging, int to_host, uint32_t workgroups,
                            hfk_stream_t stream) {
     if (n_planes == 0 || n_blocks == 0) return HFK_OK;
+    return staged_swap(dev_plane_ptrs, host_plane_addrs, dev_block_ids, host_block_ids, n_planes, n_blocks, block_bytes,
+                       dev_block_stride, host_block_stride, dev_blocks, host_blocks, staging, to_host, workgroups,
+                       static_cast<hipStream_t>(stream));
+}
+
+int hfk_swap_blocks_staged_static(const void* dev_plane_ptrs, void* const* host_plane_addrs,
+                                  const int64_t* dev_block_ids, const int64_t* host_block_ids, uint32_t n_planes,
+                                  uint64_t n_blocks, uint64_t block_bytes, uint64_t dev_block_stride,
+                                  uint64_t host_block_stride, uint64_t dev_blocks, uint64_t host_blocks, int to_host,
+                                  uint32_t workgroups, hfk_stream_t stream) {
+    if (n_planes == 0 || n_blocks == 0) return HFK_OK;
+    // n_planes * n_blocks * block_bytes <= kStaticStagingBytes, without overflowing on the way
+    if (block_bytes == 0) return HFK_ERR_BAD_SIZE;
+    if (block_bytes > kStaticStagingBytes || n_blocks > kStaticStagingBytes / block_bytes ||
+        (uint64_t)n_planes > kStaticStagingBytes / (n_blocks * block_bytes)) {
+        return HFK_ERR_STAGING_TOO_SMALL;
+    }
+    void* staging = nullptr;
+    int rc = static_staging(&staging);
+    if (rc != 0) return rc;
     return staged_swap(dev_plane_ptrs, host_plane_addrs, dev_block_ids, host_block_ids, n_planes, n_blocks, block_bytes,
                        dev_block_stride, host_block_stride, dev_blocks, host_blocks, staging, to_host, workgroups,
                        static_cast<hipStream_t>(stream));

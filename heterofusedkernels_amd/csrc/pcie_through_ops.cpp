@@ -4,7 +4,7 @@
 // (pcieThrough/csrc/host/gather_torch.cpp:60,
 //  pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:113-114);
 // multi_layer_block_table_transfer, swap_blocks, swap_blocks_duplex, swap_blocks_staged,
-// swap_blocks_auto, gather_blocks and gather_into are additive. Every op unpacks its tensors into
+// swap_blocks_staged_static, swap_blocks_auto, gather_blocks and gather_into are additive. Every op unpacks its tensors into
 // raw device-visible addresses, takes the current HIP stream of the device that
 // owns the device-side tensor, and calls the C-ABI of libhfk_hip.so; nothing is
 // allocated and nothing waits.
@@ -335,6 +335,40 @@ void swap_blocks_staged(const at::Tensor& devicePlanePtrs, const at::Tensor& hos
                  "hfk_swap_blocks_staged");
 }
 
+// The staged swap through the library's own staging array: no staging tensor, no allocation
+// (at most HFK_STATIC_STAGING_BYTES per call); see hfk_swap_blocks_staged_static.
+void swap_blocks_staged_static(const at::Tensor& devicePlanePtrs, const at::Tensor& hostPlaneAddrs,
+                               const at::Tensor& deviceBlockIds, const at::Tensor& hostBlockIds, int64_t blockBytes,
+                               int64_t deviceBlockStride, int64_t hostBlockStride, bool toHost, int64_t deviceBlocks,
+                               int64_t hostBlocks, std::optional<int64_t> workgroups) {
+    check_ptr_table(devicePlanePtrs, "devicePlanePtrs");
+    check_ptr_table(hostPlaneAddrs, "hostPlaneAddrs");
+    check_ptr_table(deviceBlockIds, "deviceBlockIds");
+    check_ptr_table(hostBlockIds, "hostBlockIds");
+    TORCH_CHECK(devicePlanePtrs.is_cuda(), "devicePlanePtrs must be a device tensor");
+    TORCH_CHECK(hostPlaneAddrs.device().is_cpu() && hostBlockIds.device().is_cpu(),
+                "hostPlaneAddrs and hostBlockIds must be CPU tensors");
+    TORCH_CHECK(devicePlanePtrs.numel() == hostPlaneAddrs.numel(), "plane tables differ in length");
+    TORCH_CHECK(devicePlanePtrs.numel() <= 0xffffffffLL, "too many planes");
+    TORCH_CHECK(deviceBlockIds.dim() == 1 && hostBlockIds.dim() == 1 && deviceBlockIds.numel() == hostBlockIds.numel(),
+                "deviceBlockIds and hostBlockIds must be 1-dimensional and equally long");
+    TORCH_CHECK(blockBytes > 0 && deviceBlockStride >= blockBytes && hostBlockStride >= blockBytes,
+                "swap_blocks_staged_static: strides must be at least blockBytes, blockBytes positive");
+    TORCH_CHECK(deviceBlocks >= 0 && hostBlocks >= 0, "swap_blocks_staged_static: block counts must be non-negative");
+    const uint64_t planes = static_cast<uint64_t>(devicePlanePtrs.numel());
+    const uint64_t n = static_cast<uint64_t>(deviceBlockIds.numel());
+    if (planes == 0 || n == 0) return;
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(devicePlanePtrs));
+    check_status(hfk_swap_blocks_staged_static(
+                     devicePlanePtrs.data_ptr(), reinterpret_cast<void* const*>(hostPlaneAddrs.data_ptr<int64_t>()),
+                     static_cast<const int64_t*>(device_visible(deviceBlockIds, "deviceBlockIds")),
+                     hostBlockIds.data_ptr<int64_t>(), static_cast<uint32_t>(planes), n,
+                     static_cast<uint64_t>(blockBytes), static_cast<uint64_t>(deviceBlockStride),
+                     static_cast<uint64_t>(hostBlockStride), static_cast<uint64_t>(deviceBlocks),
+                     static_cast<uint64_t>(hostBlocks), toHost ? 1 : 0, workgroup_cap(workgroups), current_stream()),
+                 "hfk_swap_blocks_staged_static");
+}
+
 // Block-table swap that picks, per run of consecutive host slots, between the staged mover
 // (HBM kernel + DMA copies) and the direct one; see hfk_swap_blocks_auto. blockPairs rows are
 // (device_block, host_block) when toHost, (host_block, device_block) otherwise. hostPlaneAddrs
@@ -442,6 +476,10 @@ TORCH_LIBRARY(pcie_through, m) {
         "gather_blocks(Tensor dstPlanePtrs, Tensor srcPlanePtrs, Tensor blockIds, int blockBytes, int "
         "srcBlockStride, int srcBlocks=0, int? workgroups=None, int flags=0) -> ()");
     m.def(
+        "swap_blocks_staged_static(Tensor devicePlanePtrs, Tensor hostPlaneAddrs, Tensor deviceBlockIds, Tensor "
+        "hostBlockIds, int blockBytes, int deviceBlockStride, int hostBlockStride, bool toHost, int deviceBlocks=0, int "
+        "hostBlocks=0, int? workgroups=None) -> ()");
+    m.def(
         "swap_blocks_auto(Tensor devicePlanePtrs, Tensor hostPlanePtrs, Tensor blockPairs, int blockBytes, int "
         "deviceBlockStride, int hostBlockStride, bool toHost, Tensor? hostPlaneAddrs=None, Tensor? hostBlockIds=None, "
         "Tensor(a!)? staging=None, int deviceBlocks=0, int hostBlocks=0, int minRunBlocks=0, int flags=0) -> ()");
@@ -460,5 +498,6 @@ TORCH_LIBRARY_IMPL(pcie_through, CUDA, m) {
     m.impl("swap_blocks_duplex", TORCH_FN(pciethrough::swap_blocks_duplex));
     m.impl("swap_blocks_staged", TORCH_FN(pciethrough::swap_blocks_staged));
     m.impl("gather_blocks", TORCH_FN(pciethrough::gather_blocks));
+    m.impl("swap_blocks_staged_static", TORCH_FN(pciethrough::swap_blocks_staged_static));
     m.impl("swap_blocks_auto", TORCH_FN(pciethrough::swap_blocks_auto));
 }

@@ -41,7 +41,8 @@ enum hfk_status {
     HFK_ERR_TOO_LARGE = -3,    /* a count exceeds what one launch can index      */
     HFK_ERR_BAD_KNOB = -4,     /* unknown tuning knob or value out of range      */
     HFK_ERR_OUT_OF_RANGE = -5, /* an index passed in host memory is out of range */
-    HFK_ERR_BAD_FLAGS = -6     /* a flags argument has unknown bits set            */
+    HFK_ERR_BAD_FLAGS = -6,    /* a flags argument has unknown bits set            */
+    HFK_ERR_STAGING_TOO_SMALL = -7 /* the transfer does not fit the library's static staging buffer */
 };
 
 /* HFK_VERSION_MAJOR * 1000 + HFK_VERSION_MINOR of the loaded library. */
@@ -288,6 +289,33 @@ HFK_API int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host
                                    uint64_t dev_block_stride, uint64_t host_block_stride,
                                    uint64_t dev_blocks, uint64_t host_blocks, void* staging,
                                    int to_host, uint32_t workgroups, hfk_stream_t stream);
+
+/*
+ * hfk_swap_blocks_staged without the staging argument and without any allocation: the staging
+ * buffer is an array of HFK_STATIC_STAGING_BYTES bytes that lives in the library's device image
+ * (one copy per GPU the library is used on, held until the process ends).
+ *
+ * No counterpart in the reference. It is for callers that cannot allocate or cannot keep a
+ * workspace alive: code that runs under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc. The call itself makes no hipMalloc / hipFree and calls no routine that does.
+ *
+ *   - n_planes * n_blocks * block_bytes must not exceed HFK_STATIC_STAGING_BYTES, else
+ *     HFK_ERR_STAGING_TOO_SMALL and nothing is enqueued.
+ *   - Every call on one GPU uses the same array: calls that overlap in time on one GPU (two
+ *     streams, two threads) race on it. Calls on one stream are ordered and safe.
+ *   - The array keeps the last call's blocks; nothing needs clearing between calls (every staging
+ *     byte that reaches a destination was written by the same call first).
+ *   - The first call on a device asks the runtime for that device's address of the array; make it
+ *     before a graph capture begins, not inside one.
+ * Everything else (arguments, order of operations, result) as hfk_swap_blocks_staged.
+ */
+#define HFK_STATIC_STAGING_BYTES (64ull << 20)
+HFK_API int hfk_swap_blocks_staged_static(const void* dev_plane_ptrs, void* const* host_plane_addrs,
+                                          const int64_t* dev_block_ids, const int64_t* host_block_ids,
+                                          uint32_t n_planes, uint64_t n_blocks, uint64_t block_bytes,
+                                          uint64_t dev_block_stride, uint64_t host_block_stride,
+                                          uint64_t dev_blocks, uint64_t host_blocks, int to_host,
+                                          uint32_t workgroups, hfk_stream_t stream);
 
 /*
  * Block-table swap that chooses the mover per run of host slots: the selection between the direct

@@ -52,6 +52,7 @@ def test_capi_loads_and_reports():
     assert capi.set_tuning(capi.KNOB_UNROLL, 3) == -4
     assert capi.set_tuning(99, 1) == -4
     assert "flag" in capi.status_string(-6)
+    assert "static staging" in capi.status_string(capi.ERR_STAGING_TOO_SMALL)
     # the PCIe link rate: an override is reported back, -1 returns to auto-detection (0 = unknown without a device)
     assert capi.set_tuning(capi.KNOB_LINK_MBPS, 31500) == 0
     assert capi.get_tuning(capi.KNOB_LINK_MBPS) == 31500
@@ -101,6 +102,13 @@ def test_argument_errors_are_reported_before_any_gpu_work():
     assert capi.swap_blocks_duplex(None, None, 4, 4096, flags=capi.SWAP_BESIDE_COMPUTE) == 0
     assert capi.gather_blocks(8, 8, 8, 2, 2, 16, 16, flags=capi.SWAP_DST_HOST) == -6
     assert capi.gather_blocks(0, 0, 0, 0, 0, 16, 16, flags=capi.SWAP_SRC_HOST | capi.SWAP_BESIDE_COMPUTE) == 0
+    # the staged swap through the library's own staging array: size limit and host arrays, before any GPU call
+    big = (8, planes.ctypes.data, 8, ids.ctypes.data, 2, 3, capi.STATIC_STAGING_BYTES // 4, 1 << 30, 1 << 30, 0, 8, True)
+    assert capi.swap_blocks_staged_static(*big) == capi.ERR_STAGING_TOO_SMALL      # 2 * 3 * 16 MiB > 64 MiB
+    assert capi.swap_blocks_staged_static(8, planes.ctypes.data, 8, ids.ctypes.data, 2, 0, 64, 64, 64, 0, 8, True) == 0
+    assert capi.swap_blocks_staged_static(8, planes.ctypes.data, 8, ids.ctypes.data, 2, 3, 0, 64, 64, 0, 8, True) == -2
+    assert capi.swap_blocks_staged_static(8, planes.ctypes.data, 8, ids.ctypes.data, 1 << 31, 1 << 40, 1 << 20, 1 << 20,
+                                          1 << 20, 0, 0, True) == capi.ERR_STAGING_TOO_SMALL   # no overflow on the way
     # the run-splitting swap: flags, sizes and host slots are validated on the host
     auto = dict(dev_planes=8, host_planes_mapped=8, host_plane_addrs=planes.ctypes.data, pairs=8,
                 host_ids=ids.ctypes.data, n_planes=2, n_pairs=3, block_bytes=64, dev_stride=64, host_stride=64,

@@ -264,17 +264,24 @@ def test_random_duplex_and_staged(seed):
         if bad_dev:         # a device id out of range: skipped on the way in, zeros in the host slot on the way out
             dev_ids[rng.integers(0, n, 2)] = np.array([-1, dev_blocks], dtype=np.int64)[rng.integers(0, 2, 2)]
         ok = (dev_ids >= 0) & (dev_ids < dev_blocks)
-        announce("random staged seed %d case %d: %d blocks, to_host %s, bad device ids %s" % (seed, case, n, to_host, bad_dev))
+        static = bool(rng.integers(0, 2)) and n_planes * n * bb <= capi.STATIC_STAGING_BYTES
+        announce("random staged seed %d case %d: %d blocks, to_host %s, bad device ids %s, library staging %s"
+                 % (seed, case, n, to_host, bad_dev, static))
         dev2 = Arena(doff + n_planes * dev_blocks * dstride, False, rng)
         host2 = Arena(hoff + n_planes * host_blocks * hstride, True, rng)
         staging = torch.full((n_planes * n * bb,), 0xC3, dtype=torch.uint8, device=DEV)
         dtab2 = _table(_planes(dev2.addr, doff, n_planes, dev_blocks, dstride))
         host_addrs = (ctypes.c_void_p * n_planes)(*_planes(host2.host_addr, hoff, n_planes, host_blocks, hstride))
         ids_d = torch.from_numpy(dev_ids).to(DEV)
-        capi.check(capi.swap_blocks_staged(dtab2.data_ptr(), host_addrs, ids_d.data_ptr(), host_ids.ctypes.data,
-                                           n_planes, n, bb, dstride, hstride, dev_blocks, host_blocks,
-                                           staging.data_ptr(), int(to_host), wg, stream_handle()),
-                   "hfk_swap_blocks_staged")
+        if static:
+            capi.check(capi.swap_blocks_staged_static(dtab2.data_ptr(), host_addrs, ids_d.data_ptr(), host_ids.ctypes.data,
+                                                      n_planes, n, bb, dstride, hstride, dev_blocks, host_blocks,
+                                                      int(to_host), wg, stream_handle()), "hfk_swap_blocks_staged_static")
+        else:
+            capi.check(capi.swap_blocks_staged(dtab2.data_ptr(), host_addrs, ids_d.data_ptr(), host_ids.ctypes.data,
+                                               n_planes, n, bb, dstride, hstride, dev_blocks, host_blocks,
+                                               staging.data_ptr(), int(to_host), wg, stream_handle()),
+                       "hfk_swap_blocks_staged")
         torch.cuda.synchronize()
         if to_host:
             want = _expect_swap(host2.before, dev2.before, hoff, doff, n_planes, host_blocks, dev_blocks, hstride, dstride,
