@@ -85,6 +85,7 @@ def build_managed_memory():
     _run(
         [
             "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__=1",
+            "-DHFK_MANAGED_MEM_NO_TORCH=1",   # the library itself is torch-free; its header serves both kinds of caller
             "-I" + os.path.join(ROCM, "include"), "-I" + INCLUDE, "-I" + CSRC,
             os.path.join(CSRC, "managed_mem.cpp"), "-o", MANAGED_MEMORY_SO,
             "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-pthread",

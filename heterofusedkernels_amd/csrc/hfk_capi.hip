@@ -220,6 +220,22 @@ int finish_launch() {
 // Raw PCIe rate of a device's link in MB/s (lanes x GT/s x line encoding), from sysfs; 0 if unknown.
 std::atomic<int> g_link_mbps[kMaxDevices];   // 0 = not read yet, -1 = unknown
 
+// One sysfs attribute of a PCI device as text ("" when unreadable).
+void read_pci_attribute(const char* bdf, const char* name, char* out, size_t out_size) {
+    out[0] = 0;
+    char path[160];
+    std::snprintf(path, sizeof(path), "/sys/bus/pci/devices/%s/%s", bdf, name);
+    if (FILE* f = std::fopen(path, "r")) {
+        if (std::fgets(out, (int)out_size, f) == nullptr) out[0] = 0;
+        std::fclose(f);
+    }
+}
+
+// The link's rate as trained at its best: a link that idles in a low-power speed, or that is read
+// while it retrains, reports less in current_link_* than it delivers under load, and a pace derived
+// from that would throttle every paced swap for the life of the process. A pace that is too high
+// degrades gracefully (the launch behaves like an unpaced one), one that is too low does not, so the
+// larger of the current and the maximum rate is used. HFK_KNOB_LINK_MBPS overrides both.
 int read_link_mbps(int dev) {
     char bdf[32] = {0};
     if (hipDeviceGetPCIBusId(bdf, (int)sizeof(bdf), dev) != hipSuccess) {
@@ -227,22 +243,14 @@ int read_link_mbps(int dev) {
         return -1;
     }
     for (char* c = bdf; *c; ++c) *c = (char)std::tolower((unsigned char)*c);
-    char path[128];
-    double gts = 0.0;
-    int width = 0;
-    std::snprintf(path, sizeof(path), "/sys/bus/pci/devices/%s/current_link_speed", bdf);
-    if (FILE* f = std::fopen(path, "r")) {
-        if (std::fscanf(f, "%lf", &gts) != 1) gts = 0.0;
-        std::fclose(f);
-    }
-    std::snprintf(path, sizeof(path), "/sys/bus/pci/devices/%s/current_link_width", bdf);
-    if (FILE* f = std::fopen(path, "r")) {
-        if (std::fscanf(f, "%d", &width) != 1) width = 0;
-        std::fclose(f);
-    }
-    if (gts <= 0.0 || width <= 0 || width > 32) return -1;
-    const double encoding = gts >= 8.0 ? 128.0 / 130.0 : 0.8;     // 8b/10b below 8 GT/s
-    return (int)(gts * 1000.0 * width * encoding / 8.0);
+    char speed[64], width[64];
+    read_pci_attribute(bdf, "current_link_speed", speed, sizeof(speed));
+    read_pci_attribute(bdf, "current_link_width", width, sizeof(width));
+    const int now = hfk::link_mbps_from_sysfs(speed, width);
+    read_pci_attribute(bdf, "max_link_speed", speed, sizeof(speed));
+    read_pci_attribute(bdf, "max_link_width", width, sizeof(width));
+    const int best = hfk::link_mbps_from_sysfs(speed, width);
+    return now > best ? now : best;
 }
 
 int current_link_mbps() {

@@ -4,6 +4,7 @@
 #pragma once
 
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "hfk.h"
 #include "hfk_bodies.h"
@@ -18,6 +19,20 @@ constexpr uint64_t kU32Max = 0xffffffffull;
 constexpr uint64_t kWideRowBytes = 4096;
 constexpr int kFlatUnroll = 4;
 constexpr int kTransposeUnroll = 4;
+
+// Raw rate of a PCIe link in MB/s (lanes x GT/s x line encoding / 8) from the two strings sysfs
+// shows for it, e.g. "32.0 GT/s PCIe" and "16"; -1 when either does not parse. Links below
+// 8 GT/s use 8b/10b encoding, faster ones 128b/130b.
+inline int link_mbps_from_sysfs(const char* speed_text, const char* width_text) {
+    if (speed_text == nullptr || width_text == nullptr) return -1;
+    char* end = nullptr;
+    const double gts = strtod(speed_text, &end);
+    if (end == speed_text || !(gts > 0.0) || gts > 1024.0) return -1;
+    const long width = strtol(width_text, &end, 10);
+    if (end == width_text || width <= 0 || width > 32) return -1;
+    const double encoding = gts >= 8.0 ? 128.0 / 130.0 : 0.8;
+    return (int)(gts * 1000.0 * (double)width * encoding / 8.0);
+}
 
 // A block smaller than 256 * unroll vectors would leave lanes idle, so the unroll
 // is halved until one chunk fits inside the block (down to 1).

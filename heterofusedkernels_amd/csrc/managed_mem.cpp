@@ -40,11 +40,11 @@ HostRegisteredMemoryManager::~HostRegisteredMemoryManager() { unregisterAll(); }
 
 int HostRegisteredMemoryManager::lastError() { return t_last_error; }
 
-const RegisteredMemoryRecord* HostRegisteredMemoryManager::findContaining(uintptr_t addr) const {
+RegisteredMemoryRecord* HostRegisteredMemoryManager::findContaining(uintptr_t addr) const {
     auto it = records_.upper_bound(addr);
     if (it == records_.begin()) return nullptr;
     --it;
-    const RegisteredMemoryRecord& r = it->second;
+    RegisteredMemoryRecord& r = it->second;
     return (addr - r.ptr < r.buffSize) ? &r : nullptr;
 }
 
@@ -59,7 +59,7 @@ bool HostRegisteredMemoryManager::overlapsOther(uintptr_t start, size_t size) co
     return false;
 }
 
-const RegisteredMemoryRecord* HostRegisteredMemoryManager::adoptMapping(void* hostPtr, void* devPtr,
+RegisteredMemoryRecord* HostRegisteredMemoryManager::adoptMapping(void* hostPtr, void* devPtr,
                                                                         size_t bufferSize, int32_t device,
                                                                         int32_t kind) {
     if (hostPtr == nullptr || devPtr == nullptr || bufferSize == 0) {
@@ -89,7 +89,7 @@ const RegisteredMemoryRecord* HostRegisteredMemoryManager::adoptMapping(void* ho
     return &ins.first->second;
 }
 
-const RegisteredMemoryRecord* HostRegisteredMemoryManager::registerHostPtr(void* hostPtr, size_t bufferSize) {
+RegisteredMemoryRecord* HostRegisteredMemoryManager::registerHostPtr(void* hostPtr, size_t bufferSize) {
     if (hostPtr == nullptr || bufferSize == 0) {
         t_last_error = HFK_MM_ERR_BAD_ARGUMENT;
         return nullptr;
@@ -100,7 +100,7 @@ const RegisteredMemoryRecord* HostRegisteredMemoryManager::registerHostPtr(void*
         auto hit = records_.find(start);
         if (hit != records_.end() && bufferSize <= hit->second.buffSize) return &hit->second;  // idempotent
         // A range inside an existing record is already device-visible.
-        const RegisteredMemoryRecord* outer = findContaining(start);
+        RegisteredMemoryRecord* outer = findContaining(start);
         if (outer != nullptr && start + bufferSize <= outer->ptr + outer->buffSize) return outer;
     }
 
@@ -110,67 +110,40 @@ const RegisteredMemoryRecord* HostRegisteredMemoryManager::registerHostPtr(void*
         device = -1;
     }
 
-    // Already pinned by someone else (hipHostMalloc, torch's pinned allocator)?
+    // The memory must be pinned already (hipHostMalloc, torch's pinned allocator, or a
+    // hipHostRegister the caller made itself): it is adopted through hipHostGetDevicePointer.
+    // This library never pins existing pageable memory. The runtime call that does so is refused
+    // on some platforms (and the error it leaves is reported by an unrelated later call), so a
+    // caller whose platform allows it registers the range itself and then hands it over; everyone
+    // else allocates with hfk_mm_alloc_pinned / alloc_numa_pinned_tensor.
     hipPointerAttribute_t attr;
     std::memset(&attr, 0, sizeof(attr));
     hipError_t e = hipPointerGetAttributes(&attr, hostPtr);
-    int32_t kind = HFK_MM_KIND_ADOPTED;
     if (e != hipSuccess) drop_hip_error();
     if (e != hipSuccess || attr.type != hipMemoryTypeHost) {
-        e = hipHostRegister(hostPtr, bufferSize, hipHostRegisterMapped | hipHostRegisterPortable);
-        if (e != hipSuccess) {
-            drop_hip_error();
-            t_last_error = static_cast<int>(e);
-            std::fprintf(stderr, "managed_memory: hipHostRegister(%p, %zu) failed: %s\n", hostPtr, bufferSize,
-                         hipGetErrorString(e));
-            return nullptr;
-        }
-        kind = HFK_MM_KIND_REGISTERED;
+        t_last_error = HFK_MM_ERR_NOT_PINNED;
+        return nullptr;
     }
     void* devPtr = nullptr;
     e = hipHostGetDevicePointer(&devPtr, hostPtr, 0);
     if (e != hipSuccess || devPtr == nullptr) {
         drop_hip_error();
-        if (kind == HFK_MM_KIND_REGISTERED) (void)hipHostUnregister(hostPtr);
         t_last_error = e != hipSuccess ? static_cast<int>(e) : HFK_MM_ERR_BAD_ARGUMENT;
         return nullptr;
     }
-    const RegisteredMemoryRecord* rec = adoptMapping(hostPtr, devPtr, bufferSize, device, kind);
-    if (rec == nullptr && kind == HFK_MM_KIND_REGISTERED) (void)hipHostUnregister(hostPtr);
-    return rec;
+    return adoptMapping(hostPtr, devPtr, bufferSize, device, HFK_MM_KIND_ADOPTED);
 }
 
 int HostRegisteredMemoryManager::unregisterHostPtr(void* hostPtr) {
     if (hostPtr == nullptr) return HFK_MM_ERR_BAD_ARGUMENT;
-    RegisteredMemoryRecord rec;
-    {
-        const std::unique_lock<std::shared_mutex> guard(mux_);
-        auto hit = records_.find(reinterpret_cast<uintptr_t>(hostPtr));
-        if (hit == records_.end()) return HFK_MM_OK;  // never registered: nothing to undo
-        rec = hit->second;
-        records_.erase(hit);
-    }
-    if (rec.kind == HFK_MM_KIND_REGISTERED) {
-        hipError_t e = hipHostUnregister(hostPtr);
-        if (e != hipSuccess) {
-            drop_hip_error();
-            return static_cast<int>(e);
-        }
-    }
-    return HFK_MM_OK;
+    const std::unique_lock<std::shared_mutex> guard(mux_);
+    records_.erase(reinterpret_cast<uintptr_t>(hostPtr));   // never registered: nothing to undo
+    return HFK_MM_OK;   // the pinning itself belongs to whoever made it (the allocator here, or the caller)
 }
 
 void HostRegisteredMemoryManager::unregisterAll() {
-    std::map<uintptr_t, RegisteredMemoryRecord> drained;
-    {
-        const std::unique_lock<std::shared_mutex> guard(mux_);
-        drained.swap(records_);
-    }
-    for (const auto& kv : drained) {
-        if (kv.second.kind == HFK_MM_KIND_REGISTERED) {
-            if (hipHostUnregister(reinterpret_cast<void*>(kv.first)) != hipSuccess) drop_hip_error();
-        }
-    }
+    const std::unique_lock<std::shared_mutex> guard(mux_);
+    records_.clear();
 }
 
 void* HostRegisteredMemoryManager::getDevicePtr(const void* hostPtr) const {
@@ -209,6 +182,17 @@ int unregister_ptr(void* ptr) { return HostRegisteredMemoryManager::GetInstance(
 uintptr_t get_device_ptr(uintptr_t ptr) {
     return reinterpret_cast<uintptr_t>(
         HostRegisteredMemoryManager::GetInstance().getDevicePtr(reinterpret_cast<const void*>(ptr)));
+}
+
+// The reference's allocator entry points (common/csrc/mem_alloc.cpp:66-115) under their own names.
+uintptr_t alloc_pinned_numa_ptr(std::size_t size, int numaNode) {
+    void* p = nullptr;
+    if (hfk_mm_alloc_pinned(size, numaNode, 0, &p) != HFK_MM_OK) return 0;
+    return reinterpret_cast<uintptr_t>(p);
+}
+
+void free_pinned_numa_ptr(void* ptr) {
+    if (ptr != nullptr) (void)hfk_mm_free_pinned(ptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -403,6 +387,9 @@ const char* hfk_mm_status_string(int status) {
         case HFK_MM_ERR_OVERLAP: return "managed_memory: range overlaps a different registration";
         case HFK_MM_ERR_NOT_FOUND: return "managed_memory: pointer is not registered";
         case HFK_MM_ERR_OS: return "managed_memory: operating-system call failed";
+        case HFK_MM_ERR_NOT_PINNED:
+            return "managed_memory: the range is not pinned host memory (allocate it with hfk_mm_alloc_pinned / "
+                   "alloc_numa_pinned_tensor, or pin it yourself before registering it)";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));

@@ -17,6 +17,7 @@
 #include <optional>
 
 #include "hfk.h"
+#define HFK_MANAGED_MEM_NO_TORCH 1   // only the manager is used here; keeps pybind11 out of this library
 #include "managed_mem.h"
 
 namespace pciethrough {

@@ -26,13 +26,15 @@ enum hfk_mm_status {
     HFK_MM_ERR_BAD_ARGUMENT = -1, /* null pointer or zero size                           */
     HFK_MM_ERR_OVERLAP = -2,      /* range overlaps a different existing registration   */
     HFK_MM_ERR_NOT_FOUND = -3,
-    HFK_MM_ERR_OS = -4            /* mmap / sysfs / policy failure, see errno           */
+    HFK_MM_ERR_OS = -4,           /* mmap / sysfs / policy failure, see errno           */
+    HFK_MM_ERR_NOT_PINNED = -5    /* the range is pageable memory: this library adopts pinned
+                                     memory and allocates its own, it never pins existing memory */
 };
 
 /* How a record came to exist; decides what unregistering undoes. */
 enum hfk_mm_kind {
     HFK_MM_KIND_ALLOCATED = 0,  /* hfk_mm_alloc_pinned: freed with the allocation        */
-    HFK_MM_KIND_REGISTERED = 1, /* hipHostRegister done here: hipHostUnregister on drop  */
+    HFK_MM_KIND_REGISTERED = 1, /* unused (kept for numbering): this library pins nothing itself */
     HFK_MM_KIND_ADOPTED = 2     /* already pinned elsewhere / caller-supplied mapping    */
 };
 
@@ -40,9 +42,11 @@ enum hfk_mm_kind {
 #define HFK_MM_ALLOC_NONCOHERENT 1u /* coarse-grained (GPU-cacheable) host memory */
 
 /*
- * Make [host_ptr, host_ptr + bytes) device-visible and record it.
- * Memory that is already pinned (hipHostMalloc, torch pin_memory) is adopted via
- * hipHostGetDevicePointer; anything else goes through hipHostRegister(Mapped).
+ * Record [host_ptr, host_ptr + bytes) and the address kernels use for it.
+ * The memory must be pinned already (hipHostMalloc, torch pin_memory, or a
+ * hipHostRegister(Mapped) the caller made itself on a platform that allows it); it is
+ * adopted via hipHostGetDevicePointer. Pageable memory is refused with
+ * HFK_MM_ERR_NOT_PINNED and leaves no record: use hfk_mm_alloc_pinned instead.
  * Registering the same start address again returns the existing record.
  * Replaces common/csrc/managed_memory/managed_mem.cpp:45-66 (`registerHostPtr`)
  * and :305-323 (`register_ptr`).
@@ -57,8 +61,8 @@ HFK_MM_API int hfk_mm_register(void* host_ptr, size_t bytes, void** dev_ptr_out)
 HFK_MM_API int hfk_mm_adopt(void* host_ptr, void* dev_ptr, size_t bytes, int device);
 
 /*
- * Drop the record that starts at host_ptr (undoing hipHostRegister if this
- * library did it). Unknown pointers are not an error.
+ * Drop the record that starts at host_ptr (the pinning stays with whoever made it).
+ * Unknown pointers are not an error.
  * Replaces managed_mem.cpp:105-118 (`aclUnregisterHostPtr`), :325-334 (`unregister_ptr`).
  */
 HFK_MM_API int hfk_mm_unregister(void* host_ptr);

@@ -557,7 +557,31 @@ void case_transpose_table(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32
 
 }  // namespace
 
+// the PCIe link-rate parser on the strings sysfs shows
+void case_link_rate() {
+    struct { const char* speed; const char* width; int want; } rows[] = {
+        {"32.0 GT/s PCIe\n", "16\n", 63015},      // Gen5 x16: 32 * 16 * 128/130 / 8 GB/s
+        {"16.0 GT/s PCIe", "16", 31507},           // Gen4 x16
+        {"8.0 GT/s PCIe", "8", 7876},              // Gen3 x8
+        {"5.0 GT/s PCIe", "16", 8000},             // Gen2: 8b/10b encoding
+        {"2.5 GT/s PCIe", "1", 250},
+        {"64.0 GT/s PCIe", "16", 126030},
+        {"Unknown", "16", -1}, {"", "16", -1}, {"32.0 GT/s PCIe", "", -1}, {"32.0 GT/s PCIe", "0", -1},
+        {"32.0 GT/s PCIe", "64", -1}, {"-8.0 GT/s", "16", -1}, {nullptr, "16", -1}, {"32.0 GT/s", nullptr, -1},
+    };
+    for (const auto& r : rows) {
+        ++g_cases;
+        const int got = link_mbps_from_sysfs(r.speed, r.width);
+        if (got != r.want) {
+            std::printf("FAIL link rate '%s' x '%s': got %d, want %d\n", r.speed ? r.speed : "(null)",
+                        r.width ? r.width : "(null)", got, r.want);
+            ++g_failures;
+        }
+    }
+}
+
 int main() {
+    case_link_rate();
     // swap: aligned fast path, every unroll, grid smaller and larger than the work
     for (int unroll : {1, 2, 4, 8, 16})
         for (uint32_t grid : {1u, 7u, 4096u}) {

@@ -41,6 +41,27 @@ def test_managed_memory_exports_every_declared_symbol():
     names = _declared("hfk_managed_memory.h", "HFK_MM_API")
     assert len(names) == 11
     assert set(names) <= _exported(_build.MANAGED_MEMORY_SO)
+    # ... and the reference's C++ free functions, under their own (mangled) names
+    cxx = subprocess.check_output(["nm", "-D", "-C", "--defined-only", _build.MANAGED_MEMORY_SO], text=True)
+    for name in ("register_ptr(void*, unsigned long)", "unregister_ptr(void*)", "get_device_ptr(unsigned long)",
+                 "alloc_pinned_numa_ptr(unsigned long, int)", "free_pinned_numa_ptr(void*)"):
+        assert name in cxx, name
+
+
+def test_reference_style_native_consumer_compiles():
+    """A C++ file that uses the registry header exactly as the reference's sources do (same include,
+    same calls, same types) compiles against the header shipped in the heterofusedkernels package."""
+    from torch.utils import cpp_extension
+    import sysconfig
+
+    shipped = os.path.join(heterofusedkernels_amd.DROPIN_DIR, "heterofusedkernels", "include")
+    assert os.path.exists(os.path.join(shipped, "managed_mem.h"))
+    cmd = ["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-Werror", "-Wno-deprecated-declarations", "-DUSE_ROCM=1",
+           "-D__HIP_PLATFORM_AMD__=1", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), "-I" + shipped]
+    cmd += ["-I" + p for p in cpp_extension.include_paths("cuda")] + ["-I" + sysconfig.get_paths()["include"]]
+    cmd.append(os.path.join(ROOT, "tests", "compat", "reference_style_consumer.cpp"))
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout[-3000:]
 
 
 def test_capi_loads_and_reports():
@@ -168,6 +189,26 @@ def test_package_layout():
     for name in ("alloc_numa_pinned_tensor", "host_register", "get_device_ptr"):  # common/csrc/pybind.cpp:8-10
         assert callable(getattr(memory, name))
     assert os.path.dirname(pkg) == heterofusedkernels_amd.DROPIN_DIR
+
+
+def test_pageable_memory_is_refused_and_leaves_no_record():
+    """The library adopts pinned memory and allocates its own; it never pins existing pageable memory."""
+    L = ctypes.CDLL(_build.MANAGED_MEMORY_SO)
+    L.hfk_mm_register.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]
+    L.hfk_mm_get_device_ptr.argtypes = [ctypes.c_void_p]
+    L.hfk_mm_get_device_ptr.restype = ctypes.c_void_p
+    L.hfk_mm_record_count.restype = ctypes.c_size_t
+    L.hfk_mm_status_string.restype = ctypes.c_char_p
+    text = open(os.path.join(ROOT, "include", "hfk_managed_memory.h")).read()
+    not_pinned = int(re.search(r"HFK_MM_ERR_NOT_PINNED = (-\d+)", text).group(1))
+    buf = ctypes.create_string_buffer(1 << 16)             # plain malloc'd memory
+    before = L.hfk_mm_record_count()
+    dev = ctypes.c_void_p(0)
+    assert L.hfk_mm_register(buf, len(buf), ctypes.byref(dev)) == not_pinned
+    assert not dev.value
+    assert L.hfk_mm_record_count() == before
+    assert not L.hfk_mm_get_device_ptr(ctypes.addressof(buf))
+    assert b"alloc_pinned" in L.hfk_mm_status_string(not_pinned)
 
 
 # ---- registry (no HIP call is made by adopt / lookup) ------------------------

@@ -139,6 +139,31 @@ def test_gather_from_registered_host_table(memory, bs, id_dtype):
     assert torch.equal(dst2.cpu().view(torch.int16), dst.cpu().view(torch.int16))
 
 
+def test_gather_from_reference_scale_host_table(memory):
+    """The reference's own table: [4 000 000, 512] fp16 (4 GB) in registered host memory, int64 ids on
+    the device, aiv=4 and default (pcieThrough/tests/test_gather.py:35-58), at batch sizes from its loop
+    (8 .. 2040 in steps of 8) and with random rows instead of its all-zero table."""
+    rows, dim = 4000000, 512
+    announce("host-table gather out of the reference's 4 000 000 x 512 fp16 table")
+    embed = _pinned(memory, rows * dim * 2).view(torch.float16).view(rows, dim)
+    part = 500000                                               # random bytes made on the device, copied over
+    for first in range(0, rows, part):
+        chunk = torch.randint(0, 256, (part, dim * 2), dtype=torch.uint8, device=DEV,
+                              generator=torch.Generator(device=DEV).manual_seed(first))
+        embed[first:first + part].view(torch.uint8).copy_(chunk)
+    gen = torch.Generator().manual_seed(4000000)
+    for bs in (8, 16, 128, 1024, 2040):
+        ids = torch.randint(0, rows, (bs,), generator=gen, dtype=torch.int64)
+        ids[0], ids[-1] = 0, rows - 1                           # both ends of the table
+        for aiv in (4, None):
+            dst = torch.zeros(bs, dim, dtype=torch.float16, device=DEV)
+            torch.ops.pcie_through.gather(embed, dst, ids.to(DEV), aiv=aiv)
+            torch.cuda.synchronize()
+            want = embed[ids]                                   # tests/test_memcpy.py:18
+            assert np.array_equal(bytes_np(dst), bytes_np(want)), "bs %d aiv %s" % (bs, aiv)
+        assert np.array_equal(bytes_np(dst), O.c_gather_rows(bytes_np(embed), ids.numpy())), "bs %d vs oracle" % bs
+
+
 def test_gather_from_torch_pinned_table_without_registration(memory):
     """A tensor pinned by torch itself can be handed to the op directly; nothing is recorded for it."""
     announce("host-table gather from a torch.pin_memory() tensor, never registered")

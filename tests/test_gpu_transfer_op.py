@@ -28,7 +28,7 @@ def memory():
 @pytest.mark.parametrize("layers", [1, 32, 64])
 @pytest.mark.parametrize("heads", [1, 8])               # 8: the README's second geometry (tests/README.md:73,75)
 @pytest.mark.parametrize("head_dim", [128])
-@pytest.mark.parametrize("num_blocks", [1, 8])
+@pytest.mark.parametrize("num_blocks", [1, 8, 16])       # tests/test_transfer_kernel.py:19
 @pytest.mark.parametrize("use_fused_copy", [False, True])
 def test_multi_layer_block_kv_transfer(memory, block_size, layers, heads, head_dim, num_blocks, use_fused_copy):
     device = "cuda"
