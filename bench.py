@@ -812,7 +812,7 @@ def main():
     out_kernel_gbps = rate(w_payload, kernel_ms_out)
     in_kernel_gbps = rate(w_payload, kernel_ms_in)
     gather_alg_bytes = 2 * w_payload + 8 * headline_config["blocks_per_launch"]
-    paced = (args.out_flags & capi.SWAP_DST_HOST) and link_known and w_payload >= (256 << 20) and \
+    paced = (args.out_flags & capi.SWAP_DST_HOST) and link_known and w_payload >= (64 << 20) and \
         capi.get_tuning(capi.KNOB_THROUGHPUT_PACE_PERMILLE) > 0
     result = {
         "metric": "KV swap GB/s (% of PCIe5 x16 peak); block gather GB/s (% of HBM peak)",

@@ -128,6 +128,7 @@ constexpr uint32_t kTransferWorkgroups = 48;
 constexpr uint32_t kSingleBlockTransferWorkgroups = 128;
 constexpr uint32_t kHostGatherWorkgroups = 64;
 constexpr uint64_t kLongHostGatherBytes = 4ull << 20;
+constexpr uint64_t kAskTableSideBytes = 64ull << 10;
 // The duplex swap wants little in flight per workgroup: one vector per lane and direction
 // (unroll 8 loses 6 %). 32 workgroups reach 98.1-98.4 GB/s summed for 16, 32 and 72 KiB
 // blocks; 40-64 dip to 89-94, 96-192 are a flat 98-99.
@@ -175,7 +176,7 @@ int named_side_unroll() { return g_paced_unroll.load(std::memory_order_relaxed);
 constexpr double kPaceShareOfLink = 0.84;
 // Share offered by a throughput-mode swap-out: the cap itself (HFK_KNOB_THROUGHPUT_PACE_PERMILLE, default 0.90).
 double throughput_share_of_link() { return g_throughput_pace_permille.load(std::memory_order_relaxed) / 1000.0; }
-constexpr uint64_t kPaceFromBytes = 256ull << 20;
+constexpr uint64_t kPaceFromBytes = 64ull << 20;
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
@@ -345,42 +346,49 @@ void launch_duplex_nt(const DuplexCopyArgs& a, uint32_t grid, int nt, hipStream_
 }
 
 // ---- flat gather ----------------------------------------------------------
-template <typename V, typename IdT, typename IndexT>
-void launch_flat_gather_v(const FlatGatherArgs<IdT>& a, uint32_t grid, int nt, hipStream_t s) {
+template <typename V, typename IdT, typename IndexT, int UNROLL>
+void launch_flat_gather_u(const FlatGatherArgs<IdT>& a, uint32_t grid, int nt, hipStream_t s) {
     if (nt & 3) {
-        hipLaunchKernelGGL((flat_gather_kernel<V, IdT, IndexT, hfk::kFlatUnroll, 3>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((flat_gather_kernel<V, IdT, IndexT, UNROLL, 3>), dim3(grid), dim3(256), 0, s, a);
     } else {
-        hipLaunchKernelGGL((flat_gather_kernel<V, IdT, IndexT, hfk::kFlatUnroll, 0>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((flat_gather_kernel<V, IdT, IndexT, UNROLL, 0>), dim3(grid), dim3(256), 0, s, a);
     }
+}
+
+template <typename V, typename IdT, typename IndexT>
+void launch_flat_gather_v(const FlatGatherArgs<IdT>& a, uint32_t grid, int nt, int unroll, hipStream_t s) {
+    if (unroll == hfk::kFlatUnrollHost) launch_flat_gather_u<V, IdT, IndexT, hfk::kFlatUnrollHost>(a, grid, nt, s);
+    else launch_flat_gather_u<V, IdT, IndexT, hfk::kFlatUnrollDevice>(a, grid, nt, s);
 }
 
 template <typename IdT>
 int launch_flat_gather(uint64_t table, uint64_t dst, const IdT* ids, uint64_t n_ids, uint64_t row_bytes,
-                       uint64_t row_limit, uint32_t workgroups, hipStream_t s) {
+                       uint64_t row_limit, uint32_t workgroups, bool table_in_host, hipStream_t s) {
     FlatGatherArgs<IdT> a;
     hfk::FlatGatherPlan p;
-    int rc = hfk::plan_flat_gather<IdT>(a, p, table, dst, ids, n_ids, row_bytes, row_limit);
+    const int unroll = table_in_host ? hfk::kFlatUnrollHost : hfk::kFlatUnrollDevice;
+    int rc = hfk::plan_flat_gather<IdT>(a, p, table, dst, ids, n_ids, row_bytes, row_limit, unroll);
     if (rc != 0) return rc;
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
     if (p.unit == 16u) {
-        if (p.index32) launch_flat_gather_v<vec16, IdT, uint32_t>(a, grid, nt, s);
-        else launch_flat_gather_v<vec16, IdT, uint64_t>(a, grid, nt, s);
+        if (p.index32) launch_flat_gather_v<vec16, IdT, uint32_t>(a, grid, nt, unroll, s);
+        else launch_flat_gather_v<vec16, IdT, uint64_t>(a, grid, nt, unroll, s);
     } else if (p.unit == 4u) {
-        if (p.index32) launch_flat_gather_v<uint32_t, IdT, uint32_t>(a, grid, nt, s);
-        else launch_flat_gather_v<uint32_t, IdT, uint64_t>(a, grid, nt, s);
+        if (p.index32) launch_flat_gather_v<uint32_t, IdT, uint32_t>(a, grid, nt, unroll, s);
+        else launch_flat_gather_v<uint32_t, IdT, uint64_t>(a, grid, nt, unroll, s);
     } else {
-        if (p.index32) launch_flat_gather_v<uint8_t, IdT, uint32_t>(a, grid, nt, s);
-        else launch_flat_gather_v<uint8_t, IdT, uint64_t>(a, grid, nt, s);
+        if (p.index32) launch_flat_gather_v<uint8_t, IdT, uint32_t>(a, grid, nt, unroll, s);
+        else launch_flat_gather_v<uint8_t, IdT, uint64_t>(a, grid, nt, unroll, s);
     }
     return finish_launch();
 }
 
 template <typename IdT>
 int gather_rows_typed(const void* table, void* dst, const IdT* ids, uint64_t n_ids, uint64_t row_bytes,
-                      uint64_t table_rows, uint32_t workgroups, hipStream_t s) {
+                      uint64_t table_rows, uint32_t workgroups, bool table_in_host, hipStream_t s) {
     const uint64_t limit = table_rows ? table_rows : hfk::kUnchecked;
     if (row_bytes >= hfk::kWideRowBytes) {
         BlockCopyArgs<IdT> a;
@@ -389,7 +397,7 @@ int gather_rows_typed(const void* table, void* dst, const IdT* ids, uint64_t n_i
         return launch_block_copy<Role::kGatherRows, IdT>(a, workgroups, s);
     }
     return launch_flat_gather<IdT>((uint64_t)(uintptr_t)table, (uint64_t)(uintptr_t)dst, ids, n_ids, row_bytes,
-                                   limit, workgroups, s);
+                                   limit, workgroups, table_in_host, s);
 }
 
 // ---- transpose ------------------------------------------------------------
@@ -463,9 +471,10 @@ int launch_swap(const BlockCopyArgs<int64_t>& a, uint32_t flags, uint32_t workgr
         // Toward the host the link accepts the most when it is offered exactly what it can take
         // (offering 1.5-2x its rate lowers what it accepts to 47-49 GB/s). A swap that shares the GPU
         // offers 0.84 of the raw rate, one that owns it the payload-efficiency cap, 0.90; should the
-        // cap be lower than assumed the launch degrades to an unpaced one. A paced launch ends about
-        // 0.1 ms behind its schedule, which only a long one amortises (32 MiB: 49 GB/s paced, 54.6
-        // unpaced), so a short throughput-mode swap stays unpaced.
+        // cap be lower than assumed the launch degrades to an unpaced one. A paced launch starts its
+        // workgroups staggered over one interval and ends behind its schedule, which only a long one
+        // amortises (2 MiB: 71 us paced, 51 us unpaced; 32 MiB: 52.6 against 54.5 GB/s; 64 MiB: 55.1
+        // against 55.0; 128 MiB: 55.9 against 55.5), so a short throughput-mode swap stays unpaced.
         uint32_t pace_mbps = 0;
         if (beside) {
             pace_mbps = (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed);
@@ -685,7 +694,10 @@ int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i
     if (table == nullptr || dst == nullptr || ids == nullptr) return HFK_ERR_NULL_POINTER;
     if (row_bytes == 0) return HFK_ERR_BAD_SIZE;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (workgroups == 0 && n_ids * row_bytes > kLongHostGatherBytes && memory_side(table) == 1) {
+    // Where the table lives shapes the launch; the runtime is asked only when the answer can matter
+    // (a gather of less than 64 KiB is over before either shape could differ).
+    const bool table_in_host = n_ids * row_bytes >= kAskTableSideBytes && memory_side(table) == 1;
+    if (workgroups == 0 && table_in_host && n_ids * row_bytes > kLongHostGatherBytes) {
         // A table in host memory (the reference's embedding case) is read over the PCIe link: 64
         // workgroups already run it at the link's rate (55-57 GB/s for 1 KiB rows), and every further
         // one only slows kernels on other streams. Gathers of a few MiB keep one workgroup per chunk
@@ -694,10 +706,10 @@ int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i
     }
     if (ids_are_i64) {
         return gather_rows_typed<int64_t>(table, dst, static_cast<const int64_t*>(ids), n_ids, row_bytes,
-                                          table_rows, workgroups, s);
+                                          table_rows, workgroups, table_in_host, s);
     }
     return gather_rows_typed<int32_t>(table, dst, static_cast<const int32_t*>(ids), n_ids, row_bytes,
-                                      table_rows, workgroups, s);
+                                      table_rows, workgroups, table_in_host, s);
 }
 
 int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* src_block, uint32_t T,

@@ -183,7 +183,7 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *                   the copy beside it runs 6x slower, the GEMM 4.4x / 1.6x (out / in): what a swap
  *                   holds in flight beyond the link's bandwidth-delay product queues in front of
  *                   every other kernel's traffic.
- *                 - HFK_SWAP_DST_HOST (swap-out): 16 workgroups x 1 vector per lane; a swap of 256 MiB
+ *                 - HFK_SWAP_DST_HOST (swap-out): 16 workgroups x 1 vector per lane; a swap of 64 MiB
  *                   or more is paced at 0.90 of the link's raw rate (HFK_KNOB_LINK_MBPS), which the
  *                   link accepts better than an unbounded offer: 56.6 GB/s / 1.08x / 2.7x.
  *                 - HFK_SWAP_SRC_HOST (swap-in): 40 x 1, unpaced: 57.4 GB/s / 1.95x / 1.6x.
@@ -403,7 +403,7 @@ enum hfk_knob {
                                        the default                                                  */
     HFK_KNOB_DUPLEX_WORKGROUPS = 8, /* default grid bound of hfk_swap_blocks_duplex                       */
     HFK_KNOB_THROUGHPUT_PACE_PERMILLE = 9, /* share of HFK_KNOB_LINK_MBPS, in thousandths, that a swap-out or
-                                       duplex swap of 256 MiB or more offers toward the host when it is
+                                       duplex swap of 64 MiB or more offers toward the host when it is
                                        not marked HFK_SWAP_BESIDE_COMPUTE; 0 = unpaced; default 900      */
     HFK_KNOB_PACED_UNROLL = 11,     /* like HFK_KNOB_UNROLL, for the paced and the HFK_SWAP_BESIDE_COMPUTE launch
                                        shapes of hfk_swap_blocks                                          */

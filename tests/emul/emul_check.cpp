@@ -97,23 +97,31 @@ void run_block_copy(BlockCopyArgs<IdT> a, int preferred_unroll, uint32_t grid_ca
     }
 }
 
+template <typename V, typename IdT, typename IndexT, int NT>
+void walk_flat(const FlatGatherArgs<IdT>& a, uint32_t grid, int unroll) {
+    if (unroll == kFlatUnrollHost) walk(a, grid, flat_gather_body<V, IdT, IndexT, kFlatUnrollHost, NT>);
+    else walk(a, grid, flat_gather_body<V, IdT, IndexT, kFlatUnrollDevice, NT>);
+}
+
 template <typename IdT>
 void run_flat_gather(uint64_t table, uint64_t dst, const IdT* ids, uint64_t n_ids, uint64_t row_bytes,
                      uint64_t limit, uint32_t grid_cap, bool force64) {
-    FlatGatherArgs<IdT> a;
-    FlatGatherPlan p;
-    if (plan_flat_gather<IdT>(a, p, table, dst, ids, n_ids, row_bytes, limit) != HFK_OK) { ++g_failures; return; }
-    const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
-    const bool i32 = p.index32 && !force64;
-    if (p.unit == 16u) {
-        if (i32) walk(a, grid, flat_gather_body<vec16, IdT, uint32_t, kFlatUnroll, 3>);
-        else walk(a, grid, flat_gather_body<vec16, IdT, uint64_t, kFlatUnroll, 0>);
-    } else if (p.unit == 4u) {
-        if (i32) walk(a, grid, flat_gather_body<uint32_t, IdT, uint32_t, kFlatUnroll, 0>);
-        else walk(a, grid, flat_gather_body<uint32_t, IdT, uint64_t, kFlatUnroll, 3>);
-    } else {
-        if (i32) walk(a, grid, flat_gather_body<uint8_t, IdT, uint32_t, kFlatUnroll, 0>);
-        else walk(a, grid, flat_gather_body<uint8_t, IdT, uint64_t, kFlatUnroll, 0>);
+    for (int unroll : {kFlatUnrollDevice, kFlatUnrollHost}) {   // both launch shapes write the same bytes
+        FlatGatherArgs<IdT> a;
+        FlatGatherPlan p;
+        if (plan_flat_gather<IdT>(a, p, table, dst, ids, n_ids, row_bytes, limit, unroll) != HFK_OK) { ++g_failures; return; }
+        const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+        const bool i32 = p.index32 && !force64;
+        if (p.unit == 16u) {
+            if (i32) walk_flat<vec16, IdT, uint32_t, 3>(a, grid, unroll);
+            else walk_flat<vec16, IdT, uint64_t, 0>(a, grid, unroll);
+        } else if (p.unit == 4u) {
+            if (i32) walk_flat<uint32_t, IdT, uint32_t, 0>(a, grid, unroll);
+            else walk_flat<uint32_t, IdT, uint64_t, 3>(a, grid, unroll);
+        } else {
+            if (i32) walk_flat<uint8_t, IdT, uint32_t, 0>(a, grid, unroll);
+            else walk_flat<uint8_t, IdT, uint64_t, 0>(a, grid, unroll);
+        }
     }
 }
 

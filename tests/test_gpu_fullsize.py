@@ -1,5 +1,5 @@
 """The benchmark configurations at their full sizes, launched exactly as the benchmark
-launches them (the caller names the host side, so a swap-out of 256 MiB or more runs
+launches them (the caller names the host side, so a swap-out of 64 MiB or more runs
 paced and a swap-in keeps half as much in flight), and checked two ways:
 
 * four planes of every case against the C oracle, whole destination planes compared
@@ -249,7 +249,7 @@ def _verify_swap_out(c2, src_ids, dst_ids, what):
 @pytest.mark.parametrize("flags", [capi.SWAP_DST_HOST, 0, capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE],
                          ids=["dst_host_paced", "no_flags", "beside_compute"])
 def test_config2_llama8b_swap_out_full(c2, flags):
-    """flags = HFK_SWAP_DST_HOST is the launch the benchmark times: 512 MiB >= 256 MiB, so it is paced."""
+    """flags = HFK_SWAP_DST_HOST is the launch the benchmark times: 512 MiB >= 64 MiB, so it is paced."""
     cfg = c2["cfg"]
     announce("config 2 full, swap-out of 256 pairs x 64 planes in one launch, flags %d" % flags)
     _clear_host(c2["host"])
