@@ -234,13 +234,18 @@ class Workload:
         return wall, ms, spread
 
     def measure_gather(self, steps, warmup):
+        """The gather is over in 0.2-2 ms: it is timed over at least 50 ms of back-to-back launches, so that
+        the figure is that of a GPU at its steady clocks, like the 10-100 ms swap launches beside it."""
         torch, cfg = self.b.torch, self.cfg
         spread = self.b.launch_spread(self.gather, min(steps, 10))
-        _, ms = self.b.timed(self.gather, steps, warmup)
+        _, probe_ms = self.b.timed(self.gather, 5, warmup)
+        iters = max(steps, min(400, int(50.0 / max(probe_ms, 1e-3)) + 1))
+        _, ms = self.b.timed(self.gather, iters, 0)
+        self.gather_iters = iters
         for p in range(cfg.planes):
             assert torch.equal(self.prefill[p], self.dev_bytes[p].index_select(0, self.ids_dev)), "gather mismatch %d" % p
-        log("%s gather: %.1f GB/s of HBM traffic (%.1f payload GB/s, %.3f ms/launch), verified" %
-            (self.key, self.gather_alg_bytes / (ms * 1e6), self.payload / (ms * 1e6), ms))
+        log("%s gather: %.1f GB/s of HBM traffic (%.1f payload GB/s, %.4f ms/launch over %d launches), verified" %
+            (self.key, self.gather_alg_bytes / (ms * 1e6), self.payload / (ms * 1e6), ms, iters))
         return ms, spread
 
 
@@ -678,7 +683,7 @@ def measure_other_config(b, key, cfg, steps, warmup, d2h_peak, h2d_peak):
         steps = max(3, min(steps, int(2.0e9 * steps / max(w.payload, 1)) or 3))   # about as many bytes as the headline config moves
         _, ms_out, _ = w.measure_swap_out(steps, min(warmup, 2), capi.SWAP_DST_HOST)
         _, ms_in, _ = w.measure_swap_in(steps, min(warmup, 2), capi.SWAP_SRC_HOST)
-        ms_g, _ = w.measure_gather(max(steps, 10), min(warmup, 2))
+        ms_g, _ = w.measure_gather(steps, min(warmup, 2))
         out_gbps, in_gbps, g_gbps = rate(w.payload, ms_out), rate(w.payload, ms_in), rate(w.gather_alg_bytes, ms_g)
         return {
             "config": config_summary(w), "steps": steps,
@@ -687,7 +692,7 @@ def measure_other_config(b, key, cfg, steps, warmup, d2h_peak, h2d_peak):
             "swap_in": {"kernel_GBps": in_gbps, "avg_launch_ms": ms_in, "frac_of_pcie5_x16": frac(in_gbps, PCIE5_X16_GBPS),
                         "frac_of_measured_h2d": frac(in_gbps, h2d_peak)},
             "gather": {"traffic_GBps": g_gbps, "avg_launch_ms": ms_g, "frac_of_hbm_peak": frac(g_gbps, HBM_PEAK_GBPS),
-                       "algorithmic_bytes_per_launch": w.gather_alg_bytes},
+                       "algorithmic_bytes_per_launch": w.gather_alg_bytes, "launches_timed": w.gather_iters},
             "verified": "bit-exact on every plane: swap_out, swap_in, gather",
         }
     finally:
@@ -758,9 +763,10 @@ def main():
         wall_in, kernel_ms_in, spread_in = w.measure_swap_in(args.steps, args.warmup, capi.SWAP_SRC_HOST)
         swap_in_gbps = args.steps * w.payload / wall_in / 1e9
 
-    kernel_ms_g = spread_gather = gather_traffic_gbps = gather_payload_gbps = torch_gather_gbps = None
+    kernel_ms_g = spread_gather = gather_traffic_gbps = gather_payload_gbps = torch_gather_gbps = gather_iters = None
     if "gather" in sections:
         kernel_ms_g, spread_gather = w.measure_gather(args.steps, args.warmup)
+        gather_iters = w.gather_iters
         gather_traffic_gbps = w.gather_alg_bytes / (kernel_ms_g * 1e6)
         gather_payload_gbps = w.payload / (kernel_ms_g * 1e6)
         _, ms_t = b.timed(lambda: b.torch.index_select(w.dev_bytes[0], 0, w.ids_dev), args.steps, args.warmup)
@@ -793,6 +799,8 @@ def main():
     headline_config = config_summary(w, {"tuning_overrides": tuned})
     link_known = capi.get_tuning(capi.KNOB_LINK_MBPS) > 0
     gather_unroll = capi.get_tuning(capi.KNOB_UNROLL)
+    paced_unroll, paced_wgs = capi.get_tuning(capi.KNOB_PACED_UNROLL), capi.get_tuning(capi.KNOB_PACED_WORKGROUPS)
+    pace_permille = capi.get_tuning(capi.KNOB_THROUGHPUT_PACE_PERMILLE)
     w.release()
 
     # ---- the other configurations, one after the other --------------------------
@@ -812,8 +820,7 @@ def main():
     out_kernel_gbps = rate(w_payload, kernel_ms_out)
     in_kernel_gbps = rate(w_payload, kernel_ms_in)
     gather_alg_bytes = 2 * w_payload + 8 * headline_config["blocks_per_launch"]
-    paced = (args.out_flags & capi.SWAP_DST_HOST) and link_known and w_payload >= (64 << 20) and \
-        capi.get_tuning(capi.KNOB_THROUGHPUT_PACE_PERMILLE) > 0
+    paced = (args.out_flags & capi.SWAP_DST_HOST) and link_known and w_payload >= (64 << 20) and pace_permille > 0
     result = {
         "metric": "KV swap GB/s (% of PCIe5 x16 peak); block gather GB/s (% of HBM peak)",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -824,7 +831,8 @@ def main():
         # PCIe Gen5 x16 link, so that is the roofline it is priced against (theoretical link rate as
         # `peak`, the rate one large pinned hipMemcpyAsync reaches in this run as `peak_measured`).
         "roofline": {
-            "kernel": ("swap_blocks_kernel<4, 3>, paced" if paced else "swap_blocks_kernel<8, 3>") +
+            "kernel": ("swap_blocks_kernel<%d, 3>, %d workgroups, paced at 0.%d of the link" %
+                       (paced_unroll, paced_wgs, pace_permille // 10) if paced else "swap_blocks_kernel<8, 3>, 16 workgroups") +
                       " via hfk_swap_blocks (swap-out, HBM -> pinned host)", "bound": "pcie",
             "achieved": out_kernel_gbps, "peak": PCIE5_X16_GBPS, "unit": "GB/s",
             "frac": frac(out_kernel_gbps, PCIE5_X16_GBPS),
@@ -838,7 +846,7 @@ def main():
             "achieved": gather_traffic_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": frac(gather_traffic_gbps, HBM_PEAK_GBPS), "traffic": traffic.get("gather_hbm_bytes_per_launch"),
             "algorithmic_bytes_per_launch": gather_alg_bytes, "avg_launch_ms": kernel_ms_g,
-            "payload_GBps": gather_payload_gbps, "torch_index_select_GBps": torch_gather_gbps,
+            "launches_timed": gather_iters, "payload_GBps": gather_payload_gbps, "torch_index_select_GBps": torch_gather_gbps,
             "torch_device_copy_GBps": d2d_copy_gbps, "launch_spread": spread_gather,
         },
         "swap_out": {"GBps": value, "kernel_GBps": out_kernel_gbps, "launch_spread": spread_out,
