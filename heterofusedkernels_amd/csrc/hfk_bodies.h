@@ -525,6 +525,18 @@ struct TransposeArgs {
     uint32_t n_work;             // n_pairs * chunks_per_block
 };
 
+// Where the body finds layer l's address. The layer differs from lane to lane (a 128-byte row is 8
+// lanes wide), so this cannot be a scalar load, and as a vector load from the device array it would
+// make every work item wait for the stores of the one before it (vector loads and stores share one
+// counter) -- microseconds, when those stores go to host memory. The kernels therefore copy the
+// table into LDS once and hand the body an accessor over that copy, whose reads are counted with
+// the scalar loads; this accessor, over the array itself, serves tables too long for the LDS copy
+// and the CPU walk of the bodies.
+struct LayerTableInMemory {
+    const uint64_t* layer_ptrs;
+    HFK_HD uint64_t operator()(uint32_t l) const { return layer_ptrs[l]; }
+};
+
 HFK_HD void unit_from_bytes(const HFK_GLOBAL uint8_t* p, uint8_t& v) { v = p[0]; }
 HFK_HD void unit_from_bytes(const HFK_GLOBAL uint8_t* p, uint32_t& v) {
     v = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
@@ -538,8 +550,8 @@ HFK_HD void unit_from_bytes(const HFK_GLOBAL uint8_t* p, vec16& v) {
     v.w = w[3];
 }
 
-template <typename V, int UNROLL, int NT, bool TO_PACKED>
-HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+template <typename V, int UNROLL, int NT, bool TO_PACKED, typename LayerTable>
+HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid, const LayerTable& layer_address) {
     constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
     const uint32_t LH = a.L * a.H;
 
@@ -571,7 +583,7 @@ HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, ui
                 const uint32_t l = lh / a.H;
                 const uint32_t h = lh - l * a.H;
                 const uint64_t unit = ((uint64_t)h * a.T + t) * a.row_units + col;
-                layered_addr[u] = a.layer_ptrs[l] + layered_off + unit * sizeof(V);
+                layered_addr[u] = layer_address(l) + layered_off + unit * sizeof(V);
             }
         }
 #pragma unroll
@@ -606,6 +618,11 @@ HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, ui
             }
         }
     }
+}
+
+template <typename V, int UNROLL, int NT, bool TO_PACKED>
+HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+    transpose_body<V, UNROLL, NT, TO_PACKED>(a, bid, nb, tid, LayerTableInMemory{a.layer_ptrs});
 }
 
 }  // namespace hfk

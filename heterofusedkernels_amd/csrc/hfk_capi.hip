@@ -87,16 +87,36 @@ __global__ __launch_bounds__(256) void flat_gather_kernel(const FlatGatherArgs<I
     hfk::flat_gather_body<V, IdT, IndexT, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
+// The transfer kernels keep the layer-address table in LDS (see LayerTableInMemory): 512 layers, 4 KiB.
+constexpr uint32_t kLayerTableLdsEntries = 512;
+
+struct LayerTableInLds {
+    const uint64_t* table;   // points into LDS; after inlining the reads are ds_read_b64
+    __device__ uint64_t operator()(uint32_t l) const { return table[l]; }
+};
+
+template <typename V, int UNROLL, int NT, bool TO_PACKED>
+__device__ void transpose_with_layer_table(const TransposeArgs& a) {
+    __shared__ uint64_t layer_table[kLayerTableLdsEntries];
+    if (a.L <= kLayerTableLdsEntries) {   // uniform over the grid
+        for (uint32_t l = threadIdx.x; l < a.L; l += 256) layer_table[l] = hfk::table_entry(a.layer_ptrs, l);
+        __syncthreads();
+        hfk::transpose_body<V, UNROLL, NT, TO_PACKED>(a, blockIdx.x, gridDim.x, threadIdx.x, LayerTableInLds{layer_table});
+    } else {
+        hfk::transpose_body<V, UNROLL, NT, TO_PACKED>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    }
+}
+
 // Packed [T,L,H,D] blocks -> per-layer [H,T,D] caches (the reference's direction) ...
 template <typename V, int UNROLL, int NT>
 __global__ __launch_bounds__(256) void transpose_kernel(const TransposeArgs a) {
-    hfk::transpose_body<V, UNROLL, NT, false>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    transpose_with_layer_table<V, UNROLL, NT, false>(a);
 }
 
 // ... and back: per-layer caches -> packed blocks.
 template <typename V, int UNROLL, int NT>
 __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const TransposeArgs a) {
-    hfk::transpose_body<V, UNROLL, NT, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    transpose_with_layer_table<V, UNROLL, NT, true>(a);
 }
 
 // ---- tuning state ---------------------------------------------------------
@@ -114,8 +134,8 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
 //    what grows with the grid is the harm to kernels on other streams (a memory-bound
 //    neighbour runs 2.3-3x slower beside 16 workgroups, 4-5.7x beside 64), so a swap
 //    defaults to 16. For the same reason the duplex swap defaults to 32 workgroups (98.2 GB/s
-//    summed against 99.1 at 128, neighbours 1.1-1.6x slower instead of 2.8-2.9x) and the
-//    block-table transfers to 48 (-1 %, neighbours 1.8-2.5x instead of 4.9-5.3x).
+//    summed against 99.1 at 128, neighbours 1.1-1.6x slower instead of 2.8-2.9x), a block-table
+//    transfer out of host memory to 24 and one into host memory to 48 (see launch_transpose).
 std::atomic<int> g_unroll{1};
 std::atomic<int> g_nontemporal{3};
 std::atomic<int> g_wg_per_cu{65536};
@@ -124,8 +144,9 @@ constexpr uint32_t kDuplexWorkgroups = 32;
 constexpr uint32_t kBesideDuplexWorkgroups = 16;
 constexpr int kBesideDuplexUnroll = 2;
 constexpr uint32_t kBesideTransferWorkgroups = 16;
-constexpr uint32_t kTransferWorkgroups = 48;
-constexpr uint32_t kSingleBlockTransferWorkgroups = 128;
+constexpr uint32_t kTransferToHostWorkgroups = 48;
+constexpr uint32_t kTransferFromHostWorkgroups = 24;
+constexpr uint32_t kSingleBlockTransferWorkgroups = 32;
 constexpr uint32_t kHostGatherWorkgroups = 64;
 constexpr uint64_t kLongHostGatherBytes = 4ull << 20;
 constexpr uint64_t kAskTableSideBytes = 64ull << 10;
@@ -440,16 +461,20 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     if (rc != 0) return rc;
     if (a.n_work == 0) return HFK_OK;  // nothing to move
     // With the packed side in host memory the PCIe link is the bound and a small grid does; an
-    // unknown pointer gets the small grid too. (Pacing, which gains a swap-out 1-2 %, does not pay
-    // here: the per-item address arithmetic makes a workgroup's service time shape-dependent, and
-    // one-head 128-byte-row shapes fall behind any schedule that helps the others.)
+    // unknown pointer gets the small grid too. Measured on the reference's four shapes, 8 blocks per
+    // launch: host -> device 56.0-57.0 GB/s on 16 workgroups, 57.1-57.6 on 24-36, 54.1-54.6 on 48-56
+    // (a dip that repeats), 56.6-57.5 on 80-96; device -> host 48-52 on 16, 51-52 on 24, 52-54.7 from
+    // 32 on and flat. (Pacing, which gains a swap-out 1-2 %, does not pay toward the host here: it
+    // gains 0.8 GB/s on the eight-head shapes and loses up to 3.5 on the one-head shapes, whose
+    // 128-byte rows come from 64 different layer caches per chunk and fall behind any schedule.)
     const int side = packed_in_device ? 0 : memory_side(packed);
     if (workgroups == 0 && side != 0) {
         // One block (the reference's op: 4-64 MiB, over in 0.1-1.2 ms) is sized for speed alone; a
         // block table may run for many milliseconds beside other kernels and gets the smaller grid.
         workgroups = pairs == nullptr ? kSingleBlockTransferWorkgroups
                      : beside_compute ? kBesideTransferWorkgroups
-                                      : kTransferWorkgroups;
+                     : to_packed      ? kTransferToHostWorkgroups
+                                      : kTransferFromHostWorkgroups;
     }
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);

@@ -140,8 +140,8 @@ HFK_API int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_pt
  *   n_packed_blocks, n_dev_blocks  pool sizes; a pair outside them is skipped,
  *                    0 disables that side's check
  *   flags            0, or HFK_SWAP_BESIDE_COMPUTE: other kernels run meanwhile and matter. Only the
- *                    default grid changes (packed pool in host memory: 48 workgroups, 16 with the
- *                    flag), never the result.
+ *                    default grid changes (packed pool in host memory: 24 workgroups host -> device,
+ *                    48 device -> host, 16 with the flag), never the result.
  * Strides must be at least one block of their side. Destination blocks must be distinct.
  */
 HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t dev_block_stride,
