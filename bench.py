@@ -512,6 +512,12 @@ def section_staged(b, w, steps, warmup, out_flags):
             "auto_fragmented_beside_compute_in": lambda st: auto(False, beside, 0, st),
             "staged_fragmented_out": lambda st: staged(True, w.ids_dev, frag_host, st),
             "staged_fragmented_in": lambda st: staged(False, back_dev, frag_host, st)}
+    # The floor: kernels that touch no memory at all and only stay resident (one sleeping wavefront; 16 workgroups)
+    bench_lib = ctypes.CDLL(b.build.HFK_BENCH_SO)
+    bench_lib.hfkb_idle_resident.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p]
+    idle_ticks = int(payload / 55e9 * 1e8)                                  # as long as one swap
+    ways["one_idle_wavefront"] = lambda st: bench_lib.hfkb_idle_resident(1, 64, idle_ticks, st)
+    ways["sixteen_idle_workgroups"] = lambda st: bench_lib.hfkb_idle_resident(16, 256, idle_ticks, st)
     # own rate of the beside-compute launch shape, GPU otherwise idle; result checked like the plain swap-out's
     for p_ in range(planes):
         w.host_planes[p_][w.dst_ids] = 0
@@ -541,7 +547,8 @@ def section_staged(b, w, steps, warmup, out_flags):
                    "neighbour_ms_alone": alone,
                    "neighbour_slowdown": slowdown,
                    "how": "each neighbour runs %s times on one stream while %d swaps of %d MiB are queued on another; "
-                          "x = its time per call / its time alone; null = the swaps ended first" %
+                          "x = its time per call / its time alone; null = the swaps ended first. one_idle_wavefront / "
+                          "sixteen_idle_workgroups: kernels that only sleep, the price of sharing the GPU at all" %
                           ("/".join(str(r) for _, r in neighbours.values()), side_reps, payload >> 20)}
     log("staged swap, verified: out %.2f GB/s, in %.2f GB/s, both on two streams %.2f GB/s summed" %
         (staged_out_json["swap_out_GBps"], staged_out_json["swap_in_GBps"], staged_duplex_gbps))

@@ -8,6 +8,9 @@
 //    one workgroup per chunk of 256 * UNROLL 16-byte vectors, UNROLL loads before the first store)
 //    when it only reads, only writes, or copies a contiguous buffer. The read-only and write-only
 //    rates bound any copy: moving N bytes takes at least N / read_rate + N / write_rate.
+//  * hfkb_idle_resident: workgroups that touch no memory and only sleep for a bounded time. What a
+//    kernel on another stream loses beside them is the price of sharing the GPU at all, the floor
+//    under every figure measured beside a swap.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -20,6 +23,13 @@ using hfk::kWorkgroupLanes;
 using hfk::vec16;
 
 enum Mode { kRead = 0, kWrite = 1, kCopy = 2 };
+
+__global__ void idle_resident_kernel(uint64_t ticks) {
+    const uint64_t t0 = wall_clock64();
+    for (uint32_t spin = 0; spin < (1u << 24) && wall_clock64() - t0 < ticks; ++spin) {
+        __builtin_amdgcn_s_sleep(20);
+    }
+}
 
 template <int MODE, int UNROLL, int NT>
 __global__ __launch_bounds__(256) void hbm_stream_kernel(uint64_t dst, uint64_t src, uint64_t n_chunks, uint32_t never) {
@@ -93,6 +103,15 @@ __attribute__((visibility("default"))) int hfkb_memcpy_block_loop(
         }
     }
     return 0;
+}
+
+// `workgroups` x `lanes` that sleep until `ticks` of the 100 MHz counter have passed (at most a few
+// seconds: the loop is bounded as well), then exit.
+__attribute__((visibility("default"))) int hfkb_idle_resident(uint32_t workgroups, uint32_t lanes, uint64_t ticks,
+                                                              void* stream) {
+    if (workgroups == 0 || lanes == 0 || lanes > 1024 || ticks > 300000000ull) return -1;
+    hipLaunchKernelGGL(idle_resident_kernel, dim3(workgroups), dim3(lanes), 0, static_cast<hipStream_t>(stream), ticks);
+    return (int)hipGetLastError();
 }
 
 // mode 0: read `bytes` from src; 1: write `bytes` to dst; 2: copy src -> dst. Buffers are device

@@ -138,3 +138,49 @@ def test_block_table_transfer_staged_through_a_device_pool():
     assert torch.equal(staged.view(torch.uint8), direct.view(torch.uint8))
     want = torch.stack(O.torch_multi_layer_block_transfer(host_pool[host_ids[0]]))     # [L, H, T, D] of the first moved block
     assert torch.equal(staged[:, dev_ids[0]].cpu().contiguous().view(torch.uint8), want.view(torch.uint8))
+
+
+@pytest.mark.parametrize("T,L,H,D,dtype", [(16, 32, 8, 128, torch.bfloat16), (64, 5, 2, 80, torch.float16)])
+def test_block_table_transfer_with_token_major_layer_caches(T, L, H, D, dtype):
+    """Layer caches laid out [blocks, T, H, D] (tokens first, the common paged-attention layout) instead of
+    the reference's [H, T, D] per block (multi_layer_block_transfer_kernel.h:60-67): a token's H x D values are
+    then contiguous on both sides, which is the same transfer with one head of H * D values. Both directions,
+    against torch indexing and the C oracle."""
+    e = torch.empty((), dtype=dtype).element_size()
+    host_blocks, dev_blocks, n = 10, 13, 6
+    announce("block-table transfer, token-major layer caches, T=%d L=%d H=%d D=%d %s" % (T, L, H, D, dtype))
+    block_bytes = T * L * H * D * e
+    gen = torch.Generator().manual_seed(L * 100 + H)
+    pool = memory.alloc_numa_pinned_tensor(host_blocks * block_bytes)
+    pool.copy_(torch.randint(-128, 128, (pool.numel(),), dtype=torch.int8, generator=gen))
+    host_pool = pool.view(dtype).view(host_blocks, T, L, H, D)
+    caches = torch.zeros(L, dev_blocks, T, H, D, dtype=dtype, device=DEV)
+    ptrs = torch.tensor([caches[l].data_ptr() for l in range(L)], dtype=torch.int64).to(DEV)
+    hb = torch.randperm(host_blocks, generator=gen)[:n]
+    db = torch.randperm(dev_blocks, generator=gen)[:n]
+    pairs = torch.stack([hb, db], 1).contiguous()
+    stride = T * H * D * e
+    torch.ops.pcie_through.multi_layer_block_table_transfer(ptrs, host_pool.view(host_blocks, T, L, 1, H * D),
+                                                            pairs.to(DEV), stride, dev_blocks)
+    torch.cuda.synchronize()
+    got = caches.cpu()
+    want = torch.zeros_like(got)
+    want[:, db] = host_pool[hb].permute(2, 0, 1, 3, 4)                    # [n, T, L, H, D] -> [L, n, T, H, D]
+    assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+    oracle_want = np.zeros((L, dev_blocks, stride), dtype=np.uint8)
+    O.c_multi_layer_block_table_transfer(oracle_want, pool.view(torch.uint8).numpy().reshape(host_blocks, block_bytes),
+                                         pairs.numpy(), T, L, 1, H * D, e, False)
+    assert np.array_equal(got.view(torch.uint8).numpy().reshape(L, dev_blocks, stride), oracle_want)
+    # and back into other host slots
+    pool2 = memory.alloc_numa_pinned_tensor(host_blocks * block_bytes)
+    host_pool2 = pool2.view(dtype).view(host_blocks, T, L, H, D)
+    hb2 = torch.randperm(host_blocks, generator=gen)[:n]
+    torch.ops.pcie_through.multi_layer_block_table_transfer(ptrs, host_pool2.view(host_blocks, T, L, 1, H * D),
+                                                            torch.stack([hb2, db], 1).contiguous().to(DEV), stride,
+                                                            dev_blocks, True)
+    torch.cuda.synchronize()
+    for j in range(n):
+        assert torch.equal(host_pool2[hb2[j]].view(torch.uint8), host_pool[hb[j]].view(torch.uint8))
+    untouched = torch.ones(host_blocks, dtype=torch.bool)
+    untouched[hb2] = False
+    assert int(pool2.view(host_blocks, block_bytes)[untouched].abs().max()) == 0
