@@ -158,7 +158,7 @@ std::atomic<int> g_duplex_workgroups{(int)kDuplexWorkgroups};
 std::atomic<int> g_hbm_lds_bytes{0};
 // Share of the link's raw rate, in thousandths, that a long throughput-mode launch offers toward the
 // host (0 = unpaced).
-std::atomic<int> g_throughput_pace_permille{900};
+std::atomic<int> g_throughput_pace_permille{890};
 std::atomic<int> g_swap_unroll{8};
 // Explicit offered rate of a swap that runs beside compute, MB/s; 0 = derive it from the link.
 std::atomic<int> g_swap_pace_mbps{0};
@@ -172,23 +172,39 @@ std::atomic<int> g_link_mbps_override{-1};
 // per workgroup iteration) and just enough workgroups. Measured on MI355X with 32 KiB blocks, as
 // own rate / slowdown of a 1 GiB device copy / of a bf16 8192^3 GEMM on another stream:
 //  * toward the host, paced (workgroups x vectors per lane):
-//      12 x 1 at 0.90 of the link: 56.4 GB/s / 1.05x / 2.2x      16 x 4 at 0.90: 56.5 / 2.7x / 4.1x
+//      12 x 1 at 0.90 of the link: 56.4 GB/s / 1.05x / 2.2x      16 x 4 at 0.90: 55.9 / 2.9x / 4.3x
 //      16 x 1 at 0.90:             56.6 GB/s / 1.08x / 2.7x
 //      12 x 1 at 0.84:             52.8 GB/s / 1.05x / 1.64x     8 x 4 at 0.84: 52.2 / 1.64x / 1.75x
 //    (8 x 1 cannot hold the pace: 42.9 GB/s; unpaced, small grids are erratic: 38-48 GB/s);
 //  * from the host, unpaced (pacing changes nothing there):
 //      24 x 1: 55.9 GB/s / 1.30x / 1.58x     40 x 1: 57.4 / 1.95x / 1.59x     16 x 4: 57.4 / 3.4x / 1.58x
-//    the copy's slowdown follows what is in flight, the GEMM's (1.55-1.6x) is what any resident kernel
-//    costs it.
-std::atomic<int> g_paced_workgroups{16};         // toward the host, throughput mode (HFK_KNOB_PACED_WORKGROUPS): 12 hold
-                                                 // the pace on an idle GPU, 16 also after a long run of other work
+//    the copy's slowdown follows what is in flight, the GEMM's (1.5-1.6x) is what any resident kernel
+//    costs it (one wavefront that only sleeps: 1.50x).
+// Toward the host, throughput mode (HFK_KNOB_PACED_WORKGROUPS x HFK_KNOB_PACED_UNROLL, at
+// HFK_KNOB_THROUGHPUT_PACE_PERMILLE of the link). A paced launch has to hold its pace whatever the
+// block table looks like and whatever ran before it. A workgroup that is late starts its next item
+// at once, so a launch that has fallen behind offers more than its pace until it has caught up; at
+// 0.90 of the link, the most it accepts, it never does, and a link that is offered more than it
+// takes accepts less. Measured over eight address patterns (consecutive, strided, descending, runs
+// of 8, random; 12 launches each) and, in a process of their own, the four benchmark configurations:
+//   0.90: 16 x 1 53.2-56.5 GB/s by pattern, single launches down to 52.6; 6 x 4 56.4-56.6, single
+//         launches down to 50.7 and one benchmark run at 49.8; 32 x 1 55.6-56.6;
+//   0.89: every shape within 55.5-56.0 on every pattern; 6 x 4 56.0 on all eight (slowest launch
+//         55.95) and 55.5 / 56.0 / 55.5 / 56.0 on the configurations in every run; 16 x 1 55.5-56.0
+//         but 53.4 in one of three runs of configuration 2.
+// One percent of headroom is what makes the pace holdable, and 96 KiB in flight hold it where 64 KiB
+// do not always. What the steadier shape costs the kernels beside it (device copy / SDPA / GEMM):
+// 1.35x / 1.32x / 2.5x against 1.07x / 1.21x / 2.3x for 16 x 1; a swap that should be gentle says so
+// (HFK_SWAP_BESIDE_COMPUTE) and gets the fine shape at 0.84, which it holds on every pattern
+// (52.7-52.8 GB/s).
+std::atomic<int> g_paced_workgroups{6};
+std::atomic<int> g_paced_unroll{4};
 constexpr uint32_t kBesidePacedWorkgroups = 12;  // toward the host, beside compute (the lower pace leaves the margin)
 constexpr uint32_t kFromHostWorkgroups = 40;     // from the host, throughput mode
 constexpr uint32_t kBesideFromHostWorkgroups = 24;
 constexpr uint32_t kBesideWorkgroups = 8;        // HFK_SWAP_BESIDE_COMPUTE with no host side named: 8 x 4, unpaced
 constexpr int kBesideUnnamedUnroll = 4;
-std::atomic<int> g_paced_unroll{1};              // vectors per lane of the named-side shapes (HFK_KNOB_PACED_UNROLL)
-int named_side_unroll() { return g_paced_unroll.load(std::memory_order_relaxed); }
+constexpr int kFineUnroll = 1;                   // one vector per lane: swaps from the host, and toward it beside compute
 // Share of the link's raw rate offered to host writes when pacing. 256-byte transaction payloads
 // cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured, reached only by a paced grid); from 0.92
 // on throughput collapses to 0.84 and the neighbours' slowdown doubles. The closer to the cap, the
@@ -511,12 +527,13 @@ int launch_swap(const BlockCopyArgs<int64_t>& a, uint32_t flags, uint32_t workgr
             if (workgroups == 0) {
                 workgroups = beside ? kBesidePacedWorkgroups : (uint32_t)g_paced_workgroups.load(std::memory_order_relaxed);
             }
-            return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, named_side_unroll(), pace_mbps);
+            const int unroll = beside ? kFineUnroll : g_paced_unroll.load(std::memory_order_relaxed);
+            return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, unroll, pace_mbps);
         }
     }
     if ((flags & HFK_SWAP_SRC_HOST) != 0) {
         const uint32_t grid = beside ? kBesideFromHostWorkgroups : kFromHostWorkgroups;
-        return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups ? workgroups : grid, s, named_side_unroll());
+        return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups ? workgroups : grid, s, kFineUnroll);
     }
     if (beside) {
         // No usable pace (no host side named, or the link's rate is unknown): the small unpaced grid
@@ -821,7 +838,7 @@ int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move*
             const double item_bytes = (double)block_bytes / a.first.chunks_per_block;
             const double q8 = item_bytes * grid / ((double)pace_mbps * 1e6) * 1e8 * 256.0 + 0.5;
             a.pace_q8 = q8 < 4294967295.0 ? (uint32_t)q8 : 0xffffffffu;
-        }
+            }
     }
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
     hipStream_t s = static_cast<hipStream_t>(stream);

@@ -183,9 +183,11 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *                   the copy beside it runs 6x slower, the GEMM 4.4x / 1.6x (out / in): what a swap
  *                   holds in flight beyond the link's bandwidth-delay product queues in front of
  *                   every other kernel's traffic.
- *                 - HFK_SWAP_DST_HOST (swap-out): 16 workgroups x 1 vector per lane; a swap of 64 MiB
- *                   or more is paced at 0.90 of the link's raw rate (HFK_KNOB_LINK_MBPS), which the
- *                   link accepts better than an unbounded offer: 56.6 GB/s / 1.08x / 2.7x.
+ *                 - HFK_SWAP_DST_HOST (swap-out): a swap of 64 MiB or more runs on 6 workgroups x 4
+ *                   vectors per lane, paced at 0.89 of the link's raw rate (HFK_KNOB_LINK_MBPS): one
+ *                   percent under the most the link accepts, which is what lets the launch hold its
+ *                   pace on every block table (55.5-56.0 GB/s; at 0.90 consecutive or strided tables
+ *                   lose up to 5 %) / 1.35x / 2.5x. A shorter one runs unpaced.
  *                 - HFK_SWAP_SRC_HOST (swap-in): 40 x 1, unpaced: 57.4 GB/s / 1.95x / 1.6x.
  *                 - with HFK_SWAP_BESIDE_COMPUTE as well: out on 12 x 1 paced at 0.84: 52.8 GB/s / 1.05x /
  *                   1.64x; in on 24 x 1: 55.9 GB/s / 1.30x / 1.58x (1.55-1.6x is what any resident
@@ -404,11 +406,11 @@ enum hfk_knob {
     HFK_KNOB_DUPLEX_WORKGROUPS = 8, /* default grid bound of hfk_swap_blocks_duplex                       */
     HFK_KNOB_THROUGHPUT_PACE_PERMILLE = 9, /* share of HFK_KNOB_LINK_MBPS, in thousandths, that a swap-out or
                                        duplex swap of 64 MiB or more offers toward the host when it is
-                                       not marked HFK_SWAP_BESIDE_COMPUTE; 0 = unpaced; default 900      */
-    HFK_KNOB_PACED_UNROLL = 11,     /* like HFK_KNOB_UNROLL, for the paced and the HFK_SWAP_BESIDE_COMPUTE launch
-                                       shapes of hfk_swap_blocks                                          */
-    HFK_KNOB_PACED_WORKGROUPS = 12, /* default grid of a paced swap toward the host (hfk_swap_blocks with
-                                       HFK_SWAP_DST_HOST)                                                  */
+                                       not marked HFK_SWAP_BESIDE_COMPUTE; 0 = unpaced; default 890      */
+    HFK_KNOB_PACED_UNROLL = 11,     /* like HFK_KNOB_UNROLL, for the paced throughput-mode swap toward the host
+                                       (default 4)                                                        */
+    HFK_KNOB_PACED_WORKGROUPS = 12, /* default grid of that swap (hfk_swap_blocks with HFK_SWAP_DST_HOST alone;
+                                       default 6)                                                          */
     HFK_KNOB_HBM_LDS_BYTES = 10     /* dynamic LDS, 0..65536 bytes, that the HBM-bound launches (gathers, the
                                        staged swap's kernel) request without using it: with 160 KiB of LDS
                                        per compute unit it bounds the workgroups a unit holds at a time   */
