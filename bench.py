@@ -31,7 +31,7 @@ if ROOT not in sys.path:
 
 PCIE5_X16_GBPS = 32.0 * 16 * (128.0 / 130.0) / 8.0   # 63.0 GB/s per direction, before packet overheads
 HBM_PEAK_GBPS = 8000.0                               # MI355X HBM3E
-ALL_SECTIONS = ("swap_out", "swap_in", "gather", "duplex", "staged", "hbm_ceiling")
+ALL_SECTIONS = ("swap_out", "swap_in", "gather", "duplex", "staged", "hbm_ceiling", "tables")
 
 
 def log(msg):
@@ -560,6 +560,54 @@ def section_staged(b, w, steps, warmup, out_flags):
     return staged_out_json, beside_json, frag
 
 
+def section_tables(b, w, steps):
+    """The swap-out over different kinds of block table (same size as the workload's own): a paced launch must hold
+    its rate whatever the table looks like. Destroys the host cache's content, so it runs after everything else;
+    every launch shape is verified on every table (two planes, moved blocks byte for byte)."""
+    torch, capi, W, cfg = b.torch, b.capi, b.W, w.cfg
+    planes, bb, n = cfg.planes, cfg.block_bytes, cfg.n_blocks
+    gen = torch.Generator().manual_seed(cfg.base_seed + 99)
+    ar = torch.arange(n)
+    assert 2 * n + 8 <= min(cfg.dev_blocks, cfg.host_blocks), "pools too small for the strided tables"
+
+    def runs_of(k, blocks):
+        starts = torch.randperm(blocks // k, generator=gen)[:n // k]
+        return (starts[:, None] * k + torch.arange(k)).flatten()[:n]
+
+    tables = {
+        "consecutive_both": (ar + 7, ar + 5),
+        "device_descending": ((n - 1 - ar) + 7, ar + 5),
+        "device_every_2nd": (2 * ar, ar + 5),
+        "host_every_2nd": (ar + 7, 2 * ar),
+        "both_every_2nd": (2 * ar, 2 * ar + 1),
+        "runs_of_8_shuffled": (runs_of(8, cfg.dev_blocks), runs_of(8, cfg.host_blocks)),
+        "random": (torch.randperm(cfg.dev_blocks, generator=gen)[:n], torch.randperm(cfg.host_blocks, generator=gen)[:n]),
+        "the_workloads_own": (w.src_ids, w.dst_ids),
+    }
+    shapes = {"host_side_named": capi.SWAP_DST_HOST, "beside_compute": capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE,
+              "no_flags": 0}
+    payload = planes * n * bb
+    out = {k: {} for k in shapes}
+    for name, (src, dst) in tables.items():
+        pairs = W.pairs_tensor(src, dst).to(b.dev)
+        src_dev = src.to(b.dev)
+        for shape, flags in shapes.items():
+            for p in (0, planes - 1):
+                w.host_planes[p][dst] = 0
+            _, ms = b.timed(lambda: capi.check(capi.swap_blocks(
+                w.host_tab.data_ptr(), w.dev_tab.data_ptr(), pairs.data_ptr(), planes, n, bb, bb, bb, cfg.dev_blocks,
+                cfg.host_blocks, 0, b.stream, flags), "hfk_swap_blocks"), max(4, steps // 2), 1)
+            for p in (0, planes - 1):
+                assert torch.equal(w.host_planes[p].index_select(0, dst), w.dev_bytes[p].index_select(0, src_dev).cpu()), \
+                    "swap-out mismatch on table %s, shape %s, plane %d" % (name, shape, p)
+            out[shape][name] = round(payload / (ms * 1e6), 2)
+    for shape, rates in out.items():
+        log("swap-out by block table, %-16s min %.2f max %.2f GB/s | %s" %
+            (shape + ":", min(rates.values()), max(rates.values()), ", ".join("%s %.1f" % kv for kv in rates.items())))
+    return {"GBps": out, "blocks": n, "how": "%d launches per table and shape, one HIP event pair around them; "
+            "two planes verified per table and shape" % max(4, steps // 2)}
+
+
 def section_hbm_ceiling(b, steps, warmup):
     """What HBM gives a kernel of the gather's shape (256-lane workgroups, one workgroup per chunk, 16-byte
     non-temporal accesses) that only reads, only writes, or copies 512 MiB of contiguous device memory.
@@ -803,6 +851,7 @@ def main():
     hbm_ceiling = section_hbm_ceiling(b, args.steps, args.warmup) if "hbm_ceiling" in sections else None
     memcpy_loop = None if args.skip_memcpy_loop else section_memcpy_loop(b, w)
     cpu_baseline = None if args.skip_cpu_baseline else section_cpu_baseline(b, w)
+    tables = section_tables(b, w, args.steps) if "tables" in sections else None
     headline_config = config_summary(w, {"tuning_overrides": tuned})
     link_known = capi.get_tuning(capi.KNOB_LINK_MBPS) > 0
     gather_unroll = capi.get_tuning(capi.KNOB_UNROLL)
@@ -869,10 +918,11 @@ def main():
         "duplex": duplex,
         "staged": staged,
         "fragmented_host_slots": fragmented,
+        "swap_out_by_block_table": tables,
         "beside_compute": beside,
         "memcpy_block_loop": memcpy_loop,
         "cpu_baseline": cpu_baseline,
-        "verified": "bit-exact on every plane: " + ", ".join(sorted(sections - {"hbm_ceiling"})),
+        "verified": "bit-exact on every plane: " + ", ".join(sorted(sections - {"hbm_ceiling", "tables"})),
     }
     print(json.dumps(result), flush=True)
 
