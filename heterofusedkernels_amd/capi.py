@@ -27,6 +27,8 @@ KNOB_PACED_WORKGROUPS = 12
 SWAP_DST_HOST = 1
 SWAP_SRC_HOST = 2
 SWAP_BESIDE_COMPUTE = 4
+SWAP_SRC_DEVICE = 8
+SWAP_DST_DEVICE = 16
 STATIC_STAGING_BYTES = 64 << 20
 ERR_STAGING_TOO_SMALL = -7
 
@@ -89,9 +91,9 @@ def load():
     L.hfk_version.restype = ci
     L.hfk_status_string.argtypes = [ci]
     L.hfk_status_string.restype = ctypes.c_char_p
-    L.hfk_gather_rows.argtypes = [vp, vp, vp, ci, u64, u64, u64, u32, vp]
+    L.hfk_gather_rows.argtypes = [vp, vp, vp, ci, u64, u64, u64, u32, u32, vp]
     L.hfk_gather_rows.restype = ci
-    L.hfk_multi_layer_block_transfer.argtypes = [vp, vp, u32, u32, u32, u32, u32, u32, vp]
+    L.hfk_multi_layer_block_transfer.argtypes = [vp, vp, u32, u32, u32, u32, u32, u32, u32, vp]
     L.hfk_multi_layer_block_transfer.restype = ci
     L.hfk_fused_memcpy_multi_layer_block_transfer.argtypes = [vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
     L.hfk_fused_memcpy_multi_layer_block_transfer.restype = ci
@@ -127,13 +129,13 @@ def check(rc, what="hfk call"):
         raise RuntimeError("%s failed: %s (%d)" % (what, status_string(rc), rc))
 
 
-def gather_rows(table, dst, ids, ids_are_i64, n_ids, row_bytes, table_rows=0, workgroups=0, stream=0):
-    return load().hfk_gather_rows(table, dst, ids, int(ids_are_i64), n_ids, row_bytes, table_rows, workgroups,
+def gather_rows(table, dst, ids, ids_are_i64, n_ids, row_bytes, table_rows=0, workgroups=0, stream=0, flags=0):
+    return load().hfk_gather_rows(table, dst, ids, int(ids_are_i64), n_ids, row_bytes, table_rows, flags, workgroups,
                                   stream)
 
 
-def multi_layer_block_transfer(layer_ptrs, src, T, L, H, D, elem_bytes, workgroups=0, stream=0):
-    return load().hfk_multi_layer_block_transfer(layer_ptrs, src, T, L, H, D, elem_bytes, workgroups, stream)
+def multi_layer_block_transfer(layer_ptrs, src, T, L, H, D, elem_bytes, workgroups=0, stream=0, flags=0):
+    return load().hfk_multi_layer_block_transfer(layer_ptrs, src, T, L, H, D, elem_bytes, flags, workgroups, stream)
 
 
 def fused_memcpy_multi_layer_block_transfer(layer_ptrs, host_block, staging, T, L, H, D, elem_bytes,

@@ -198,14 +198,14 @@ int main(int argc, char** argv) {
     for (i = 0; i < n; ++i) pairs_h[i] = perm_b[n - 1 - i];
     CHECK_HIP(hipMemcpy(ids_d, pairs_h, n * sizeof(int64_t), hipMemcpyHostToDevice));
     printf("step gather\n"); fflush(stdout);
-    CHECK_HFK(hfk_gather_rows((const void*)(uintptr_t)host_tab_h[0], rows_d, ids_d, 1, n, bb, blocks, 0, stream));
+    CHECK_HFK(hfk_gather_rows((const void*)(uintptr_t)host_tab_h[0], rows_d, ids_d, 1, n, bb, blocks, HFK_SWAP_SRC_HOST, 0, stream));
     CHECK_HIP(hipStreamSynchronize(stream));
     CHECK_HIP(hipMemcpy(scratch, rows_d, n * bb, hipMemcpyDeviceToHost));
     for (i = 0; i < n; ++i)
         if (expect_block(scratch + i * bb, 0, (uint64_t)perm_a[n - 1 - i], bb, "gather", i)) return 7;
 
     /* an argument error is a status, not a crash */
-    if (hfk_gather_rows(NULL, rows_d, ids_d, 1, n, bb, blocks, 0, stream) != HFK_ERR_NULL_POINTER) {
+    if (hfk_gather_rows(NULL, rows_d, ids_d, 1, n, bb, blocks, 0, 0, stream) != HFK_ERR_NULL_POINTER) {
         fprintf(stderr, "NULL table was not rejected\n");
         return 8;
     }

@@ -474,18 +474,26 @@ HFK_HD void flat_gather_body(const FlatGatherArgs<IdT>& a, uint32_t bid, uint32_
         const IndexT g0 = (IndexT)w * kChunkUnits + tid;
         V v[UNROLL];
         bool ok[UNROLL];
+        uint64_t id[UNROLL];
+        IndexT col[UNROLL];
+        // All row ids first, then all rows: the id loads do not wait for one another (one memory
+        // round trip per work item, not one per unit).
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const IndexT g = g0 + (IndexT)u * kWorkgroupLanes;
-            ok[u] = false;
+            id[u] = ~0ull;   // never below row_limit
+            col[u] = 0;
             if (g < total) {
                 const IndexT row = g / row_units;
-                const IndexT col = g - row * row_units;
-                const uint64_t id = (uint64_t)(int64_t)a.ids[row];
-                if (id < a.row_limit) {
-                    ok[u] = true;
-                    v[u] = load_unit<NT>(table + id * a.row_units + col);
-                }
+                col[u] = g - row * row_units;
+                id[u] = (uint64_t)(int64_t)a.ids[row];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            ok[u] = id[u] < a.row_limit;
+            if (ok[u]) {
+                v[u] = load_unit<NT>(table + id[u] * a.row_units + col[u]);
             }
         }
 #pragma unroll

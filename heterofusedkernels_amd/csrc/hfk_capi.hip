@@ -463,12 +463,13 @@ int memory_side(const void* p) {
     return -1;
 }
 
-// `packed_in_device` is what the caller knows for certain (the staged variant); otherwise the
-// runtime is asked where the packed pool lives.
+// `packed_side` is what the caller knows about the packed pool (1 host memory, 0 device memory);
+// kAskRuntime: the runtime is asked where it lives.
+constexpr int kAskRuntime = -2;
 int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64_t* pairs, uint64_t n_pairs,
                      uint64_t packed_stride, uint64_t layered_stride, uint64_t packed_blocks,
                      uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
-                     bool to_packed, bool packed_in_device, uint32_t workgroups, hipStream_t s,
+                     bool to_packed, int packed_side, uint32_t workgroups, hipStream_t s,
                      bool beside_compute = false) {
     TransposeArgs a;
     uint32_t unit = 16;
@@ -483,7 +484,7 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     // 32 on and flat. (Pacing, which gains a swap-out 1-2 %, does not pay toward the host here: it
     // gains 0.8 GB/s on the eight-head shapes and loses up to 3.5 on the one-head shapes, whose
     // 128-byte rows come from 64 different layer caches per chunk and fall behind any schedule.)
-    const int side = packed_in_device ? 0 : memory_side(packed);
+    const int side = packed_side == kAskRuntime ? memory_side(packed) : packed_side;
     if (workgroups == 0 && side != 0) {
         // One block (the reference's op: 4-64 MiB, over in 0.1-1.2 ms) is sized for speed alone; a
         // block table may run for many milliseconds beside other kernels and gets the smaller grid.
@@ -731,14 +732,18 @@ const char* hfk_status_string(int status) {
 }
 
 int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i64, uint64_t n_ids,
-                    uint64_t row_bytes, uint64_t table_rows, uint32_t workgroups, hfk_stream_t stream) {
+                    uint64_t row_bytes, uint64_t table_rows, uint32_t flags, uint32_t workgroups,
+                    hfk_stream_t stream) {
+    if (flags != 0 && flags != HFK_SWAP_SRC_HOST && flags != HFK_SWAP_SRC_DEVICE) return HFK_ERR_BAD_FLAGS;
     if (n_ids == 0) return HFK_OK;
     if (table == nullptr || dst == nullptr || ids == nullptr) return HFK_ERR_NULL_POINTER;
     if (row_bytes == 0) return HFK_ERR_BAD_SIZE;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // Where the table lives shapes the launch; the runtime is asked only when the answer can matter
+    // Where the table lives shapes the launch. A caller that does not say is answered by the runtime,
+    // which takes about 5 us of the calling thread, so it is asked only when the answer can matter
     // (a gather of less than 64 KiB is over before either shape could differ).
-    const bool table_in_host = n_ids * row_bytes >= kAskTableSideBytes && memory_side(table) == 1;
+    const bool table_in_host = flags == HFK_SWAP_SRC_HOST ||
+                               (flags == 0 && n_ids * row_bytes >= kAskTableSideBytes && memory_side(table) == 1);
     if (workgroups == 0 && table_in_host && n_ids * row_bytes > kLongHostGatherBytes) {
         // A table in host memory (the reference's embedding case) is read over the PCIe link: 64
         // workgroups already run it at the link's rate (55-57 GB/s for 1 KiB rows), and every further
@@ -755,9 +760,11 @@ int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i
 }
 
 int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* src_block, uint32_t T,
-                                   uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
+                                   uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes, uint32_t flags,
                                    uint32_t workgroups, hfk_stream_t stream) {
-    return launch_transpose(dev_layer_ptrs, src_block, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, false,
+    if (flags != 0 && flags != HFK_SWAP_SRC_HOST && flags != HFK_SWAP_SRC_DEVICE) return HFK_ERR_BAD_FLAGS;
+    const int side = flags == HFK_SWAP_SRC_HOST ? 1 : flags == HFK_SWAP_SRC_DEVICE ? 0 : kAskRuntime;
+    return launch_transpose(dev_layer_ptrs, src_block, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, side,
                             workgroups, static_cast<hipStream_t>(stream));
 }
 
@@ -772,7 +779,7 @@ int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs, cons
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipMemcpyAsync(staging, host_block, bytes, hipMemcpyHostToDevice, s);
     if (e != hipSuccess) return (int)e;
-    return launch_transpose(dev_layer_ptrs, staging, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, true,
+    return launch_transpose(dev_layer_ptrs, staging, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, 0,
                             workgroups, s);
 }
 
@@ -782,12 +789,17 @@ int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t de
                                          uint64_t n_dev_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D,
                                          uint32_t elem_bytes, int to_packed, uint32_t flags, uint32_t workgroups,
                                          hfk_stream_t stream) {
-    if ((flags & ~(uint32_t)HFK_SWAP_BESIDE_COMPUTE) != 0) return HFK_ERR_BAD_FLAGS;
+    // What the caller says about the packed pool: the source on the way to the device, the destination back.
+    const uint32_t host_flag = to_packed ? HFK_SWAP_DST_HOST : HFK_SWAP_SRC_HOST;
+    const uint32_t device_flag = to_packed ? HFK_SWAP_DST_DEVICE : HFK_SWAP_SRC_DEVICE;
+    if ((flags & ~(HFK_SWAP_BESIDE_COMPUTE | host_flag | device_flag)) != 0) return HFK_ERR_BAD_FLAGS;
+    if ((flags & host_flag) != 0 && (flags & device_flag) != 0) return HFK_ERR_BAD_FLAGS;
     if (n_pairs == 0) return HFK_OK;
     if (block_pairs == nullptr) return HFK_ERR_NULL_POINTER;
+    const int side = (flags & host_flag) != 0 ? 1 : (flags & device_flag) != 0 ? 0 : kAskRuntime;
     return launch_transpose(dev_layer_ptrs, packed_blocks, block_pairs, n_pairs, packed_block_stride,
                             dev_block_stride, n_packed_blocks, n_dev_blocks, T, L, H, D, elem_bytes, to_packed != 0,
-                            false, workgroups, static_cast<hipStream_t>(stream), (flags & HFK_SWAP_BESIDE_COMPUTE) != 0);
+                            side, workgroups, static_cast<hipStream_t>(stream), (flags & HFK_SWAP_BESIDE_COMPUTE) != 0);
 }
 
 int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, const int64_t* block_pairs,

@@ -43,7 +43,9 @@ void check_aiv(const std::optional<int64_t>& aiv) {
 // allocator recycles its blocks, so a recorded range could outlive the tensor.
 // The reference passes an unchecked nullptr to the kernel here
 // (gather_torch.cpp:51, multi_layer_block_transfer_torch.cpp:78).
-void* device_visible(const at::Tensor& t, const char* what) {
+// `in_host`, when given, is told where the memory lives (the library would otherwise ask the runtime).
+void* device_visible(const at::Tensor& t, const char* what, bool* in_host = nullptr) {
+    if (in_host != nullptr) *in_host = !t.is_cuda();
     if (t.is_cuda()) return t.data_ptr();
     TORCH_CHECK(t.device().is_cpu(), what, ": unsupported device ", t.device());
     void* dev = HostRegisteredMemoryManager::GetInstance().getDevicePtr(t.data_ptr());
@@ -133,12 +135,14 @@ void gather(const at::Tensor& gmEmbed, const at::Tensor& gmEmbedDst, const at::T
                 gmEmbedDst.nbytes(), " bytes, ", numIds * rowBytes, " needed");
 
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(gmEmbedDst));
-    const void* table = device_visible(gmEmbed, "gmEmbed");
+    bool table_in_host = false;
+    const void* table = device_visible(gmEmbed, "gmEmbed", &table_in_host);
     const void* ids = device_visible(gmIds, "gmIds");
     // workgroups 0: the library sizes the grid for where the table lives (HBM, or host memory
-    // behind the PCIe link, the reference's embedding case).
+    // behind the PCIe link, the reference's embedding case), which the tensor has just told.
     check_status(hfk_gather_rows(table, gmEmbedDst.data_ptr(), ids, gmIds.scalar_type() == at::kLong, numIds,
-                                 rowBytes, tableRows, 0, current_stream()),
+                                 rowBytes, tableRows, table_in_host ? HFK_SWAP_SRC_HOST : HFK_SWAP_SRC_DEVICE, 0,
+                                 current_stream()),
                  "hfk_gather_rows");
 }
 
@@ -150,9 +154,11 @@ void multi_layer_block_transfer(const at::Tensor& deviceBlockCachePtrs, const at
     const BlockGeometry g = block_geometry(hostBlockCache);
     check_layer_ptrs(deviceBlockCachePtrs, g.L);
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(deviceBlockCachePtrs));
-    const void* src = device_visible(hostBlockCache, "hostBlockCache");
+    bool src_in_host = false;
+    const void* src = device_visible(hostBlockCache, "hostBlockCache", &src_in_host);
     check_status(hfk_multi_layer_block_transfer(deviceBlockCachePtrs.data_ptr(), src, g.T, g.L, g.H, g.D, g.elem,
-                                                0, current_stream()),
+                                                src_in_host ? HFK_SWAP_SRC_HOST : HFK_SWAP_SRC_DEVICE, 0,
+                                                current_stream()),
                  "hfk_multi_layer_block_transfer");
 }
 
@@ -203,13 +209,20 @@ void multi_layer_block_table_transfer(const at::Tensor& deviceLayerCachePtrs, co
     if (blockPairs.size(0) == 0 || blockBytes == 0) return;
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(deviceLayerCachePtrs));
     const uint32_t cap = workgroup_cap(workgroups);   // 0: the library sizes the grid for where the pool lives
+    bool pool_in_host = false;
+    void* pool = device_visible(hostBlockPool, "hostBlockPool", &pool_in_host);
+    uint32_t bits = flag_bits(flags, "multi_layer_block_table_transfer");
+    constexpr uint32_t kSideBits = HFK_SWAP_SRC_HOST | HFK_SWAP_DST_HOST | HFK_SWAP_SRC_DEVICE | HFK_SWAP_DST_DEVICE;
+    if ((bits & kSideBits) == 0) {   // the tensor knows where the pool lives: spare the library the question
+        bits |= toHost ? (pool_in_host ? HFK_SWAP_DST_HOST : HFK_SWAP_DST_DEVICE)
+                       : (pool_in_host ? HFK_SWAP_SRC_HOST : HFK_SWAP_SRC_DEVICE);
+    }
     check_status(hfk_multi_layer_block_table_transfer(
-                     deviceLayerCachePtrs.data_ptr(), static_cast<uint64_t>(deviceBlockStride),
-                     device_visible(hostBlockPool, "hostBlockPool"), blockBytes,
+                     deviceLayerCachePtrs.data_ptr(), static_cast<uint64_t>(deviceBlockStride), pool, blockBytes,
                      static_cast<const int64_t*>(device_visible(blockPairs, "blockPairs")),
                      static_cast<uint64_t>(blockPairs.size(0)), static_cast<uint64_t>(hostBlockPool.size(0)),
-                     static_cast<uint64_t>(deviceBlocks), T, L, H, D, elem, toHost ? 1 : 0,
-                     flag_bits(flags, "multi_layer_block_table_transfer"), cap, current_stream()),
+                     static_cast<uint64_t>(deviceBlocks), T, L, H, D, elem, toHost ? 1 : 0, bits, cap,
+                     current_stream()),
                  "hfk_multi_layer_block_table_transfer");
 }
 

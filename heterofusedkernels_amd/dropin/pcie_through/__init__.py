@@ -6,6 +6,8 @@ _load_opextension_so()
 SWAP_DST_HOST = 1        # the destination planes are host memory (swap-out)
 SWAP_SRC_HOST = 2        # the source planes are host memory (swap-in)
 SWAP_BESIDE_COMPUTE = 4  # other kernels run at the same time: small, paced launch
+SWAP_SRC_DEVICE = 8      # the source is device memory (saves the library a question to the runtime)
+SWAP_DST_DEVICE = 16     # the destination is device memory
 
 
 def plane_pointer_table(planes, device):

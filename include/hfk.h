@@ -29,7 +29,7 @@ extern "C" {
 #define HFK_API __attribute__((visibility("default")))
 
 #define HFK_VERSION_MAJOR 0
-#define HFK_VERSION_MINOR 2
+#define HFK_VERSION_MINOR 3
 
 /* A hipStream_t passed as an opaque pointer; NULL is the null stream. */
 typedef void* hfk_stream_t;
@@ -65,18 +65,22 @@ HFK_API const char* hfk_status_string(int status);
  *   ids         device-visible, int64 (ids_are_i64 != 0) or int32 indices
  *   table_rows  number of rows in table; an id outside [0, table_rows) leaves its
  *               dst row untouched. 0 disables the check (the reference never checks).
- *   workgroups  upper bound on workgroups launched, 0 = library default: one workgroup per 16 KiB
- *               of output for a table in device memory; for a table in host memory (the library
- *               asks the runtime where `table` lives) a gather of more than 4 MiB runs on 64
- *               workgroups, which saturate the PCIe link (55-57 GB/s for 1 KiB rows) and slow
- *               kernels on other streams 2x where the device-sized grid slows them 5x.
+ *   flags       0, HFK_SWAP_SRC_HOST (the table is host memory) or HFK_SWAP_SRC_DEVICE (it is device
+ *               memory). Where the table lives shapes the launch; with 0 the library asks the
+ *               runtime (for gathers of 64 KiB and more), which costs the calling thread about 5 us
+ *               per call: as much as the whole launch of a small gather. A caller that knows says so.
+ *   workgroups  upper bound on workgroups launched, 0 = library default: one workgroup per chunk
+ *               of output for a table in device memory; for a table in host memory a gather of
+ *               more than 4 MiB runs on 64 workgroups, which saturate the PCIe link (55-57 GB/s
+ *               for 1 KiB rows) and slow kernels on other streams 2x where the device-sized grid
+ *               slows them 5x.
  *
  * n_ids == 0 is a successful no-op. Rows of any byte size and alignment are
  * accepted; 16-byte aligned rows take the vectorised path.
  */
 HFK_API int hfk_gather_rows(const void* table, void* dst, const void* ids, int ids_are_i64,
                     uint64_t n_ids, uint64_t row_bytes, uint64_t table_rows,
-                    uint32_t workgroups, hfk_stream_t stream);
+                    uint32_t flags, uint32_t workgroups, hfk_stream_t stream);
 
 /*
  * Layout-converting transfer of one KV block across all layers:
@@ -96,10 +100,12 @@ HFK_API int hfk_gather_rows(const void* table, void* dst, const void* ids, int i
  *                   device-visible buffer of H*T*D*elem_bytes bytes ([H,T,D])
  *   src_block       device-visible [T,L,H,D] block (pinned host memory in the
  *                   reference's use, device memory for the staged variant)
+ *   flags           0, HFK_SWAP_SRC_HOST or HFK_SWAP_SRC_DEVICE: where src_block lives, if the caller
+ *                   knows (with 0 the library asks the runtime, about 5 us per call)
  */
 HFK_API int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const void* src_block,
                                    uint32_t T, uint32_t L, uint32_t H, uint32_t D,
-                                   uint32_t elem_bytes, uint32_t workgroups,
+                                   uint32_t elem_bytes, uint32_t flags, uint32_t workgroups,
                                    hfk_stream_t stream);
 
 /*
@@ -139,9 +145,13 @@ HFK_API int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_pt
  *   block_pairs      device-visible int64 [n_pairs, 2] = (packed_block, dev_block)
  *   n_packed_blocks, n_dev_blocks  pool sizes; a pair outside them is skipped,
  *                    0 disables that side's check
- *   flags            0, or HFK_SWAP_BESIDE_COMPUTE: other kernels run meanwhile and matter. Only the
- *                    default grid changes (packed pool in host memory: 24 workgroups host -> device,
- *                    48 device -> host, 16 with the flag), never the result.
+ *   flags            any combination of HFK_SWAP_BESIDE_COMPUTE (other kernels run meanwhile and matter) and
+ *                    one statement about the packed pool, which is the source when to_packed == 0 and
+ *                    the destination otherwise: HFK_SWAP_SRC_HOST / HFK_SWAP_DST_HOST (host memory) or
+ *                    HFK_SWAP_SRC_DEVICE / HFK_SWAP_DST_DEVICE (device memory); without one the library
+ *                    asks the runtime (about 5 us per call). Only the default grid changes (packed
+ *                    pool in host memory: 24 workgroups host -> device, 48 device -> host, 16 with
+ *                    HFK_SWAP_BESIDE_COMPUTE), never the result.
  * Strides must be at least one block of their side. Destination blocks must be distinct.
  */
 HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uint64_t dev_block_stride,
@@ -202,6 +212,8 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
 #define HFK_SWAP_DST_HOST 1u
 #define HFK_SWAP_SRC_HOST 2u
 #define HFK_SWAP_BESIDE_COMPUTE 4u
+#define HFK_SWAP_SRC_DEVICE 8u    /* the source is device memory: for entry points that would otherwise ask the runtime */
+#define HFK_SWAP_DST_DEVICE 16u   /* the destination is device memory: likewise */
 HFK_API int hfk_swap_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs,
                     const int64_t* block_pairs, uint32_t n_planes, uint64_t n_pairs,
                     uint64_t block_bytes, uint64_t src_block_stride,

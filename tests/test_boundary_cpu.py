@@ -66,7 +66,7 @@ def test_reference_style_native_consumer_compiles():
 
 def test_capi_loads_and_reports():
     L = capi.load()
-    assert L.hfk_version() == 2
+    assert L.hfk_version() == 3
     assert capi.status_string(0) == "ok"
     assert "NULL" in capi.status_string(-1)
     assert capi.get_tuning(capi.KNOB_UNROLL) in (1, 2, 4, 8, 16)
@@ -93,7 +93,11 @@ def test_argument_errors_are_reported_before_any_gpu_work():
     assert capi.swap_blocks(8, 8, 8, 2, 2, 32, 16, 32) == -2           # stride < block
     assert capi.swap_blocks(8, 8, 8, 2, 2, 0, 16, 32) == -2
     assert capi.swap_blocks(8, 8, 8, 2, 1 << 33, 16, 16, 16) == -3
-    assert capi.swap_blocks(8, 8, 8, 2, 2, 16, 16, 16, flags=8) == -6  # unknown flag bit
+    assert capi.swap_blocks(8, 8, 8, 2, 2, 16, 16, 16, flags=8) == -6  # a flag this entry point does not take
+    assert capi.gather_rows(8, 8, 8, True, 4, 16, flags=capi.SWAP_DST_HOST) == -6
+    assert capi.gather_rows(8, 8, 8, True, 4, 16, flags=capi.SWAP_SRC_HOST | capi.SWAP_SRC_DEVICE) == -6
+    assert capi.gather_rows(0, 0, 0, True, 0, 16, flags=capi.SWAP_SRC_HOST) == 0
+    assert capi.multi_layer_block_transfer(8, 8, 4, 4, 4, 4, 2, flags=capi.SWAP_BESIDE_COMPUTE) == -6
     assert capi.swap_blocks(0, 0, 0, 0, 0, 16, 16, 16, flags=capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE) == 0
     assert capi.gather_blocks(8, 8, 0, 2, 2, 16, 16) == -1
     assert capi.gather_blocks(8, 8, 8, 2, 2, 32, 16) == -2

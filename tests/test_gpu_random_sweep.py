@@ -122,6 +122,13 @@ def test_random_swap_blocks(seed):
         assert np.array_equal(src.now(), src.before), "source changed"
 
 
+def _pool_side(to_packed, packed_host):
+    """The flag that says, truthfully, where the packed pool of a table transfer lives."""
+    if to_packed:
+        return capi.SWAP_DST_HOST if packed_host else capi.SWAP_DST_DEVICE
+    return capi.SWAP_SRC_HOST if packed_host else capi.SWAP_SRC_DEVICE
+
+
 @pytest.mark.parametrize("seed", range(4))
 def test_random_gather_rows_and_blocks(seed):
     rng = np.random.default_rng(2000 + seed + 17 * SEED_OFFSET)
@@ -142,8 +149,10 @@ def test_random_gather_rows_and_blocks(seed):
         if with_bad and n:
             ids[rng.integers(0, n, 3)] = np.array([-1, rows, rows + 5], dtype=id_dtype)
         ids_d = torch.from_numpy(ids).to(DEV) if n else torch.zeros(1, dtype=torch.int64, device=DEV)
+        # what the caller may say about the table: nothing, or the truth (the launch shape follows, never the bytes)
+        side = int(rng.choice([0, capi.SWAP_SRC_HOST if table_host else capi.SWAP_SRC_DEVICE]))
         capi.check(capi.gather_rows(table.addr + toff, dst.addr + doff, ids_d.data_ptr(), id_dtype is np.int64, n, rb,
-                                    rows, wg, stream_handle()), "hfk_gather_rows")
+                                    rows, wg, stream_handle(), side), "hfk_gather_rows")
         torch.cuda.synchronize()
         want = dst.before.copy()
         ok = (ids >= 0) & (ids < rows)
@@ -203,7 +212,8 @@ def test_random_block_table_transfer(seed):
         capi.check(capi.multi_layer_block_table_transfer(
             lptrs.data_ptr(), layer_bytes, packed.addr + poff, block_bytes, pairs_d.data_ptr() if pairs_d is not None else None,
             pairs_all.shape[0], packed_blocks, dev_blocks, T, L, H, D, e, int(to_packed), wg, stream_handle(),
-            int(rng.choice([0, capi.SWAP_BESIDE_COMPUTE]))), "hfk_multi_layer_block_table_transfer")
+            int(rng.choice([0, capi.SWAP_BESIDE_COMPUTE])) | int(rng.choice([0, _pool_side(to_packed, packed_host)]))),
+            "hfk_multi_layer_block_table_transfer")
         torch.cuda.synchronize()
         want_layers = layers.before.copy().reshape(L, dev_blocks, layer_bytes)
         want_packed = packed.before.copy()
