@@ -84,9 +84,11 @@ def test_swap_and_gather_replay_in_a_hip_graph():
 
 def test_duplex_staged_and_table_transfer_replay_in_a_hip_graph():
     """The newer entry points record as well: the duplex swap (one kernel), the staged swap (kernel +
-    DMA copy nodes; its host slot list is read at capture time and therefore fixed for the graph) and the
-    block-table transfer in both directions."""
-    announce("HIP graph: duplex swap + staged swap + block-table transfer, replayed 3 times")
+    DMA copy nodes; its host slot list is read at capture time and therefore fixed for the graph), the same
+    through the library's own staging array (the entry point made for callers that cannot allocate, such as
+    this one; its first call, which asks the runtime for the array's address, is the eager run before the
+    capture) and the block-table transfer in both directions."""
+    announce("HIP graph: duplex swap + staged swap (caller's and library's staging) + block-table transfer, replayed 3 times")
     planes, blocks, bb, n = 4, 48, 32768, 10
     dev = [torch.zeros(blocks, bb, dtype=torch.uint8, device=DEV) for _ in range(planes)]
     pool = memory.alloc_numa_pinned_tensor(planes * blocks * bb)
@@ -98,6 +100,9 @@ def test_duplex_staged_and_table_transfer_replay_in_a_hip_graph():
     staged_ids = torch.zeros(n, dtype=torch.int64, device=DEV)
     staged_slots = torch.arange(30, 30 + n)                               # fixed at capture
     staging = torch.zeros(planes, n, bb, dtype=torch.uint8, device=DEV)
+    n_static = 8
+    static_ids = torch.zeros(n_static, dtype=torch.int64, device=DEV)
+    static_slots = torch.arange(40, 40 + n_static)                         # fixed at capture, after the staged swap's slots
     T, L, H, D = 32, 3, 2, 64
     tpool = memory.alloc_numa_pinned_tensor(6 * T * L * H * D).view(6, T, L, H, D)
     tback = memory.alloc_numa_pinned_tensor(6 * T * L * H * D).view(6, T, L, H, D)
@@ -109,6 +114,8 @@ def test_duplex_staged_and_table_transfer_replay_in_a_hip_graph():
         torch.ops.pcie_through.swap_blocks_duplex(dtab, htab, out_pairs, in_pairs, bb, bb, bb, blocks, blocks)
         torch.ops.pcie_through.swap_blocks_staged(dtab, host_addrs, staged_ids, staged_slots, staging, bb, bb, bb, True,
                                                   blocks, blocks)
+        torch.ops.pcie_through.swap_blocks_staged_static(dtab, host_addrs, static_ids, static_slots, bb, bb, bb, True,
+                                                         blocks, blocks)
         torch.ops.pcie_through.multi_layer_block_table_transfer(lptrs, tpool, tpairs, H * T * D, 5, False)
         torch.ops.pcie_through.multi_layer_block_table_transfer(lptrs, tback, tpairs, H * T * D, 5, True)
 
@@ -128,6 +135,8 @@ def test_duplex_staged_and_table_transfer_replay_in_a_hip_graph():
         out_pairs.copy_(state["out"])
         in_pairs.copy_(state["in"])
         staged_ids.copy_(state["staged"])
+        state["static"] = 30 + torch.randperm(blocks - 30, generator=gen)[:n_static]
+        static_ids.copy_(state["static"])
         tpool.copy_(torch.randint(-128, 128, tuple(tpool.shape), dtype=torch.int8, generator=gen))
         tback.zero_()
         state["tpairs"] = torch.stack([torch.randperm(6, generator=gen)[:4], torch.randperm(5, generator=gen)[:4]], 1)
@@ -140,6 +149,7 @@ def test_duplex_staged_and_table_transfer_replay_in_a_hip_graph():
             assert torch.equal(h[st["out"][:, 1]], st["dev"][p][st["out"][:, 0]]), tag + " duplex out"
             assert torch.equal(d[st["in"][:, 1]], st["host"][p][st["in"][:, 0]]), tag + " duplex in"
             assert torch.equal(h[30:30 + n], st["dev"][p][st["staged"]]), tag + " staged"
+            assert torch.equal(h[40:40 + n_static], st["dev"][p][st["static"]]), tag + " staged through the library's array"
         for hb, _ in st["tpairs"].tolist():
             assert torch.equal(tback[hb], tpool[hb]), tag + " table transfer round trip"
 
