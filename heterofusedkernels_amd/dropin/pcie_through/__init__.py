@@ -35,3 +35,21 @@ def plane_pointer_table(planes, device):
                 raise RuntimeError("plane is not device-visible host memory")
             addrs.append(dev)
     return torch.tensor(addrs, dtype=torch.int64).to(device)
+
+
+def swap_flags(dst_planes, src_planes, beside_compute=False):
+    """The ``flags`` argument of ``swap_blocks`` for these two plane lists: names the side that is
+    host memory (so the launch is sized and paced for the PCIe link instead of guessing) and, with
+    ``beside_compute``, says that other kernels run meanwhile and matter. Planes of one side must all
+    live on the same kind of memory."""
+    def side(planes, what):
+        kinds = {bool(t.is_cuda) for t in planes}
+        if len(kinds) != 1:
+            raise ValueError("%s planes mix device and host memory" % what)
+        return kinds.pop()
+    flags = SWAP_BESIDE_COMPUTE if beside_compute else 0
+    if not side(dst_planes, "destination"):
+        flags |= SWAP_DST_HOST
+    if not side(src_planes, "source"):
+        flags |= SWAP_SRC_HOST
+    return flags

@@ -168,9 +168,24 @@ def test_op_schemas_match_reference():
 def test_flag_constants_match_the_header():
     import pcie_through
     text = open(os.path.join(ROOT, "include", "hfk.h")).read()
-    for name in ("SWAP_DST_HOST", "SWAP_SRC_HOST", "SWAP_BESIDE_COMPUTE"):
+    for name in ("SWAP_DST_HOST", "SWAP_SRC_HOST", "SWAP_BESIDE_COMPUTE", "SWAP_SRC_DEVICE", "SWAP_DST_DEVICE"):
         value = int(re.search(r"#define HFK_%s (\d+)u" % name, text).group(1))
         assert getattr(pcie_through, name) == value == getattr(capi, name)
+
+
+def test_swap_flags_helper_reads_the_sides_off_the_planes():
+    import pcie_through
+    host = [torch.zeros(4), torch.zeros(4)]
+
+    class Dev:                                         # stands for a device plane: is_cuda is all the helper reads
+        is_cuda = True
+    assert pcie_through.swap_flags(host, [Dev(), Dev()]) == pcie_through.SWAP_DST_HOST
+    assert pcie_through.swap_flags([Dev()], host) == pcie_through.SWAP_SRC_HOST
+    assert pcie_through.swap_flags([Dev()], [Dev()]) == 0
+    assert pcie_through.swap_flags(host, [Dev()], beside_compute=True) == \
+        pcie_through.SWAP_DST_HOST | pcie_through.SWAP_BESIDE_COMPUTE
+    with pytest.raises(ValueError):
+        pcie_through.swap_flags(host + [Dev()], [Dev()])
 
 
 def test_ops_have_no_cpu_fallback():
