@@ -144,7 +144,7 @@ constexpr uint32_t kDuplexWorkgroups = 32;
 constexpr uint32_t kBesideDuplexWorkgroups = 16;
 constexpr int kBesideDuplexUnroll = 2;
 constexpr uint32_t kBesideTransferWorkgroups = 16;
-constexpr uint32_t kTransferToHostWorkgroups = 48;
+constexpr uint32_t kTransferToHostWorkgroups = 32;
 constexpr uint32_t kTransferFromHostWorkgroups = 24;
 constexpr uint32_t kSingleBlockTransferWorkgroups = 32;
 constexpr uint32_t kHostGatherWorkgroups = 64;
@@ -438,9 +438,8 @@ int gather_rows_typed(const void* table, void* dst, const IdT* ids, uint64_t n_i
 }
 
 // ---- transpose ------------------------------------------------------------
-template <typename V>
-void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, bool to_packed, hipStream_t s) {
-    constexpr int U = hfk::kTransposeUnroll;
+template <typename V, int U>
+void launch_transpose_u(const TransposeArgs& a, uint32_t grid, int nt, bool to_packed, hipStream_t s) {
     if (to_packed) {
         if (nt & 3) hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, 3>), dim3(grid), dim3(256), 0, s, a);
         else hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, 0>), dim3(grid), dim3(256), 0, s, a);
@@ -449,6 +448,15 @@ void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, bool to_p
         else hipLaunchKernelGGL((transpose_kernel<V, U, 0>), dim3(grid), dim3(256), 0, s, a);
     }
 }
+
+template <typename V>
+void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, bool to_packed, int unroll, hipStream_t s) {
+    switch (unroll) {
+        case hfk::kTransposeUnroll: launch_transpose_u<V, hfk::kTransposeUnroll>(a, grid, nt, to_packed, s); break;
+        default: launch_transpose_u<V, hfk::kTransposeUnrollToHost>(a, grid, nt, to_packed, s); break;
+    }
+}
+
 
 // Where an address lives: 1 = host memory (pinned, device-mapped), 0 = device memory, -1 = the
 // runtime does not know the pointer.
@@ -471,20 +479,24 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
                      uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
                      bool to_packed, int packed_side, uint32_t workgroups, hipStream_t s,
                      bool beside_compute = false) {
+    if (dev_layer_ptrs == nullptr || packed == nullptr) return HFK_ERR_NULL_POINTER;
+    // With the packed side in host memory the PCIe link is the bound and a small grid does; an
+    // unknown pointer gets the small grid too. Measured on the reference's four shapes, 8 blocks per
+    // launch: host -> device (two units per lane) 56.0-57.0 GB/s on 16 workgroups, 57.1-57.6 on 24-36,
+    // 54.1-54.6 on 48-56 (a dip that repeats), 56.6-57.5 on 80-96; device -> host 52.2-53.2 on 48
+    // workgroups of two units per lane (49.9 on one shape in one run), 53.2-53.9 on 32 of eight: toward
+    // the host a workgroup that moves more per turn is offered to the link more evenly, as for the
+    // swap-out. (Pacing, which gains a swap-out 1-2 %, does not pay here: it gains 0.8 GB/s on the
+    // eight-head shapes and loses up to 3.5 on the one-head shapes, whose 128-byte rows come from 64
+    // different layer caches per chunk and fall behind any schedule.)
+    const int side = packed_side == kAskRuntime ? memory_side(packed) : packed_side;
+    const int unroll = to_packed && side != 0 ? hfk::kTransposeUnrollToHost : hfk::kTransposeUnroll;
     TransposeArgs a;
     uint32_t unit = 16;
     int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, packed, pairs, n_pairs, packed_stride, layered_stride,
-                                 packed_blocks, layered_blocks, T, L, H, D, elem_bytes);
+                                 packed_blocks, layered_blocks, T, L, H, D, elem_bytes, unroll);
     if (rc != 0) return rc;
     if (a.n_work == 0) return HFK_OK;  // nothing to move
-    // With the packed side in host memory the PCIe link is the bound and a small grid does; an
-    // unknown pointer gets the small grid too. Measured on the reference's four shapes, 8 blocks per
-    // launch: host -> device 56.0-57.0 GB/s on 16 workgroups, 57.1-57.6 on 24-36, 54.1-54.6 on 48-56
-    // (a dip that repeats), 56.6-57.5 on 80-96; device -> host 48-52 on 16, 51-52 on 24, 52-54.7 from
-    // 32 on and flat. (Pacing, which gains a swap-out 1-2 %, does not pay toward the host here: it
-    // gains 0.8 GB/s on the eight-head shapes and loses up to 3.5 on the one-head shapes, whose
-    // 128-byte rows come from 64 different layer caches per chunk and fall behind any schedule.)
-    const int side = packed_side == kAskRuntime ? memory_side(packed) : packed_side;
     if (workgroups == 0 && side != 0) {
         // One block (the reference's op: 4-64 MiB, over in 0.1-1.2 ms) is sized for speed alone; a
         // block table may run for many milliseconds beside other kernels and gets the smaller grid.
@@ -497,9 +509,9 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
-    if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, to_packed, s);
-    else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, to_packed, s);
-    else launch_transpose_v<uint8_t>(a, grid, nt, to_packed, s);
+    if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, to_packed, unroll, s);
+    else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, to_packed, unroll, s);
+    else launch_transpose_v<uint8_t>(a, grid, nt, to_packed, unroll, s);
     return finish_launch();
 }
 

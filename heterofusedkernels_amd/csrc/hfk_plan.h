@@ -22,9 +22,11 @@ constexpr uint64_t kWideRowBytes = 4096;
 // (a 1 MiB gather of 1 KiB rows over PCIe takes 22 us against 27).
 constexpr int kFlatUnrollDevice = 1;
 constexpr int kFlatUnrollHost = 4;
-// Units per lane of the layout-converting transfer (one block from host memory 51-55 GB/s, eight
-// blocks 56-57 GB/s in and 52-53 out; one unit per lane loses 1 GB/s on the way out, four on the way in).
+// Units per lane of the layout-converting transfer: two (one block from host memory 53-57 GB/s,
+// eight blocks 57 GB/s; one unit per lane needs twice the workgroups, four gain nothing), except
+// toward a packed pool in host memory, where eight hold 53.2-53.9 GB/s and two 52.2-53.2.
 constexpr int kTransposeUnroll = 2;
+constexpr int kTransposeUnrollToHost = 8;
 
 // Raw rate of a PCIe link in MB/s (lanes x GT/s x line encoding / 8) from the two strings sysfs
 // shows for it, e.g. "32.0 GT/s PCIe" and "16"; -1 when either does not parse. Links below
@@ -109,7 +111,7 @@ inline int plan_flat_gather(FlatGatherArgs<IdT>& a, FlatGatherPlan& p, uint64_t 
 inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_layer_ptrs, const void* packed,
                           const int64_t* pairs, uint64_t n_pairs, uint64_t packed_stride, uint64_t layered_stride,
                           uint64_t packed_blocks, uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H,
-                          uint32_t D, uint32_t elem_bytes) {
+                          uint32_t D, uint32_t elem_bytes, int unroll = kTransposeUnroll) {
     a = TransposeArgs{};
     if (dev_layer_ptrs == nullptr || packed == nullptr) return HFK_ERR_NULL_POINTER;
     if (elem_bytes == 0) return HFK_ERR_BAD_SIZE;
@@ -128,7 +130,7 @@ inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_
     const uint32_t unit = pick_unit(align);
     const uint64_t row_units = row_bytes / unit;
     const uint64_t total = rows * row_units;
-    const uint64_t chunk_units = (uint64_t)kWorkgroupLanes * kTransposeUnroll;
+    const uint64_t chunk_units = (uint64_t)kWorkgroupLanes * (uint64_t)unroll;
     const uint64_t chunks = (total + chunk_units - 1) / chunk_units;
     if (n_pairs > kU32Max || chunks * n_pairs > kU32Max) return HFK_ERR_TOO_LARGE;
     a.layer_ptrs = static_cast<const uint64_t*>(dev_layer_ptrs);

@@ -150,7 +150,7 @@ HFK_API int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_pt
  *                    the destination otherwise: HFK_SWAP_SRC_HOST / HFK_SWAP_DST_HOST (host memory) or
  *                    HFK_SWAP_SRC_DEVICE / HFK_SWAP_DST_DEVICE (device memory); without one the library
  *                    asks the runtime (about 5 us per call). Only the default grid changes (packed
- *                    pool in host memory: 24 workgroups host -> device, 48 device -> host, 16 with
+ *                    pool in host memory: 24 workgroups host -> device, 32 device -> host, 16 with
  *                    HFK_SWAP_BESIDE_COMPUTE), never the result.
  * Strides must be at least one block of their side. Destination blocks must be distinct.
  */

@@ -468,13 +468,13 @@ void case_gather_rows(uint64_t table_rows, uint64_t n_ids, uint64_t row_bytes, s
 }
 
 // ---- transpose -------------------------------------------------------------
-template <bool TO_PACKED>
+template <bool TO_PACKED, int UNROLL = kTransposeUnroll>
 void walk_transpose(const TransposeArgs& a, uint32_t unit, uint32_t grid_cap) {
     if (a.n_work == 0) return;
     const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
-    if (unit == 16u) walk(a, grid, transpose_body<vec16, kTransposeUnroll, 3, TO_PACKED>);
-    else if (unit == 4u) walk(a, grid, transpose_body<uint32_t, kTransposeUnroll, 0, TO_PACKED>);
-    else walk(a, grid, transpose_body<uint8_t, kTransposeUnroll, 0, TO_PACKED>);
+    if (unit == 16u) walk(a, grid, transpose_body<vec16, UNROLL, 3, TO_PACKED>);
+    else if (unit == 4u) walk(a, grid, transpose_body<uint32_t, UNROLL, 0, TO_PACKED>);
+    else walk(a, grid, transpose_body<uint8_t, UNROLL, 0, TO_PACKED>);
 }
 
 // single block, the reference's op
@@ -545,9 +545,14 @@ void case_transpose_table(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32
     }
     TransposeArgs a;
     uint32_t unit = 0;
+    // toward the packed side both launch shapes exist (a pool in device memory, a pool in host memory):
+    // alternate between them from case to case
+    static unsigned to_packed_cases = 0;
+    const bool to_host_shape = to_packed && (to_packed_cases++ % 2 == 1);
     int rc = plan_transpose(a, &unit, lp.data(), packed.p, pairs.data(), n_pairs, ps, ls, packed_blocks, dev_blocks, T,
-                            L, H, D, elem);
+                            L, H, D, elem, to_host_shape ? kTransposeUnrollToHost : kTransposeUnroll);
     if (rc != HFK_OK) { ++g_failures; std::printf("plan_transpose(table) rc=%d\n", rc); }
+    else if (to_host_shape) walk_transpose<true, kTransposeUnrollToHost>(a, unit, grid_cap);
     else if (to_packed) walk_transpose<true>(a, unit, grid_cap);
     else walk_transpose<false>(a, unit, grid_cap);
     oracle_multi_layer_block_table_transfer(ep.data(), ls, packed_exp.p, ps, good.data(), good.size() / 2, T, L, H, D,
