@@ -1,6 +1,10 @@
+import weakref
+
 from ._load import _load_opextension_so
 
 _load_opextension_so()
+
+_table_in_host = {}   # data_ptr of a plane pointer table -> whether its planes are host memory
 
 # flags of torch.ops.pcie_through.swap_blocks (hfk.h: HFK_SWAP_*)
 SWAP_DST_HOST = 1        # the destination planes are host memory (swap-out)
@@ -22,6 +26,7 @@ def plane_pointer_table(planes, device):
     import torch
     from heterofusedkernels import memory
 
+    planes = list(planes)
     addrs = []
     for t in planes:
         if t.is_cuda:
@@ -34,7 +39,29 @@ def plane_pointer_table(planes, device):
             if dev == 0:
                 raise RuntimeError("plane is not device-visible host memory")
             addrs.append(dev)
-    return torch.tensor(addrs, dtype=torch.int64).to(device)
+    table = torch.tensor(addrs, dtype=torch.int64).to(device)
+    kinds = {bool(t.is_cuda) for t in planes}
+    if len(kinds) == 1:   # remembered for swap_blocks() below, for as long as the table lives
+        key = table.data_ptr()
+        _table_in_host[key] = not kinds.pop()
+        weakref.finalize(table, _table_in_host.pop, key, None)
+    return table
+
+
+def swap_blocks(dst_table, src_table, block_pairs, block_bytes, src_block_stride, dst_block_stride, src_blocks=0,
+                dst_blocks=0, workgroups=None, flags=None, beside_compute=False):
+    """``torch.ops.pcie_through.swap_blocks`` with the flags filled in: for tables that came from
+    ``plane_pointer_table`` the side that is host memory is known and named, so the launch is sized
+    and paced for the PCIe link instead of guessing. ``flags`` given explicitly are passed through."""
+    import torch
+    if flags is None:
+        flags = SWAP_BESIDE_COMPUTE if beside_compute else 0
+        if _table_in_host.get(dst_table.data_ptr()):
+            flags |= SWAP_DST_HOST
+        if _table_in_host.get(src_table.data_ptr()):
+            flags |= SWAP_SRC_HOST
+    torch.ops.pcie_through.swap_blocks(dst_table, src_table, block_pairs, block_bytes, src_block_stride,
+                                       dst_block_stride, src_blocks, dst_blocks, workgroups, flags)
 
 
 def swap_flags(dst_planes, src_planes, beside_compute=False):

@@ -580,6 +580,35 @@ def test_strided_planes():
     assert (d[:, 0] == 0).all() and d[:, 1].sum() == s[[0, 9, 4], 0].sum()
 
 
+def test_python_swap_wrapper_names_the_host_side_by_itself(memory):
+    """pcie_through.swap_blocks: the op with its flags read off tables that plane_pointer_table built."""
+    import gc
+    announce("pcie_through.swap_blocks wrapper: out and back, flags inferred from the tables")
+    planes, blocks, bb, n = 3, 40, 32768, 12
+    gen = torch.Generator().manual_seed(321)
+    dev = [torch.randint(0, 256, (blocks, bb), dtype=torch.uint8, generator=gen).to(DEV) for _ in range(planes)]
+    pool = memory.alloc_numa_pinned_tensor(planes * blocks * bb)
+    host = list(pool.view(torch.uint8).view(planes, blocks, bb).unbind(0))
+    dtab, htab = pcie_through.plane_pointer_table(dev, DEV), pcie_through.plane_pointer_table(host, DEV)
+    assert pcie_through._table_in_host[htab.data_ptr()] is True and pcie_through._table_in_host[dtab.data_ptr()] is False
+    src, dst = torch.randperm(blocks, generator=gen)[:n], torch.randperm(blocks, generator=gen)[:n]
+    before = [d.cpu() for d in dev]
+    pcie_through.swap_blocks(htab, dtab, torch.stack([src, dst], 1).to(DEV), bb, bb, bb, blocks, blocks)
+    back = torch.roll(src, 1)
+    pcie_through.swap_blocks(dtab, htab, torch.stack([dst, back], 1).to(DEV), bb, bb, bb, blocks, blocks,
+                             beside_compute=True)
+    torch.cuda.synchronize()
+    for p in range(planes):
+        assert torch.equal(host[p][dst], before[p][src]), "swap-out through the wrapper"
+        want = before[p].clone()
+        want[back] = before[p][src]
+        assert torch.equal(dev[p].cpu(), want), "swap-in through the wrapper"
+    key = htab.data_ptr()
+    del htab
+    gc.collect()
+    assert key not in pcie_through._table_in_host          # the note goes when the table goes
+
+
 @pytest.mark.parametrize("args", [(), ("3", "40", "4112", "20"), ("64", "128", "32768", "64")],
                          ids=["defaults", "odd_block_size", "config2_planes"])
 def test_plain_c_client_runs_the_swap_path(args):
