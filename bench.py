@@ -518,6 +518,20 @@ def section_staged(b, w, steps, warmup, out_flags):
     idle_ticks = int(payload / 55e9 * 1e8)                                  # as long as one swap
     ways["one_idle_wavefront"] = lambda st: bench_lib.hfkb_idle_resident(1, 64, idle_ticks, st)
     ways["sixteen_idle_workgroups"] = lambda st: bench_lib.hfkb_idle_resident(16, 256, idle_ticks, st)
+    # Reading host memory and nothing else, through the vector memory path (24 workgroups, like the
+    # beside-compute swap-in) and through the scalar path (40 workgroups of 8 wavefronts): the same bytes
+    # of the host pool, a checksum kept.
+    bench_lib.hfkb_host_read.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_void_p,
+                                         ctypes.c_void_p]
+    read_bytes = min(payload, w.host_pools[0].numel()) & ~255
+    read_from = b.memory.get_device_ptr(w.host_pools[0].data_ptr())
+    checksums = torch.zeros(40 * 256, dtype=torch.int32, device=b.dev)
+    ways["host_read_vector_path"] = lambda st: bench_lib.hfkb_host_read(0, read_from, read_bytes, 24, checksums.data_ptr(), st)
+    ways["host_read_scalar_path"] = lambda st: bench_lib.hfkb_host_read(1, read_from, read_bytes, 40, checksums.data_ptr(), st)
+    host_read_gbps = {}
+    for name in ("host_read_vector_path", "host_read_scalar_path"):
+        _, ms_r = b.timed(lambda: ways[name](stream), max(3, steps // 4), 1)
+        host_read_gbps[name] = round(read_bytes / (ms_r * 1e6), 2)
     # own rate of the beside-compute launch shape, GPU otherwise idle; result checked like the plain swap-out's
     for p_ in range(planes):
         w.host_planes[p_][w.dst_ids] = 0
@@ -545,6 +559,7 @@ def section_staged(b, w, steps, warmup, out_flags):
     beside_json = {"swap_out_GBps": payload / (ms_bo * 1e6), "swap_in_GBps": payload / (ms_bi * 1e6),
                    "link_MBps_from_sysfs": capi.get_tuning(capi.KNOB_LINK_MBPS),
                    "neighbour_ms_alone": alone,
+                   "host_read_GBps": host_read_gbps,
                    "neighbour_slowdown": slowdown,
                    "how": "each neighbour runs %s times on one stream while %d swaps of %d MiB are queued on another; "
                           "x = its time per call / its time alone; null = the swaps ended first. one_idle_wavefront / "

@@ -8,6 +8,10 @@
 //    one workgroup per chunk of 256 * UNROLL 16-byte vectors, UNROLL loads before the first store)
 //    when it only reads, only writes, or copies a contiguous buffer. The read-only and write-only
 //    rates bound any copy: moving N bytes takes at least N / read_rate + N / write_rate.
+//  * hfkb_host_read: reads pinned host memory and keeps only a checksum, either through the vector
+//    memory path (what every copy kernel uses) or through the scalar (constant) path. A compute unit
+//    returns the loads of each path in order, so a neighbour's loads queue behind host reads that
+//    take microseconds; which neighbour suffers depends on which path it shares with them.
 //  * hfkb_idle_resident: workgroups that touch no memory and only sleep for a bounded time. What a
 //    kernel on another stream loses beside them is the price of sharing the GPU at all, the floor
 //    under every figure measured beside a swap.
@@ -23,6 +27,33 @@ using hfk::kWorkgroupLanes;
 using hfk::vec16;
 
 enum Mode { kRead = 0, kWrite = 1, kCopy = 2 };
+
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// One wavefront per 256-byte unit and turn: four 64-byte scalar loads, uniform over the wavefront.
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void host_read_scalar_kernel(uint64_t host, uint64_t n_units, uint32_t* out) {
+    typedef const __attribute__((address_space(4))) u32x16* constant_units;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint64_t first = (uint64_t)blockIdx.x * WAVES + wave, stride = (uint64_t)gridDim.x * WAVES;
+    uint32_t acc = 0;
+    for (uint64_t u = first; u < n_units; u += stride) {
+        constant_units p = (constant_units)(host + u * 256);
+        const u32x16 x = p[0] ^ p[1] ^ p[2] ^ p[3];
+        acc ^= x[0] ^ x[5] ^ x[10] ^ x[15];
+    }
+    if ((threadIdx.x & 63u) == 0) out[first] = acc;   // an ordinary vector store
+}
+
+__global__ __launch_bounds__(256) void host_read_vector_kernel(const u32x4* host, uint64_t n_vec, uint32_t* out) {
+    uint32_t acc = 0;
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n_vec; i += (uint64_t)gridDim.x * 256) {
+        const u32x4 v = __builtin_nontemporal_load(host + i);
+        acc ^= v[0] ^ v[3];
+    }
+    out[blockIdx.x * 256 + threadIdx.x] = acc;
+}
 
 __global__ void idle_resident_kernel(uint64_t ticks) {
     const uint64_t t0 = wall_clock64();
@@ -103,6 +134,23 @@ __attribute__((visibility("default"))) int hfkb_memcpy_block_loop(
         }
     }
     return 0;
+}
+
+// Reads `bytes` (a multiple of 256) of device-mapped pinned host memory and leaves one checksum word
+// per wavefront (scalar path: workgroups of 8 wavefronts) or per lane (vector path) in `out`, which
+// must hold workgroups * 256 words.
+__attribute__((visibility("default"))) int hfkb_host_read(int scalar_path, const void* host_mapped, uint64_t bytes,
+                                                          uint32_t workgroups, uint32_t* out, void* stream) {
+    if (host_mapped == nullptr || out == nullptr || workgroups == 0 || (bytes & 255u) != 0) return -1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (scalar_path) {
+        hipLaunchKernelGGL(host_read_scalar_kernel<8>, dim3(workgroups), dim3(512), 0, s, (uint64_t)(uintptr_t)host_mapped,
+                           bytes / 256, out);
+    } else {
+        hipLaunchKernelGGL(host_read_vector_kernel, dim3(workgroups), dim3(256), 0, s,
+                           static_cast<const u32x4*>(host_mapped), bytes / 16, out);
+    }
+    return (int)hipGetLastError();
 }
 
 // `workgroups` x `lanes` that sleep until `ticks` of the 100 MHz counter have passed (at most a few
