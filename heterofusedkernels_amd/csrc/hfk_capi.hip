@@ -199,21 +199,15 @@ std::atomic<int> g_link_mbps_override{-1};
 // (52.7-52.8 GB/s).
 std::atomic<int> g_paced_workgroups{6};
 std::atomic<int> g_paced_unroll{4};
-constexpr uint32_t kBesidePacedWorkgroups = 12;  // toward the host, beside compute (the lower pace leaves the margin)
-constexpr uint32_t kFromHostWorkgroups = 40;     // from the host, throughput mode
-constexpr uint32_t kBesideFromHostWorkgroups = 24;
-constexpr uint32_t kBesideWorkgroups = 8;        // HFK_SWAP_BESIDE_COMPUTE with no host side named: 8 x 4, unpaced
-constexpr int kBesideUnnamedUnroll = 4;
-constexpr int kFineUnroll = 1;                   // one vector per lane: swaps from the host, and toward it beside compute
 // Share of the link's raw rate offered to host writes when pacing. 256-byte transaction payloads
 // cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured, reached only by a paced grid); from 0.92
 // on throughput collapses to 0.84 and the neighbours' slowdown doubles. The closer to the cap, the
-// longer the fabric's queues: a GEMM beside the 12 x 1 swap runs 1.64x slower at 0.84, 1.93x at 0.88,
-// 2.2x at 0.90 (1.55-1.6x is what any resident kernel costs this GEMM).
-constexpr double kPaceShareOfLink = 0.84;
-// Share offered by a throughput-mode swap-out: the cap itself (HFK_KNOB_THROUGHPUT_PACE_PERMILLE, default 0.90).
+// longer the fabric's queues: a GEMM beside the 12 x 1 swap runs 1.64x slower at 0.84
+// (hfk::kBesidePaceShareOfLink), 1.93x at 0.88, 2.2x at 0.90 (1.5-1.6x is what any resident kernel
+// costs this GEMM).
 double throughput_share_of_link() { return g_throughput_pace_permille.load(std::memory_order_relaxed) / 1000.0; }
-constexpr uint64_t kPaceFromBytes = 64ull << 20;
+using hfk::kPaceFromBytes;
+constexpr double kPaceShareOfLink = hfk::kBesidePaceShareOfLink;
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
@@ -520,44 +514,26 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
 constexpr uint32_t kSwapFlagMask = HFK_SWAP_DST_HOST | HFK_SWAP_SRC_HOST | HFK_SWAP_BESIDE_COMPUTE;
 
 int launch_swap(const BlockCopyArgs<int64_t>& a, uint32_t flags, uint32_t workgroups, uint64_t bytes, hipStream_t s) {
-    const bool beside = (flags & HFK_SWAP_BESIDE_COMPUTE) != 0;
-    if ((flags & HFK_SWAP_DST_HOST) != 0 && (beside || bytes >= kPaceFromBytes)) {
-        // Toward the host the link accepts the most when it is offered exactly what it can take
-        // (offering 1.5-2x its rate lowers what it accepts to 47-49 GB/s). A swap that shares the GPU
-        // offers 0.84 of the raw rate, one that owns it the payload-efficiency cap, 0.90; should the
-        // cap be lower than assumed the launch degrades to an unpaced one. A paced launch starts its
-        // workgroups staggered over one interval and ends behind its schedule, which only a long one
-        // amortises (2 MiB: 71 us paced, 51 us unpaced; 32 MiB: 52.6 against 54.5 GB/s; 64 MiB: 55.1
-        // against 55.0; 128 MiB: 55.9 against 55.5), so a short throughput-mode swap stays unpaced.
-        uint32_t pace_mbps = 0;
-        if (beside) {
-            pace_mbps = (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed);
-            if (pace_mbps == 0) pace_mbps = (uint32_t)(kPaceShareOfLink * current_link_mbps());
-        } else {
-            pace_mbps = (uint32_t)(throughput_share_of_link() * current_link_mbps());
-        }
-        if (pace_mbps != 0) {
-            if (workgroups == 0) {
-                workgroups = beside ? kBesidePacedWorkgroups : (uint32_t)g_paced_workgroups.load(std::memory_order_relaxed);
-            }
-            const int unroll = beside ? kFineUnroll : g_paced_unroll.load(std::memory_order_relaxed);
-            return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, unroll, pace_mbps);
-        }
-    }
-    if ((flags & HFK_SWAP_SRC_HOST) != 0) {
-        const uint32_t grid = beside ? kBesideFromHostWorkgroups : kFromHostWorkgroups;
-        return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups ? workgroups : grid, s, kFineUnroll);
-    }
-    if (beside) {
-        // No usable pace (no host side named, or the link's rate is unknown): the small unpaced grid
-        // (49.8 GB/s toward the host: between the link rate and twice it, offering more gets less accepted).
-        return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups ? workgroups : kBesideWorkgroups, s,
-                                                             kBesideUnnamedUnroll);
-    }
-    // Nothing known about the sides: sized for the PCIe link, which a small grid saturates
-    // (16 workgroups x 8 vectors per lane: 55.4-55.7 GB/s out, 57.0-57.4 in).
-    if (workgroups == 0) workgroups = (uint32_t)g_swap_workgroups.load(std::memory_order_relaxed);
-    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, workgroups, s, g_swap_unroll.load(std::memory_order_relaxed));
+    // Toward the host the link accepts the most when it is offered what it can take (offering 1.5-2x
+    // its rate lowers what it accepts to 47-49 GB/s). A swap that shares the GPU offers 0.84 of the raw
+    // rate, one that owns it 0.89; should the link take less than assumed the launch degrades to an
+    // unpaced one. A paced launch starts its workgroups staggered over one interval and ends behind
+    // its schedule, which only a long one amortises (2 MiB: 71 us paced, 51 us unpaced; 32 MiB: 52.6
+    // against 54.5 GB/s; 64 MiB: 55.1 against 55.0; 128 MiB: 55.9 against 55.5), so a short
+    // throughput-mode swap stays unpaced. Without a usable pace (no host side named, or the link's rate
+    // unknown) a beside-compute swap gets a small unpaced grid (49.8 GB/s toward the host), and a swap
+    // about which nothing is known the shape that saturates the link either way (16 workgroups x 8
+    // vectors per lane: 55.4-56.0 GB/s out, 57.0-57.4 in).
+    const bool wants_pace = (flags & HFK_SWAP_DST_HOST) != 0;
+    const hfk::SwapTuning tuning{(uint32_t)g_swap_workgroups.load(std::memory_order_relaxed),
+                                 g_swap_unroll.load(std::memory_order_relaxed),
+                                 (uint32_t)g_paced_workgroups.load(std::memory_order_relaxed),
+                                 g_paced_unroll.load(std::memory_order_relaxed),
+                                 (uint32_t)g_throughput_pace_permille.load(std::memory_order_relaxed),
+                                 (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed)};
+    const hfk::SwapShape shape =
+        hfk::choose_swap_shape(flags, bytes, wants_pace ? (uint32_t)current_link_mbps() : 0u, workgroups, tuning);
+    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, shape.workgroups, s, shape.unroll, shape.pace_mbps);
 }
 
 // ---- staged swap: HBM-only kernel + DMA copies ----------------------------

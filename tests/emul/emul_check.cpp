@@ -570,6 +570,49 @@ void case_transpose_table(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32
 
 }  // namespace
 
+// the launch shape of a swap, by flags, size and link rate: the rules as the header documents them
+void case_swap_shape() {
+    const SwapTuning t{16, 8, 6, 4, 890, 0};
+    const uint32_t link = 63015, out = HFK_SWAP_DST_HOST, in = HFK_SWAP_SRC_HOST, beside = HFK_SWAP_BESIDE_COMPUTE;
+    const uint64_t big = 512ull << 20, small = 2ull << 20;
+    struct { uint32_t flags; uint64_t bytes; uint32_t link; uint32_t asked; uint32_t wg; int unroll; uint32_t pace; const char* what; } rows[] = {
+        {0, big, link, 0, 16, 8, 0, "nothing known: 16 x 8 unpaced"},
+        {out, big, link, 0, 6, 4, 56083, "swap-out of 64 MiB or more: 6 x 4 paced at 0.89"},
+        {out, kPaceFromBytes, link, 0, 6, 4, 56083, "exactly 64 MiB is paced"},
+        {out, kPaceFromBytes - 1, link, 0, 16, 8, 0, "a shorter swap-out stays unpaced"},
+        {out, small, link, 0, 16, 8, 0, "a 2 MiB swap-out stays unpaced"},
+        {out, big, 0, 0, 16, 8, 0, "link rate unknown: unpaced"},
+        {out | beside, small, link, 0, 12, 1, 52932, "beside compute: 12 x 1 paced at 0.84 whatever the size"},
+        {out | beside, big, 0, 0, 8, 4, 0, "beside compute, link unknown: 8 x 4 unpaced"},
+        {beside, big, link, 0, 8, 4, 0, "beside compute, no side named: 8 x 4 unpaced"},
+        {in, big, link, 0, 40, 1, 0, "swap-in: 40 x 1"},
+        {in | beside, big, link, 0, 24, 1, 0, "swap-in beside compute: 24 x 1"},
+        {in | out, big, link, 0, 6, 4, 56083, "both sides host memory: the paced shape wins"},
+        {out, big, link, 20, 20, 4, 56083, "the caller's grid bound is kept"},
+        {in, big, link, 7, 7, 1, 0, "the caller's grid bound is kept (swap-in)"},
+        {0, big, link, 300, 300, 8, 0, "the caller's grid bound is kept (no flags)"},
+    };
+    for (const auto& r : rows) {
+        const SwapShape got = choose_swap_shape(r.flags, r.bytes, r.link, r.asked, t);
+        ++g_cases;
+        if (got.workgroups != r.wg || got.unroll != r.unroll || got.pace_mbps != r.pace) {
+            ++g_failures;
+            std::printf("swap shape: %s: got %u x %d paced %u, want %u x %d paced %u\n", r.what, got.workgroups, got.unroll,
+                        got.pace_mbps, r.wg, r.unroll, r.pace);
+        }
+    }
+    SwapTuning forced = t;
+    forced.beside_pace_mbps = 1;      // an explicit pace (the test of the bounded wait uses 1 MB/s)
+    const SwapShape s1 = choose_swap_shape(out | beside, small, 0, 0, forced);
+    ++g_cases;
+    if (s1.workgroups != 12 || s1.unroll != 1 || s1.pace_mbps != 1) { ++g_failures; std::printf("swap shape: explicit pace\n"); }
+    forced = t;
+    forced.throughput_pace_permille = 0;   // pacing switched off
+    const SwapShape s2 = choose_swap_shape(out, big, link, 0, forced);
+    ++g_cases;
+    if (s2.workgroups != 16 || s2.unroll != 8 || s2.pace_mbps != 0) { ++g_failures; std::printf("swap shape: pace 0\n"); }
+}
+
 // the PCIe link-rate parser on the strings sysfs shows
 void case_link_rate() {
     struct { const char* speed; const char* width; int want; } rows[] = {
@@ -595,6 +638,7 @@ void case_link_rate() {
 
 int main() {
     case_link_rate();
+    case_swap_shape();
     // swap: aligned fast path, every unroll, grid smaller and larger than the work
     for (int unroll : {1, 2, 4, 8, 16})
         for (uint32_t grid : {1u, 7u, 4096u}) {
