@@ -232,6 +232,33 @@ int current_cu_count(int* out) {
     return 0;
 }
 
+// Ticks per second of the counter the pacer reads (wall_clock64): 100 MHz on MI355X; asked of the
+// runtime once per device rather than assumed, and assumed where the runtime does not say.
+std::atomic<int> g_wall_clock_khz[kMaxDevices];
+
+double pacer_ticks_per_second() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return 1e8;
+    }
+    int khz = g_wall_clock_khz[dev].load(std::memory_order_relaxed);
+    if (khz == 0) {
+        if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || khz <= 0) {
+            (void)hipGetLastError();
+            khz = 100000;
+        }
+        g_wall_clock_khz[dev].store(khz, std::memory_order_relaxed);
+    }
+    return khz * 1e3;
+}
+
+// The pacer's interval for work items of `item_bytes` on `grid` workgroups at `pace_mbps`, in 1/256 ticks.
+uint32_t pace_interval_q8(double item_bytes, uint32_t grid, uint32_t pace_mbps) {
+    const double q8 = item_bytes * grid / ((double)pace_mbps * 1e6) * pacer_ticks_per_second() * 256.0 + 0.5;
+    return q8 < 4294967295.0 ? (uint32_t)q8 : 0xffffffffu;   // absurdly low rates: the wait's spin limit rules
+}
+
 int pick_grid(uint32_t n_work, uint32_t workgroups, uint32_t* grid) {
     uint32_t cap = workgroups;
     if (cap == 0) {
@@ -351,10 +378,8 @@ int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, 
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
     if (pace_mbps != 0) {
-        // bytes per work item (average over a block) * workgroups / rate, in 1/256 ticks of 10 ns
-        const double item_bytes = (double)a.block_bytes / a.chunks_per_block;
-        const double q8 = item_bytes * grid / ((double)pace_mbps * 1e6) * 1e8 * 256.0 + 0.5;
-        a.pace_q8 = q8 < 4294967295.0 ? (uint32_t)q8 : 0xffffffffu;   // absurdly low rates: the wait's spin limit rules
+        // bytes per work item (average over a block) * workgroups / rate
+        a.pace_q8 = pace_interval_q8((double)a.block_bytes / a.chunks_per_block, grid, pace_mbps);
     }
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
     // HBM-bound launches may ask for LDS they never touch: it bounds how many workgroups a compute
@@ -835,9 +860,7 @@ int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move*
             pace_mbps = (uint32_t)(throughput_share_of_link() * current_link_mbps());
         }
         if (pace_mbps != 0) {
-            const double item_bytes = (double)block_bytes / a.first.chunks_per_block;
-            const double q8 = item_bytes * grid / ((double)pace_mbps * 1e6) * 1e8 * 256.0 + 0.5;
-            a.pace_q8 = q8 < 4294967295.0 ? (uint32_t)q8 : 0xffffffffu;
+            a.pace_q8 = pace_interval_q8((double)block_bytes / a.first.chunks_per_block, grid, pace_mbps);
             }
     }
     const int nt = g_nontemporal.load(std::memory_order_relaxed);
