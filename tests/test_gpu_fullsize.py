@@ -175,9 +175,10 @@ def test_config4_mla_round_trip_full(named):
 
 def test_config5_fp8_fragmented_full():
     cfg = W.C5_FP8_FRAGMENTED
-    host_blocks = 4096
-    _need(4, 13)
-    announce("config 5 full: 32 layers x {K,V} [8192,16,8,128] fp8, 4096 fragmented ids: gather + swap-out")
+    host_blocks = 8192
+    _need(8, 17)
+    announce("config 5 full: 32 layers x {K,V} [8192,16,8,128] fp8, 4096 fragmented ids: gather + swap-out, then the "
+             "run-splitting swap over fragmented host slots, out and back")
     planes, dev_bytes = _device_cache(cfg, cfg.dev_blocks)
     ids = W.fragmented_ids(cfg.dev_blocks, cfg.n_blocks)
     ids_dev = ids.to(DEV)
@@ -194,7 +195,8 @@ def test_config5_fp8_fragmented_full():
          dst_blocks=host_blocks, flags=capi.SWAP_DST_HOST)
     torch.cuda.synchronize()
     for p in range(cfg.planes):
-        assert torch.equal(host[p], prefill[p].cpu()), "plane %d swap-out" % p
+        assert torch.equal(host[p][:cfg.n_blocks], prefill[p].cpu()), "plane %d swap-out" % p
+        assert int(host[p][cfg.n_blocks:].max()) == 0, "plane %d: swap-out wrote outside its slots" % p
     sel = _oracle_planes(cfg.planes)
     zeros = torch.zeros(host_blocks, cfg.block_bytes, dtype=torch.uint8)
     _check_against_oracle([host[p] for p in sel], [zeros] * len(sel), [dev_bytes[p].cpu() for p in sel], pairs, sel,
@@ -203,6 +205,44 @@ def test_config5_fp8_fragmented_full():
     for p in sel:                                                        # the gather against the oracle as well
         assert np.array_equal(prefill[p].cpu().numpy(), O.c_gather_rows(dev_bytes[p].cpu().numpy(), ids.numpy())), \
             "plane %d gather differs from the oracle" % p
+
+    # The same fragmented device blocks onto fragmented HOST slots through the mover that chooses per run of host
+    # slots (long runs: staging + copy engines; the rest: the small paced kernel), 4 GiB out and back.
+    host_ids = W.fragmented_ids(host_blocks, cfg.n_blocks, seed=11)
+    for h in host:
+        h.zero_()
+    n, bb = cfg.n_blocks, cfg.block_bytes
+    staging = torch.empty(cfg.planes * n * bb, dtype=torch.uint8, device=DEV)
+    host_addrs = (ctypes.c_void_p * cfg.planes)(*[h.data_ptr() for h in host])
+    host_np = host_ids.numpy().astype(np.int64)
+    dtab, htab = ptr_table(planes), host_ptr_table(host)
+    src_before = {p: dev_bytes[p].cpu() for p in sel}
+    out_pairs = W.pairs_tensor(ids, host_ids)                            # rows = (device block, host slot)
+    capi.check(capi.swap_blocks_auto(dtab.data_ptr(), htab.data_ptr(), host_addrs, out_pairs.to(DEV).data_ptr(),
+                                     host_np.ctypes.data, cfg.planes, n, bb, bb, bb, cfg.dev_blocks, host_blocks,
+                                     staging.data_ptr(), staging.numel(), True, 0, capi.SWAP_BESIDE_COMPUTE,
+                                     stream_handle()), "hfk_swap_blocks_auto (out)")
+    torch.cuda.synchronize()
+    untouched = torch.ones(host_blocks, dtype=torch.bool)
+    untouched[host_ids] = False
+    for p in range(cfg.planes):
+        assert torch.equal(host[p].index_select(0, host_ids), prefill[p].cpu()), "plane %d run-splitting swap-out" % p
+        assert int(host[p][untouched].max()) == 0, "plane %d: run-splitting swap-out wrote outside its slots" % p
+    _check_against_oracle([host[p] for p in sel], [torch.zeros(host_blocks, bb, dtype=torch.uint8)] * len(sel),
+                          [src_before[p] for p in sel], out_pairs, sel, "config 5 run-splitting swap-out")
+    # ... and back into other device blocks of the same set
+    back = torch.roll(ids, 7)
+    in_pairs = W.pairs_tensor(host_ids, back)                            # rows = (host slot, device block)
+    capi.check(capi.swap_blocks_auto(dtab.data_ptr(), htab.data_ptr(), host_addrs, in_pairs.to(DEV).data_ptr(),
+                                     host_np.ctypes.data, cfg.planes, n, bb, bb, bb, cfg.dev_blocks, host_blocks,
+                                     staging.data_ptr(), staging.numel(), False, 0, 0, stream_handle()),
+               "hfk_swap_blocks_auto (in)")
+    torch.cuda.synchronize()
+    back_dev = back.to(DEV)
+    for p in range(cfg.planes):
+        assert torch.equal(dev_bytes[p].index_select(0, back_dev), prefill[p]), "plane %d run-splitting swap-in" % p
+    _check_against_oracle([dev_bytes[p].cpu() for p in sel], [src_before[p] for p in sel], [host[p] for p in sel],
+                          W.pairs_tensor(host_ids, back), sel, "config 5 run-splitting swap-in")
 
 
 # ---- configuration 2: one pair of caches shared by every way of launching the same swap. Kept last in
