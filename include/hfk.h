@@ -387,8 +387,8 @@ HFK_API int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_pl
  * Same reference anchors as hfk_gather_rows; the plane loop is additive.
  *   flags  0 = source planes in device memory (grid of one workgroup per chunk, HBM-bound).
  *          HFK_SWAP_SRC_HOST = the source planes are host memory: the gather is then a swap-in with
- *          consecutive destinations and gets that launch shape (16 workgroups); with
- *          HFK_SWAP_BESIDE_COMPUTE as well, the 8-16 workgroup shape. The result never depends on flags.
+ *          consecutive destinations and gets that launch shape (40 workgroups of one vector per
+ *          lane); with HFK_SWAP_BESIDE_COMPUTE as well, 24. The result never depends on flags.
  */
 HFK_API int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs,
                       const int64_t* ids, uint32_t n_planes, uint64_t n_ids,
