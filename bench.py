@@ -715,6 +715,16 @@ def section_cpu_baseline(b, w):
             O.torch_gather_rows(s, w.src_ids)
         gpasses += 1
     cpu_gather_gbps = gpasses * sample_planes * n * bb / (time.perf_counter() - t1) / 1e9
+    # the C restatement of the same swap (one thread, memcpy per block), on the same planes, about 2 s of it
+    src_np = [W.as_bytes(s).numpy().reshape(-1, bb) for s in cpu_src]
+    dst_np = [W.as_bytes(d).numpy().reshape(-1, bb) for d in cpu_dst]
+    pairs_np = W.pairs_tensor(w.src_ids, w.dst_ids).numpy()
+    O.c_swap_blocks(dst_np, src_np, pairs_np)
+    cpasses, t2 = 0, time.perf_counter()
+    while time.perf_counter() - t2 < 2.0:
+        O.c_swap_blocks(dst_np, src_np, pairs_np)
+        cpasses += 1
+    c_oracle_gbps = cpasses * sample_planes * n * bb / (time.perf_counter() - t2) / 1e9
     cpu_model = ""
     try:
         with open("/proc/cpuinfo") as f:
@@ -724,14 +734,15 @@ def section_cpu_baseline(b, w):
                     break
     except OSError:
         pass
-    log("CPU baseline (torch, %d threads): swap %.2f GB/s, gather %.2f GB/s payload" %
-        (torch.get_num_threads(), cpu_gbps, cpu_gather_gbps))
+    log("CPU baseline (torch, %d threads): swap %.2f GB/s, gather %.2f GB/s payload; the C restatement on one thread: "
+        "swap %.2f GB/s" % (torch.get_num_threads(), cpu_gbps, cpu_gather_gbps, c_oracle_gbps))
     return {
         "value": cpu_gbps, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": "torch CPU dst.index_copy_(0, dst_ids, src.index_select(0, src_ids)) per plane on %d of %d "
                   "planes of the same block table (%d blocks x %d B each), %d passes in %.1fs" %
                   (sample_planes, planes, n, bb, passes, dt),
-        "gather_index_select_GBps": cpu_gather_gbps, "os_cpu_count": os.cpu_count(),
+        "gather_index_select_GBps": cpu_gather_gbps, "c_restatement_one_thread_GBps": c_oracle_gbps,
+        "os_cpu_count": os.cpu_count(),
         "affinity": len(os.sched_getaffinity(0)), "cpu_model": cpu_model,
     }
 
