@@ -421,7 +421,7 @@ def test_staged_swap_equals_direct_swap(memory, cfg, n, pattern):
     W.C5_FP8_FRAGMENTED.scaled(layers=2, dev_blocks=512, host_blocks=512, n_blocks=200),
 ], ids=lambda c: c.name)
 def test_swap_beside_compute_moves_the_same_bytes(memory, cfg):
-    """HFK_SWAP_BESIDE_COMPUTE only changes the launch shape (8-16 workgroups, paced toward the host):
+    """HFK_SWAP_BESIDE_COMPUTE only changes the launch shape (8-24 workgroups, paced toward the host):
     swap-out then swap-in with the flags == index_select / index_copy_, untouched blocks included."""
     announce("swap beside compute %s: %d planes, %d pairs, %d B blocks, link %d MB/s"
              % (cfg.name, cfg.planes, cfg.n_blocks, cfg.block_bytes, capi.get_tuning(capi.KNOB_LINK_MBPS)))
