@@ -24,6 +24,10 @@ KNOB_THROUGHPUT_PACE_PERMILLE = 9
 KNOB_HBM_LDS_BYTES = 10
 KNOB_PACED_UNROLL = 11
 KNOB_PACED_WORKGROUPS = 12
+KNOB_PACE_REPORT = 13
+KNOB_DUPLEX_PACE_PERMILLE = 14
+KNOB_TRANSFER_PACE_PERMILLE = 15
+KNOB_TRANSFER_UNROLL = 16
 SWAP_DST_HOST = 1
 SWAP_SRC_HOST = 2
 SWAP_BESIDE_COMPUTE = 4
@@ -31,6 +35,11 @@ SWAP_SRC_DEVICE = 8
 SWAP_DST_DEVICE = 16
 STATIC_STAGING_BYTES = 64 << 20
 ERR_STAGING_TOO_SMALL = -7
+
+
+class KnobValue(ctypes.Structure):
+    """struct hfk_knob_value."""
+    _fields_ = [("knob", ctypes.c_int), ("value", ctypes.c_int64)]
 
 
 class BlockMove(ctypes.Structure):
@@ -55,6 +64,8 @@ ENTRY_POINTS = (
     "hfk_gather_blocks",
     "hfk_set_tuning",
     "hfk_get_tuning",
+    "hfk_thread_tuning_begin",
+    "hfk_thread_tuning_end",
 )
 
 
@@ -116,6 +127,10 @@ def load():
     L.hfk_set_tuning.restype = ci
     L.hfk_get_tuning.argtypes = [ci]
     L.hfk_get_tuning.restype = i64
+    L.hfk_thread_tuning_begin.argtypes = [ctypes.POINTER(KnobValue), u32]
+    L.hfk_thread_tuning_begin.restype = ci
+    L.hfk_thread_tuning_end.argtypes = []
+    L.hfk_thread_tuning_end.restype = None
     _lib = L
     return L
 
@@ -203,3 +218,20 @@ def set_tuning(knob, value):
 
 def get_tuning(knob):
     return load().hfk_get_tuning(knob)
+
+
+class thread_tuning:
+    """``with capi.thread_tuning({capi.KNOB_UNROLL: 4, ...}):`` -- knob values for the calls this thread
+    makes inside the block (hfk_thread_tuning_begin / _end); the process-wide values stay as they are."""
+
+    def __init__(self, overrides):
+        self.overrides = dict(overrides)
+
+    def __enter__(self):
+        items = (KnobValue * max(1, len(self.overrides)))(*[KnobValue(k, v) for k, v in self.overrides.items()])
+        check(load().hfk_thread_tuning_begin(items, len(self.overrides)), "hfk_thread_tuning_begin")
+        return self
+
+    def __exit__(self, *exc):
+        load().hfk_thread_tuning_end()
+        return False

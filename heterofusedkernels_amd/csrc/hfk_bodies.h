@@ -60,9 +60,14 @@ struct Pacer {
     uint64_t t0;
     uint64_t due_q8;
     uint32_t pace_q8;
+    // What the schedule did to this workgroup, for callers that ask (pace report): turns taken, turns
+    // that began behind schedule (no waiting), and the largest delay behind schedule seen, in 1/256 ticks.
+    uint32_t turns;
+    uint32_t late_turns;
+    uint64_t max_late_q8;
 
     HFK_HD Pacer(uint32_t pace, uint32_t bid, uint32_t nb)
-        : t0(0), due_q8(0), pace_q8(HFK_CAN_PACE ? pace : 0) {
+        : t0(0), due_q8(0), pace_q8(HFK_CAN_PACE ? pace : 0), turns(0), late_turns(0), max_late_q8(0) {
         if (pace_q8 != 0) {
             t0 = HFK_TICKS_100MHZ();
             due_q8 = (uint64_t)pace_q8 * bid / nb;  // workgroups take turns within an interval
@@ -72,10 +77,34 @@ struct Pacer {
     // Call before each work item. The counter always advances; the spin limit ends the wait regardless.
     HFK_HD void wait_turn() {
         if (pace_q8 == 0) return;
-        for (uint32_t spin = 0; spin < (1u << 16) && ((HFK_TICKS_100MHZ() - t0) << 8) < due_q8; ++spin) {
-            HFK_NAP();
+        const uint64_t now_q8 = (HFK_TICKS_100MHZ() - t0) << 8;
+        if (now_q8 >= due_q8) {
+            ++late_turns;
+            if (now_q8 - due_q8 > max_late_q8) max_late_q8 = now_q8 - due_q8;
+        } else {
+            for (uint32_t spin = 0; spin < (1u << 16) && ((HFK_TICKS_100MHZ() - t0) << 8) < due_q8; ++spin) {
+                HFK_NAP();
+            }
         }
+        ++turns;
         due_q8 += pace_q8;
+    }
+
+    // Pace report: eight 64-bit words per workgroup at report + 8 * bid, written by lane 0 when the
+    // workgroup has finished: ticks it ran, ticks its schedule allotted (the time its next turn
+    // would have come), turns, turns that began late, largest delay in ticks, the interval in 1/256
+    // ticks; two words unused. A launch that holds its pace ends with ran <= allotted.
+    HFK_HD void report(uint64_t* out, uint32_t bid, uint32_t tid) const {
+        if (out == nullptr || pace_q8 == 0 || tid != 0) return;
+        HFK_GLOBAL uint64_t* row = reinterpret_cast<HFK_GLOBAL uint64_t*>(reinterpret_cast<uint64_t>(out)) + 8 * (uint64_t)bid;
+        row[0] = HFK_TICKS_100MHZ() - t0;
+        row[1] = due_q8 >> 8;
+        row[2] = turns;
+        row[3] = late_turns;
+        row[4] = max_late_q8 >> 8;
+        row[5] = pace_q8;
+        row[6] = 0;
+        row[7] = 0;
     }
 };
 
@@ -168,6 +197,7 @@ struct BlockCopyArgs {
     uint32_t run_mode;
     uint32_t run_min;            // a run is "long" from this many consecutive ids on
     const int64_t* run_ids;      // entry j at run_ids[j * id_stride]
+    uint64_t* pace_report;       // null, or where each workgroup of a paced launch leaves Pacer::report
 };
 
 // Which pairs of a block table a launch moves, when the table is split by run length: pair j belongs to
@@ -379,6 +409,7 @@ HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t 
         }
         w += nb;
     }
+    pacer.report(a.pace_report, bid, tid);
 }
 
 // ---------------------------------------------------------------------------
@@ -531,6 +562,7 @@ struct TransposeArgs {
     uint32_t row_units;          // D * elem_bytes / sizeof(V)
     uint32_t total_units;        // T * L * H * row_units, per block
     uint32_t n_work;             // n_pairs * chunks_per_block
+    uint32_t pace_q8;            // see Pacer; 0 = unpaced
 };
 
 // Where the body finds layer l's address. The layer differs from lane to lane (a 128-byte row is 8
@@ -562,6 +594,7 @@ template <typename V, int UNROLL, int NT, bool TO_PACKED, typename LayerTable>
 HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid, const LayerTable& layer_address) {
     constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
     const uint32_t LH = a.L * a.H;
+    Pacer pacer(a.pace_q8, bid, nb);
 
     for (uint64_t w64 = bid; w64 < a.n_work; w64 += nb) {
         const uint32_t w = (uint32_t)w64;
@@ -572,6 +605,7 @@ HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, ui
         if (pb >= a.packed_limit || db >= a.layered_limit) {
             continue;
         }
+        pacer.wait_turn();
         const uint64_t packed_addr = a.packed + pb * a.packed_stride;
         const uint64_t layered_off = db * a.layered_stride;
         const uint64_t g0 = (uint64_t)chunk * kChunkUnits + tid;

@@ -136,11 +136,66 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
 //    defaults to 16. For the same reason the duplex swap defaults to 32 workgroups (98.2 GB/s
 //    summed against 99.1 at 128, neighbours 1.1-1.6x slower instead of 2.8-2.9x), a block-table
 //    transfer out of host memory to 24 and one into host memory to 48 (see launch_transpose).
-std::atomic<int> g_unroll{1};
-std::atomic<int> g_nontemporal{3};
-std::atomic<int> g_wg_per_cu{65536};
-std::atomic<int> g_swap_workgroups{16};
-constexpr uint32_t kDuplexWorkgroups = 32;
+//
+// Every knob has a process-wide value (hfk_set_tuning) and, per thread, an optional override that
+// lasts from hfk_thread_tuning_begin to hfk_thread_tuning_end: a caller that wants a launch shape
+// of its own for a few calls changes nothing another thread can see.
+constexpr int kKnobCount = 17;
+std::atomic<int64_t> g_knob[kKnobCount] = {
+    1,       // HFK_KNOB_UNROLL
+    3,       // HFK_KNOB_NONTEMPORAL
+    65536,   // HFK_KNOB_WORKGROUPS_PER_CU
+    16,      // HFK_KNOB_SWAP_WORKGROUPS
+    1,       // HFK_KNOB_DUPLEX_UNROLL
+    8,       // HFK_KNOB_SWAP_UNROLL
+    0,       // HFK_KNOB_SWAP_PACE_MBPS
+    -1,      // HFK_KNOB_LINK_MBPS
+    32,      // HFK_KNOB_DUPLEX_WORKGROUPS
+    0,       // HFK_KNOB_THROUGHPUT_PACE_PERMILLE
+    0,       // HFK_KNOB_HBM_LDS_BYTES
+    4,       // HFK_KNOB_PACED_UNROLL
+    6,       // HFK_KNOB_PACED_WORKGROUPS
+    0,       // HFK_KNOB_PACE_REPORT
+    890,     // HFK_KNOB_DUPLEX_PACE_PERMILLE
+    0,       // HFK_KNOB_TRANSFER_PACE_PERMILLE
+    8,       // HFK_KNOB_TRANSFER_UNROLL
+};
+
+struct ThreadTuning {
+    uint32_t mask = 0;                 // bit k: this thread overrides knob k
+    int64_t value[kKnobCount] = {};
+};
+thread_local ThreadTuning t_tuning;
+
+int64_t knob_value(int k) {
+    return ((t_tuning.mask >> k) & 1u) != 0 ? t_tuning.value[k] : g_knob[k].load(std::memory_order_relaxed);
+}
+
+bool is_unroll(int64_t v) { return v == 1 || v == 2 || v == 4 || v == 8 || v == 16; }
+
+bool knob_value_valid(int k, int64_t v) {
+    switch (k) {
+        case HFK_KNOB_UNROLL:
+        case HFK_KNOB_DUPLEX_UNROLL:
+        case HFK_KNOB_SWAP_UNROLL:
+        case HFK_KNOB_PACED_UNROLL: return is_unroll(v);
+        case HFK_KNOB_NONTEMPORAL: return v >= 0 && v <= 3;
+        case HFK_KNOB_WORKGROUPS_PER_CU: return v >= 1 && v <= 65536;
+        case HFK_KNOB_SWAP_WORKGROUPS:
+        case HFK_KNOB_DUPLEX_WORKGROUPS:
+        case HFK_KNOB_PACED_WORKGROUPS: return v >= 1 && v <= (1 << 20);
+        case HFK_KNOB_SWAP_PACE_MBPS: return v >= 0 && v <= 1000000;
+        case HFK_KNOB_LINK_MBPS: return v >= -1 && v <= 1000000;
+        case HFK_KNOB_THROUGHPUT_PACE_PERMILLE: return v >= 0 && v <= 2000;
+        case HFK_KNOB_HBM_LDS_BYTES: return v >= 0 && v <= 65536;
+        case HFK_KNOB_PACE_REPORT: return (v & 7) == 0;   // an address of 64-bit words, or 0
+        case HFK_KNOB_DUPLEX_PACE_PERMILLE:
+        case HFK_KNOB_TRANSFER_PACE_PERMILLE: return v >= 0 && v <= 2000;
+        case HFK_KNOB_TRANSFER_UNROLL: return v == 2 || v == 8;
+        default: return false;
+    }
+}
+
 constexpr uint32_t kBesideDuplexWorkgroups = 16;
 constexpr int kBesideDuplexUnroll = 2;
 constexpr uint32_t kBesideTransferWorkgroups = 16;
@@ -153,17 +208,10 @@ constexpr uint64_t kAskTableSideBytes = 64ull << 10;
 // The duplex swap wants little in flight per workgroup: one vector per lane and direction
 // (unroll 8 loses 6 %). 32 workgroups reach 98.1-98.4 GB/s summed for 16, 32 and 72 KiB
 // blocks; 40-64 dip to 89-94, 96-192 are a flat 98-99.
-std::atomic<int> g_duplex_unroll{1};
-std::atomic<int> g_duplex_workgroups{(int)kDuplexWorkgroups};
-std::atomic<int> g_hbm_lds_bytes{0};
 // Share of the link's raw rate, in thousandths, that a long throughput-mode launch offers toward the
 // host (0 = unpaced).
-std::atomic<int> g_throughput_pace_permille{890};
-std::atomic<int> g_swap_unroll{8};
 // Explicit offered rate of a swap that runs beside compute, MB/s; 0 = derive it from the link.
-std::atomic<int> g_swap_pace_mbps{0};
 // PCIe link rate override, MB/s; -1 = read each device's link from sysfs on first use.
-std::atomic<int> g_link_mbps_override{-1};
 
 // Launch shapes of a swap whose host side the caller has named. What a host-facing launch keeps in
 // flight beyond the link's bandwidth-delay product (about 64 KiB toward the host, 128 KiB from it)
@@ -197,16 +245,13 @@ std::atomic<int> g_link_mbps_override{-1};
 // 1.35x / 1.32x / 2.5x against 1.07x / 1.21x / 2.3x for 16 x 1; a swap that should be gentle says so
 // (HFK_SWAP_BESIDE_COMPUTE) and gets the fine shape at 0.84, which it holds on every pattern
 // (52.7-52.8 GB/s).
-std::atomic<int> g_paced_workgroups{6};
-std::atomic<int> g_paced_unroll{4};
 // Share of the link's raw rate offered to host writes when pacing. 256-byte transaction payloads
 // cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured, reached only by a paced grid); from 0.92
 // on throughput collapses to 0.84 and the neighbours' slowdown doubles. The closer to the cap, the
 // longer the fabric's queues: a GEMM beside the 12 x 1 swap runs 1.64x slower at 0.84
 // (hfk::kBesidePaceShareOfLink), 1.93x at 0.88, 2.2x at 0.90 (1.5-1.6x is what any resident kernel
 // costs this GEMM).
-double throughput_share_of_link() { return g_throughput_pace_permille.load(std::memory_order_relaxed) / 1000.0; }
-using hfk::kPaceFromBytes;
+using hfk::kLongSwapBytes;
 constexpr double kPaceShareOfLink = hfk::kBesidePaceShareOfLink;
 
 constexpr int kMaxDevices = 64;
@@ -265,7 +310,7 @@ int pick_grid(uint32_t n_work, uint32_t workgroups, uint32_t* grid) {
         int cus = 0;
         int rc = current_cu_count(&cus);
         if (rc != 0) return rc;
-        cap = (uint32_t)cus * (uint32_t)g_wg_per_cu.load(std::memory_order_relaxed);
+        cap = (uint32_t)cus * (uint32_t)knob_value(HFK_KNOB_WORKGROUPS_PER_CU);
     }
     *grid = n_work < cap ? n_work : cap;
     return 0;
@@ -313,8 +358,8 @@ int read_link_mbps(int dev) {
 }
 
 int current_link_mbps() {
-    const int forced = g_link_mbps_override.load(std::memory_order_relaxed);
-    if (forced >= 0) return forced;
+    const int64_t forced = knob_value(HFK_KNOB_LINK_MBPS);
+    if (forced >= 0) return (int)forced;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) {
         (void)hipGetLastError();
@@ -368,9 +413,9 @@ void launch_block_copy_nt(const BlockCopyArgs<IdT>& a, uint32_t grid, int nt, ui
 
 template <Role ROLE, typename IdT>
 int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, int preferred_unroll = 0,
-                      uint32_t pace_mbps = 0) {
+                      uint32_t pace_mbps = 0, bool plain_stores = false) {
     int unroll = 1;
-    if (preferred_unroll == 0) preferred_unroll = g_unroll.load(std::memory_order_relaxed);
+    if (preferred_unroll == 0) preferred_unroll = (int)knob_value(HFK_KNOB_UNROLL);
     // Everything but the swap runs one workgroup per chunk and wants whole chunks.
     int rc = hfk::plan_block_copy<IdT>(a, preferred_unroll, &unroll, ROLE != Role::kSwapBlocks);
     if (rc != 0) return rc;
@@ -380,11 +425,12 @@ int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, 
     if (pace_mbps != 0) {
         // bytes per work item (average over a block) * workgroups / rate
         a.pace_q8 = pace_interval_q8((double)a.block_bytes / a.chunks_per_block, grid, pace_mbps);
+        a.pace_report = reinterpret_cast<uint64_t*>((uintptr_t)knob_value(HFK_KNOB_PACE_REPORT));
     }
-    const int nt = g_nontemporal.load(std::memory_order_relaxed);
+    const int nt = (int)knob_value(HFK_KNOB_NONTEMPORAL) & (plain_stores ? 1 : 3);
     // HBM-bound launches may ask for LDS they never touch: it bounds how many workgroups a compute
     // unit holds at a time (HFK_KNOB_HBM_LDS_BYTES).
-    const uint32_t lds = ROLE == Role::kSwapBlocks ? 0u : (uint32_t)g_hbm_lds_bytes.load(std::memory_order_relaxed);
+    const uint32_t lds = ROLE == Role::kSwapBlocks ? 0u : (uint32_t)knob_value(HFK_KNOB_HBM_LDS_BYTES);
     switch (unroll) {
         case 1: launch_block_copy_nt<ROLE, IdT, 1>(a, grid, nt, lds, s); break;
         case 2: launch_block_copy_nt<ROLE, IdT, 2>(a, grid, nt, lds, s); break;
@@ -428,7 +474,7 @@ int launch_flat_gather(uint64_t table, uint64_t dst, const IdT* ids, uint64_t n_
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
-    const int nt = g_nontemporal.load(std::memory_order_relaxed);
+    const int nt = (int)knob_value(HFK_KNOB_NONTEMPORAL);
     if (p.unit == 16u) {
         if (p.index32) launch_flat_gather_v<vec16, IdT, uint32_t>(a, grid, nt, unroll, s);
         else launch_flat_gather_v<vec16, IdT, uint64_t>(a, grid, nt, unroll, s);
@@ -457,14 +503,19 @@ int gather_rows_typed(const void* table, void* dst, const IdT* ids, uint64_t n_i
 }
 
 // ---- transpose ------------------------------------------------------------
+template <typename V, int U, int NT>
+void launch_transpose_nt(const TransposeArgs& a, uint32_t grid, bool to_packed, hipStream_t s) {
+    if (to_packed) hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, NT>), dim3(grid), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((transpose_kernel<V, U, NT>), dim3(grid), dim3(256), 0, s, a);
+}
+
 template <typename V, int U>
 void launch_transpose_u(const TransposeArgs& a, uint32_t grid, int nt, bool to_packed, hipStream_t s) {
-    if (to_packed) {
-        if (nt & 3) hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, 3>), dim3(grid), dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, 0>), dim3(grid), dim3(256), 0, s, a);
-    } else {
-        if (nt & 3) hipLaunchKernelGGL((transpose_kernel<V, U, 3>), dim3(grid), dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((transpose_kernel<V, U, 0>), dim3(grid), dim3(256), 0, s, a);
+    switch (nt & 3) {
+        case 0: launch_transpose_nt<V, U, 0>(a, grid, to_packed, s); break;
+        case 1: launch_transpose_nt<V, U, 1>(a, grid, to_packed, s); break;
+        case 2: launch_transpose_nt<V, U, 2>(a, grid, to_packed, s); break;
+        default: launch_transpose_nt<V, U, 3>(a, grid, to_packed, s); break;
     }
 }
 
@@ -509,7 +560,7 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     // eight-head shapes and loses up to 3.5 on the one-head shapes, whose 128-byte rows come from 64
     // different layer caches per chunk and fall behind any schedule.)
     const int side = packed_side == kAskRuntime ? memory_side(packed) : packed_side;
-    const int unroll = to_packed && side != 0 ? hfk::kTransposeUnrollToHost : hfk::kTransposeUnroll;
+    const int unroll = to_packed && side != 0 ? (int)knob_value(HFK_KNOB_TRANSFER_UNROLL) : hfk::kTransposeUnroll;
     TransposeArgs a;
     uint32_t unit = 16;
     int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, packed, pairs, n_pairs, packed_stride, layered_stride,
@@ -527,7 +578,11 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
-    const int nt = g_nontemporal.load(std::memory_order_relaxed);
+    if (to_packed && side != 0 && knob_value(HFK_KNOB_TRANSFER_PACE_PERMILLE) != 0) {
+        const uint32_t pace_mbps = (uint32_t)(knob_value(HFK_KNOB_TRANSFER_PACE_PERMILLE) / 1000.0 * current_link_mbps());
+        if (pace_mbps != 0) a.pace_q8 = pace_interval_q8((double)a.total_units * unit / a.chunks_per_block, grid, pace_mbps);
+    }
+    const int nt = (int)knob_value(HFK_KNOB_NONTEMPORAL);
     if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, to_packed, unroll, s);
     else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, to_packed, unroll, s);
     else launch_transpose_v<uint8_t>(a, grid, nt, to_packed, unroll, s);
@@ -550,15 +605,16 @@ int launch_swap(const BlockCopyArgs<int64_t>& a, uint32_t flags, uint32_t workgr
     // about which nothing is known the shape that saturates the link either way (16 workgroups x 8
     // vectors per lane: 55.4-56.0 GB/s out, 57.0-57.4 in).
     const bool wants_pace = (flags & HFK_SWAP_DST_HOST) != 0;
-    const hfk::SwapTuning tuning{(uint32_t)g_swap_workgroups.load(std::memory_order_relaxed),
-                                 g_swap_unroll.load(std::memory_order_relaxed),
-                                 (uint32_t)g_paced_workgroups.load(std::memory_order_relaxed),
-                                 g_paced_unroll.load(std::memory_order_relaxed),
-                                 (uint32_t)g_throughput_pace_permille.load(std::memory_order_relaxed),
-                                 (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed)};
+    const hfk::SwapTuning tuning{(uint32_t)knob_value(HFK_KNOB_SWAP_WORKGROUPS),
+                                 (int)knob_value(HFK_KNOB_SWAP_UNROLL),
+                                 (uint32_t)knob_value(HFK_KNOB_PACED_WORKGROUPS),
+                                 (int)knob_value(HFK_KNOB_PACED_UNROLL),
+                                 (uint32_t)knob_value(HFK_KNOB_THROUGHPUT_PACE_PERMILLE),
+                                 (uint32_t)knob_value(HFK_KNOB_SWAP_PACE_MBPS)};
     const hfk::SwapShape shape =
         hfk::choose_swap_shape(flags, bytes, wants_pace ? (uint32_t)current_link_mbps() : 0u, workgroups, tuning);
-    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, shape.workgroups, s, shape.unroll, shape.pace_mbps);
+    return launch_block_copy<Role::kSwapBlocks, int64_t>(a, shape.workgroups, s, shape.unroll, shape.pace_mbps,
+                                                         shape.plain_stores);
 }
 
 // ---- staged swap: HBM-only kernel + DMA copies ----------------------------
@@ -839,31 +895,31 @@ int hfk_swap_blocks_duplex(const hfk_block_move* out_move, const hfk_block_move*
     // Beside compute: half the workgroups, two vectors per lane and direction, paced (97-98 GB/s summed
     // on 16 workgroups where one vector per lane leaves them latency-bound at 64).
     int rc = hfk::plan_duplex(a, out_move, in_move, n_planes, block_bytes,
-                              beside ? kBesideDuplexUnroll : g_duplex_unroll.load(std::memory_order_relaxed), &unroll);
+                              beside ? kBesideDuplexUnroll : (int)knob_value(HFK_KNOB_DUPLEX_UNROLL), &unroll);
     if (rc != 0) return rc;
     if (a.n_work == 0) return HFK_OK;
     if (workgroups == 0) {
-        workgroups = beside ? kBesideDuplexWorkgroups : (uint32_t)g_duplex_workgroups.load(std::memory_order_relaxed);
+        workgroups = beside ? kBesideDuplexWorkgroups : (uint32_t)knob_value(HFK_KNOB_DUPLEX_WORKGROUPS);
     }
     uint32_t grid = 0;
     rc = pick_grid(a.n_work, workgroups, &grid);
     if (rc != 0) return rc;
     const uint64_t out_bytes = out_move ? (uint64_t)n_planes * out_move->n_pairs * block_bytes : 0;
-    if (a.first.n_work != 0 && (beside || out_bytes >= kPaceFromBytes)) {
+    if (a.first.n_work != 0 && (beside || out_bytes >= kLongSwapBytes)) {
         // Every iteration moves one chunk toward the host (and one from it): offer the link what the
         // paced one-way swap offers it in the same mode.
         uint32_t pace_mbps = 0;
         if (beside) {
-            pace_mbps = (uint32_t)g_swap_pace_mbps.load(std::memory_order_relaxed);
+            pace_mbps = (uint32_t)knob_value(HFK_KNOB_SWAP_PACE_MBPS);
             if (pace_mbps == 0) pace_mbps = (uint32_t)(kPaceShareOfLink * current_link_mbps());
         } else {
-            pace_mbps = (uint32_t)(throughput_share_of_link() * current_link_mbps());
+            pace_mbps = (uint32_t)(knob_value(HFK_KNOB_DUPLEX_PACE_PERMILLE) / 1000.0 * current_link_mbps());
         }
         if (pace_mbps != 0) {
             a.pace_q8 = pace_interval_q8((double)block_bytes / a.first.chunks_per_block, grid, pace_mbps);
             }
     }
-    const int nt = g_nontemporal.load(std::memory_order_relaxed);
+    const int nt = (int)knob_value(HFK_KNOB_NONTEMPORAL);
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (unroll) {
         case 1: launch_duplex_nt<1>(a, grid, nt, s); break;
@@ -993,81 +1049,30 @@ int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, co
 }
 
 int hfk_set_tuning(int knob, int64_t value) {
-    switch (knob) {
-        case HFK_KNOB_UNROLL:
-            if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return HFK_ERR_BAD_KNOB;
-            g_unroll.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_NONTEMPORAL:
-            if (value < 0 || value > 3) return HFK_ERR_BAD_KNOB;
-            g_nontemporal.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_WORKGROUPS_PER_CU:
-            if (value < 1 || value > 65536) return HFK_ERR_BAD_KNOB;
-            g_wg_per_cu.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_SWAP_WORKGROUPS:
-            if (value < 1 || value > (1 << 20)) return HFK_ERR_BAD_KNOB;
-            g_swap_workgroups.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_DUPLEX_UNROLL:
-            if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return HFK_ERR_BAD_KNOB;
-            g_duplex_unroll.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_SWAP_UNROLL:
-            if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return HFK_ERR_BAD_KNOB;
-            g_swap_unroll.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_SWAP_PACE_MBPS:
-            if (value < 0 || value > 1000000) return HFK_ERR_BAD_KNOB;
-            g_swap_pace_mbps.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_LINK_MBPS:
-            if (value < -1 || value > 1000000) return HFK_ERR_BAD_KNOB;
-            g_link_mbps_override.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_DUPLEX_WORKGROUPS:
-            if (value < 1 || value > (1 << 20)) return HFK_ERR_BAD_KNOB;
-            g_duplex_workgroups.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_THROUGHPUT_PACE_PERMILLE:
-            if (value < 0 || value > 2000) return HFK_ERR_BAD_KNOB;
-            g_throughput_pace_permille.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_PACED_UNROLL:
-            if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16) return HFK_ERR_BAD_KNOB;
-            g_paced_unroll.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_PACED_WORKGROUPS:
-            if (value < 1 || value > (1 << 20)) return HFK_ERR_BAD_KNOB;
-            g_paced_workgroups.store((int)value);
-            return HFK_OK;
-        case HFK_KNOB_HBM_LDS_BYTES:
-            if (value < 0 || value > 65536) return HFK_ERR_BAD_KNOB;
-            g_hbm_lds_bytes.store((int)value);
-            return HFK_OK;
-        default:
-            return HFK_ERR_BAD_KNOB;
-    }
+    if (knob < 0 || knob >= kKnobCount || !knob_value_valid(knob, value)) return HFK_ERR_BAD_KNOB;
+    g_knob[knob].store(value, std::memory_order_relaxed);
+    return HFK_OK;
 }
 
 int64_t hfk_get_tuning(int knob) {
-    switch (knob) {
-        case HFK_KNOB_UNROLL: return g_unroll.load();
-        case HFK_KNOB_NONTEMPORAL: return g_nontemporal.load();
-        case HFK_KNOB_WORKGROUPS_PER_CU: return g_wg_per_cu.load();
-        case HFK_KNOB_SWAP_WORKGROUPS: return g_swap_workgroups.load();
-        case HFK_KNOB_DUPLEX_UNROLL: return g_duplex_unroll.load();
-        case HFK_KNOB_SWAP_UNROLL: return g_swap_unroll.load();
-        case HFK_KNOB_SWAP_PACE_MBPS: return g_swap_pace_mbps.load();
-        case HFK_KNOB_LINK_MBPS: return current_link_mbps();
-        case HFK_KNOB_DUPLEX_WORKGROUPS: return g_duplex_workgroups.load();
-        case HFK_KNOB_THROUGHPUT_PACE_PERMILLE: return g_throughput_pace_permille.load();
-        case HFK_KNOB_HBM_LDS_BYTES: return g_hbm_lds_bytes.load();
-        case HFK_KNOB_PACED_UNROLL: return g_paced_unroll.load();
-        case HFK_KNOB_PACED_WORKGROUPS: return g_paced_workgroups.load();
-        default: return HFK_ERR_BAD_KNOB;
-    }
+    if (knob < 0 || knob >= kKnobCount) return HFK_ERR_BAD_KNOB;
+    if (knob == HFK_KNOB_LINK_MBPS) return current_link_mbps();
+    return knob_value(knob);
 }
+
+int hfk_thread_tuning_begin(const hfk_knob_value* overrides, uint32_t n) {
+    if (n != 0 && overrides == nullptr) return HFK_ERR_NULL_POINTER;
+    ThreadTuning next;
+    for (uint32_t i = 0; i < n; ++i) {
+        const int k = overrides[i].knob;
+        if (k < 0 || k >= kKnobCount || !knob_value_valid(k, overrides[i].value)) return HFK_ERR_BAD_KNOB;
+        next.mask |= 1u << k;
+        next.value[k] = overrides[i].value;
+    }
+    t_tuning = next;   // replaces whatever this thread had; nothing is kept on a rejected list
+    return HFK_OK;
+}
+
+void hfk_thread_tuning_end(void) { t_tuning = ThreadTuning{}; }
 
 }  // extern "C"

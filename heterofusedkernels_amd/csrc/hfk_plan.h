@@ -31,8 +31,11 @@ constexpr int kTransposeUnrollToHost = 8;
 // ---- launch shape of a block-table swap -------------------------------------
 // What a swap launch looks like follows from what the caller says about it (flags), how much it
 // moves, and the link's rate; the rules live here, apart from the launching code, so that a CPU
-// test can pin them. Workgroups x 16-byte vectors per lane, and the rate offered toward the host
-// (0 = unpaced). The measurements behind each shape stand beside the tunables in hfk_capi.hip.
+// test can pin them. Workgroups x 16-byte vectors per lane, the rate offered toward the host
+// (0 = unpaced), and whether the stores are plain (through the L2) or non-temporal (streamed). The
+// measurements behind each shape stand beside the tunables in hfk_capi.hip.
+constexpr uint32_t kToHostWorkgroups = 12;         // toward the host, throughput mode: 12 x 8, plain stores
+constexpr int kToHostUnroll = 8;
 constexpr uint32_t kBesidePacedWorkgroups = 12;    // toward the host, beside compute: 12 x 1 paced at 0.84
 constexpr uint32_t kFromHostWorkgroups = 40;       // from the host: 40 x 1
 constexpr uint32_t kBesideFromHostWorkgroups = 24; // from the host, beside compute: 24 x 1
@@ -40,14 +43,16 @@ constexpr uint32_t kBesideWorkgroups = 8;          // beside compute, no usable 
 constexpr int kBesideUnnamedUnroll = 4;
 constexpr int kFineUnroll = 1;
 constexpr double kBesidePaceShareOfLink = 0.84;
-constexpr uint64_t kPaceFromBytes = 64ull << 20;   // a shorter throughput-mode swap stays unpaced
+// From this size on a throughput-mode swap toward the host writes through the L2 (and a paced one,
+// if pacing is switched on, is paced); a shorter one is over before either could pay.
+constexpr uint64_t kLongSwapBytes = 64ull << 20;
 
 struct SwapTuning {              // what hfk_set_tuning can change
     uint32_t swap_workgroups;    // no side named
     int swap_unroll;
-    uint32_t paced_workgroups;   // toward a named host side, throughput mode
+    uint32_t paced_workgroups;   // toward a named host side, throughput mode, when paced
     int paced_unroll;
-    uint32_t throughput_pace_permille;
+    uint32_t throughput_pace_permille;   // 0 (default) = that swap is not paced
     uint32_t beside_pace_mbps;   // 0 = kBesidePaceShareOfLink of the link
 };
 
@@ -55,27 +60,29 @@ struct SwapShape {
     uint32_t workgroups;
     int unroll;
     uint32_t pace_mbps;
+    bool plain_stores;
 };
 
 // `workgroups` != 0 is the caller's own grid bound and is kept; `link_mbps` 0 = unknown.
 inline SwapShape choose_swap_shape(uint32_t flags, uint64_t bytes, uint32_t link_mbps, uint32_t workgroups,
                                    const SwapTuning& t) {
     const bool beside = (flags & HFK_SWAP_BESIDE_COMPUTE) != 0;
-    if ((flags & HFK_SWAP_DST_HOST) != 0 && (beside || bytes >= kPaceFromBytes)) {
+    if ((flags & HFK_SWAP_DST_HOST) != 0 && (beside || bytes >= kLongSwapBytes)) {
         uint32_t pace = 0;
         if (beside) pace = t.beside_pace_mbps != 0 ? t.beside_pace_mbps : (uint32_t)(kBesidePaceShareOfLink * link_mbps);
         else pace = (uint32_t)(t.throughput_pace_permille / 1000.0 * link_mbps);
         if (pace != 0) {
             const uint32_t grid = beside ? kBesidePacedWorkgroups : t.paced_workgroups;
-            return SwapShape{workgroups ? workgroups : grid, beside ? kFineUnroll : t.paced_unroll, pace};
+            return SwapShape{workgroups ? workgroups : grid, beside ? kFineUnroll : t.paced_unroll, pace, false};
         }
+        if (!beside) return SwapShape{workgroups ? workgroups : kToHostWorkgroups, kToHostUnroll, 0, true};
     }
     if ((flags & HFK_SWAP_SRC_HOST) != 0) {
         const uint32_t grid = beside ? kBesideFromHostWorkgroups : kFromHostWorkgroups;
-        return SwapShape{workgroups ? workgroups : grid, kFineUnroll, 0};
+        return SwapShape{workgroups ? workgroups : grid, kFineUnroll, 0, false};
     }
-    if (beside) return SwapShape{workgroups ? workgroups : kBesideWorkgroups, kBesideUnnamedUnroll, 0};
-    return SwapShape{workgroups ? workgroups : t.swap_workgroups, t.swap_unroll, 0};
+    if (beside) return SwapShape{workgroups ? workgroups : kBesideWorkgroups, kBesideUnnamedUnroll, 0, false};
+    return SwapShape{workgroups ? workgroups : t.swap_workgroups, t.swap_unroll, 0, false};
 }
 
 // Raw rate of a PCIe link in MB/s (lanes x GT/s x line encoding / 8) from the two strings sysfs

@@ -8,7 +8,8 @@
  *   - returns 0 on success, a negative hfk_status for a rejected argument, or a
  *     positive hipError_t reported by the HIP runtime,
  *   - never throws, owns no memory and keeps no state between calls apart from
- *     cached device properties and the values set through hfk_set_tuning().
+ *     cached device properties and the values set through hfk_set_tuning() (process-wide)
+ *     or hfk_thread_tuning_begin() (calling thread only).
  *
  * "Device-visible" below means an address a kernel may dereference: device
  * memory, or pinned host memory in its mapped (hipHostGetDevicePointer) form.
@@ -193,11 +194,13 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *                   the copy beside it runs 6x slower, the GEMM 4.4x / 1.6x (out / in): what a swap
  *                   holds in flight beyond the link's bandwidth-delay product queues in front of
  *                   every other kernel's traffic.
- *                 - HFK_SWAP_DST_HOST (swap-out): a swap of 64 MiB or more runs on 6 workgroups x 4
- *                   vectors per lane, paced at 0.89 of the link's raw rate (HFK_KNOB_LINK_MBPS): one
- *                   percent under the most the link accepts, which is what lets the launch hold its
- *                   pace on every block table (55.5-56.0 GB/s; at 0.90 consecutive or strided tables
- *                   lose up to 5 %) / 1.35x / 2.5x. A shorter one runs unpaced.
+ *                 - HFK_SWAP_DST_HOST (swap-out): a swap of 64 MiB or more runs on 12 workgroups x 8
+ *                   vectors per lane, unpaced, with non-temporal loads and plain stores (through the
+ *                   L2, which hands the link whole lines): 56.6-56.7 GB/s on every block table, 99 % of
+ *                   what hipMemcpy reaches toward the host / 5.9x / 4.0x. This is the fast shape, not
+ *                   the gentle one; the gentle one is asked for with HFK_SWAP_BESIDE_COMPUTE. (Paced
+ *                   through HFK_KNOB_THROUGHPUT_PACE_PERMILLE it runs on 6 x 4 with non-temporal stores:
+ *                   at 890, 55.5-56.0 GB/s / 1.35x / 2.5x.) A shorter one runs as with no flags.
  *                 - HFK_SWAP_SRC_HOST (swap-in): 40 x 1, unpaced: 57.4 GB/s / 1.95x / 1.6x.
  *                 - with HFK_SWAP_BESIDE_COMPUTE as well: out on 12 x 1 paced at 0.84: 52.8 GB/s / 1.05x /
  *                   1.64x; in on 24 x 1: 55.9 GB/s / 1.30x / 1.58x (1.55-1.6x is what any resident
@@ -246,7 +249,7 @@ typedef struct hfk_block_move {
  * be read by one and written by the other); either move may be empty (n_pairs 0).
  * `in_move` should be the one that reads host memory.
  * flags: 0, or HFK_SWAP_BESIDE_COMPUTE (other kernels run meanwhile and matter): 16 workgroups
- * instead of 32, one vector per lane and direction, and the launch offers the link 0.84 of its raw
+ * instead of 32, two vectors per lane and direction, and the launch offers the link 0.84 of its raw
  * rate in each direction (see hfk_swap_blocks). The result never depends on flags.
  *
  * No counterpart in the reference (its transfer op is host -> device only and one
@@ -397,8 +400,10 @@ HFK_API int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_
                       hfk_stream_t stream);
 
 /*
- * Benchmark/tuning knobs (process-wide, not thread-safe against concurrent
- * launches). Defaults are the measured best for MI355X.
+ * Tuning knobs. Defaults are the measured best for MI355X. hfk_set_tuning changes a knob for the whole
+ * process (every thread, every later call); hfk_thread_tuning_begin / _end change knobs for the calls
+ * the calling thread makes in between and touch nothing another thread can see: that is the way to
+ * give one call, or one engine thread, a launch shape of its own.
  */
 enum hfk_knob {
     HFK_KNOB_UNROLL = 0,        /* 16-byte accesses in flight per lane of the HBM-bound launches
@@ -412,23 +417,53 @@ enum hfk_knob {
     HFK_KNOB_SWAP_PACE_MBPS = 6,    /* rate a HFK_SWAP_BESIDE_COMPUTE swap offers toward the host, MB/s;
                                        0 (default) = 84 % of HFK_KNOB_LINK_MBPS               */
     HFK_KNOB_LINK_MBPS = 7,         /* raw rate of the current device's PCIe link, MB/s. Default: lanes x
-                                       GT/s x line encoding read from sysfs (0 if unreadable: such swaps
-                                       then run unpaced). Setting it overrides every device; -1 restores
-                                       the default                                                  */
+                                       GT/s x line encoding, the larger of the link's current and its maximum
+                                       rate as sysfs shows them (0 if unreadable: such swaps then run
+                                       unpaced). Setting it overrides every device; -1 restores the default */
     HFK_KNOB_DUPLEX_WORKGROUPS = 8, /* default grid bound of hfk_swap_blocks_duplex                       */
-    HFK_KNOB_THROUGHPUT_PACE_PERMILLE = 9, /* share of HFK_KNOB_LINK_MBPS, in thousandths, that a swap-out or
-                                       duplex swap of 64 MiB or more offers toward the host when it is
-                                       not marked HFK_SWAP_BESIDE_COMPUTE; 0 = unpaced; default 890      */
-    HFK_KNOB_PACED_UNROLL = 11,     /* like HFK_KNOB_UNROLL, for the paced throughput-mode swap toward the host
-                                       (default 4)                                                        */
-    HFK_KNOB_PACED_WORKGROUPS = 12, /* default grid of that swap (hfk_swap_blocks with HFK_SWAP_DST_HOST alone;
-                                       default 6)                                                          */
-    HFK_KNOB_HBM_LDS_BYTES = 10     /* dynamic LDS, 0..65536 bytes, that the HBM-bound launches (gathers, the
+    HFK_KNOB_THROUGHPUT_PACE_PERMILLE = 9, /* share of HFK_KNOB_LINK_MBPS, in thousandths, that a swap-out of
+                                       64 MiB or more offers toward a named host side when it is not marked
+                                       HFK_SWAP_BESIDE_COMPUTE. Default 0 = unpaced: 12 workgroups x 8 vectors
+                                       per lane with plain stores, the fastest shape and the one whose rate does
+                                       not depend on a clock; paced, HFK_KNOB_PACED_WORKGROUPS x
+                                       HFK_KNOB_PACED_UNROLL with non-temporal stores, gentler on kernels that
+                                       run beside it                                                       */
+    HFK_KNOB_HBM_LDS_BYTES = 10,    /* dynamic LDS, 0..65536 bytes, that the HBM-bound launches (gathers, the
                                        staged swap's kernel) request without using it: with 160 KiB of LDS
                                        per compute unit it bounds the workgroups a unit holds at a time   */
+    HFK_KNOB_PACED_UNROLL = 11,     /* like HFK_KNOB_UNROLL, for the paced throughput-mode swap toward the host */
+    HFK_KNOB_PACED_WORKGROUPS = 12, /* default grid of that swap (hfk_swap_blocks with HFK_SWAP_DST_HOST alone) */
+    HFK_KNOB_PACE_REPORT = 13,      /* diagnostic, default 0 = off: device-visible address of 8 x grid 64-bit
+                                       words. Every workgroup b of a paced hfk_swap_blocks launch writes, when
+                                       it has finished, at word 8 * b: ticks of the 100 MHz counter it ran,
+                                       ticks its schedule allotted, turns taken, turns that began behind
+                                       schedule, largest delay behind schedule in ticks, the pacing interval in
+                                       1/256 ticks, and two zeros. ran > allotted means the launch could not
+                                       hold its pace. The buffer must hold 64 bytes per workgroup launched     */
+    HFK_KNOB_DUPLEX_PACE_PERMILLE = 14, /* share of HFK_KNOB_LINK_MBPS, in thousandths, that a duplex swap of 64 MiB
+                                       or more toward the host offers in that direction when it is not marked
+                                       HFK_SWAP_BESIDE_COMPUTE; 0 = unpaced; default 890                        */
+    HFK_KNOB_TRANSFER_PACE_PERMILLE = 15, /* the same for a block-table transfer into a packed pool in host
+                                       memory; 0 (default) = unpaced                                            */
+    HFK_KNOB_TRANSFER_UNROLL = 16   /* 16-byte units per lane of that transfer, 2 or 8 (default 8)              */
 };
 HFK_API int hfk_set_tuning(int knob, int64_t value);
 HFK_API int64_t hfk_get_tuning(int knob);
+
+/*
+ * Knob values for the calling thread only. From hfk_thread_tuning_begin until hfk_thread_tuning_end
+ * every hfk_* call made by this thread reads the listed knobs from `overrides` and every other knob
+ * from the process-wide values; other threads see no change. A second begin replaces the first
+ * (there is no nesting). A list with an unknown knob or an invalid value is rejected as a whole
+ * (HFK_ERR_BAD_KNOB) and leaves the thread's overrides as they were. hfk_get_tuning shows the
+ * calling thread's view.
+ */
+typedef struct hfk_knob_value {
+    int knob;       /* enum hfk_knob */
+    int64_t value;
+} hfk_knob_value;
+HFK_API int hfk_thread_tuning_begin(const hfk_knob_value* overrides, uint32_t n);
+HFK_API void hfk_thread_tuning_end(void);
 
 #ifdef __cplusplus
 }

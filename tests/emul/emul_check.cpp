@@ -572,33 +572,40 @@ void case_transpose_table(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32
 
 // the launch shape of a swap, by flags, size and link rate: the rules as the header documents them
 void case_swap_shape() {
-    const SwapTuning t{16, 8, 6, 4, 890, 0};
+    const SwapTuning t{16, 8, 6, 4, 0, 0};        // the defaults: a throughput-mode swap-out is not paced
+    SwapTuning paced = t;
+    paced.throughput_pace_permille = 890;         // ... unless the knob says so
     const uint32_t link = 63015, out = HFK_SWAP_DST_HOST, in = HFK_SWAP_SRC_HOST, beside = HFK_SWAP_BESIDE_COMPUTE;
     const uint64_t big = 512ull << 20, small = 2ull << 20;
-    struct { uint32_t flags; uint64_t bytes; uint32_t link; uint32_t asked; uint32_t wg; int unroll; uint32_t pace; const char* what; } rows[] = {
-        {0, big, link, 0, 16, 8, 0, "nothing known: 16 x 8 unpaced"},
-        {out, big, link, 0, 6, 4, 56083, "swap-out of 64 MiB or more: 6 x 4 paced at 0.89"},
-        {out, kPaceFromBytes, link, 0, 6, 4, 56083, "exactly 64 MiB is paced"},
-        {out, kPaceFromBytes - 1, link, 0, 16, 8, 0, "a shorter swap-out stays unpaced"},
-        {out, small, link, 0, 16, 8, 0, "a 2 MiB swap-out stays unpaced"},
-        {out, big, 0, 0, 16, 8, 0, "link rate unknown: unpaced"},
-        {out | beside, small, link, 0, 12, 1, 52932, "beside compute: 12 x 1 paced at 0.84 whatever the size"},
-        {out | beside, big, 0, 0, 8, 4, 0, "beside compute, link unknown: 8 x 4 unpaced"},
-        {beside, big, link, 0, 8, 4, 0, "beside compute, no side named: 8 x 4 unpaced"},
-        {in, big, link, 0, 40, 1, 0, "swap-in: 40 x 1"},
-        {in | beside, big, link, 0, 24, 1, 0, "swap-in beside compute: 24 x 1"},
-        {in | out, big, link, 0, 6, 4, 56083, "both sides host memory: the paced shape wins"},
-        {out, big, link, 20, 20, 4, 56083, "the caller's grid bound is kept"},
-        {in, big, link, 7, 7, 1, 0, "the caller's grid bound is kept (swap-in)"},
-        {0, big, link, 300, 300, 8, 0, "the caller's grid bound is kept (no flags)"},
+    struct { const SwapTuning* tuning; uint32_t flags; uint64_t bytes; uint32_t link; uint32_t asked;
+             uint32_t wg; int unroll; uint32_t pace; bool plain; const char* what; } rows[] = {
+        {&t, 0, big, link, 0, 16, 8, 0, false, "nothing known: 16 x 8 unpaced"},
+        {&t, out, big, link, 0, 12, 8, 0, true, "swap-out of 64 MiB or more: 12 x 8 unpaced, plain stores"},
+        {&t, out, kLongSwapBytes, link, 0, 12, 8, 0, true, "exactly 64 MiB counts as long"},
+        {&t, out, kLongSwapBytes - 1, link, 0, 16, 8, 0, false, "a shorter swap-out runs as with no flags"},
+        {&t, out, small, link, 0, 16, 8, 0, false, "a 2 MiB swap-out runs as with no flags"},
+        {&t, out, big, 0, 0, 12, 8, 0, true, "link rate unknown: the unpaced shape needs none"},
+        {&t, out | beside, small, link, 0, 12, 1, 52932, false, "beside compute: 12 x 1 paced at 0.84 whatever the size"},
+        {&t, out | beside, big, 0, 0, 8, 4, 0, false, "beside compute, link unknown: 8 x 4 unpaced"},
+        {&t, beside, big, link, 0, 8, 4, 0, false, "beside compute, no side named: 8 x 4 unpaced"},
+        {&t, in, big, link, 0, 40, 1, 0, false, "swap-in: 40 x 1"},
+        {&t, in | beside, big, link, 0, 24, 1, 0, false, "swap-in beside compute: 24 x 1"},
+        {&t, in | out, big, link, 0, 12, 8, 0, true, "both sides host memory: the destination decides"},
+        {&t, out, big, link, 20, 20, 8, 0, true, "the caller's grid bound is kept"},
+        {&t, in, big, link, 7, 7, 1, 0, false, "the caller's grid bound is kept (swap-in)"},
+        {&t, 0, big, link, 300, 300, 8, 0, false, "the caller's grid bound is kept (no flags)"},
+        {&paced, out, big, link, 0, 6, 4, 56083, false, "pacing switched on: 6 x 4 at 0.89, non-temporal stores"},
+        {&paced, out, kLongSwapBytes - 1, link, 0, 16, 8, 0, false, "pacing switched on, short swap: unpaced"},
+        {&paced, out, big, 0, 0, 12, 8, 0, true, "pacing switched on, link unknown: the unpaced shape"},
+        {&paced, out, big, link, 20, 20, 4, 56083, false, "pacing switched on, the caller's grid bound is kept"},
     };
     for (const auto& r : rows) {
-        const SwapShape got = choose_swap_shape(r.flags, r.bytes, r.link, r.asked, t);
+        const SwapShape got = choose_swap_shape(r.flags, r.bytes, r.link, r.asked, *r.tuning);
         ++g_cases;
-        if (got.workgroups != r.wg || got.unroll != r.unroll || got.pace_mbps != r.pace) {
+        if (got.workgroups != r.wg || got.unroll != r.unroll || got.pace_mbps != r.pace || got.plain_stores != r.plain) {
             ++g_failures;
-            std::printf("swap shape: %s: got %u x %d paced %u, want %u x %d paced %u\n", r.what, got.workgroups, got.unroll,
-                        got.pace_mbps, r.wg, r.unroll, r.pace);
+            std::printf("swap shape: %s: got %u x %d paced %u plain %d, want %u x %d paced %u plain %d\n", r.what,
+                        got.workgroups, got.unroll, got.pace_mbps, (int)got.plain_stores, r.wg, r.unroll, r.pace, (int)r.plain);
         }
     }
     SwapTuning forced = t;
@@ -606,11 +613,6 @@ void case_swap_shape() {
     const SwapShape s1 = choose_swap_shape(out | beside, small, 0, 0, forced);
     ++g_cases;
     if (s1.workgroups != 12 || s1.unroll != 1 || s1.pace_mbps != 1) { ++g_failures; std::printf("swap shape: explicit pace\n"); }
-    forced = t;
-    forced.throughput_pace_permille = 0;   // pacing switched off
-    const SwapShape s2 = choose_swap_shape(out, big, link, 0, forced);
-    ++g_cases;
-    if (s2.workgroups != 16 || s2.unroll != 8 || s2.pace_mbps != 0) { ++g_failures; std::printf("swap shape: pace 0\n"); }
 }
 
 // the PCIe link-rate parser on the strings sysfs shows

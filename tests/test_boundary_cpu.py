@@ -83,6 +83,33 @@ def test_capi_loads_and_reports():
     assert capi.set_tuning(capi.KNOB_SWAP_PACE_MBPS, 0) == 0
 
 
+def test_thread_tuning_is_seen_by_the_calling_thread_only():
+    """hfk_thread_tuning_begin / _end: the overrides are this thread's view, another thread keeps the
+    process-wide values, a bad list is rejected whole, and _end restores the process-wide view."""
+    import threading
+
+    base = capi.get_tuning(capi.KNOB_SWAP_WORKGROUPS)
+    seen = {}
+    with capi.thread_tuning({capi.KNOB_SWAP_WORKGROUPS: base + 5, capi.KNOB_UNROLL: 4}):
+        assert capi.get_tuning(capi.KNOB_SWAP_WORKGROUPS) == base + 5
+        assert capi.get_tuning(capi.KNOB_UNROLL) == 4
+        t = threading.Thread(target=lambda: seen.update(other=capi.get_tuning(capi.KNOB_SWAP_WORKGROUPS)))
+        t.start()
+        t.join()
+        assert seen["other"] == base
+        # a list with one bad entry changes nothing
+        bad = (capi.KnobValue * 2)(capi.KnobValue(capi.KNOB_UNROLL, 2), capi.KnobValue(capi.KNOB_UNROLL, 3))
+        assert capi.load().hfk_thread_tuning_begin(bad, 2) == -4
+        assert capi.get_tuning(capi.KNOB_UNROLL) == 4
+        assert capi.load().hfk_thread_tuning_begin(None, 1) == -1
+        # the process-wide value can change underneath; the override still wins here
+        assert capi.set_tuning(capi.KNOB_SWAP_WORKGROUPS, base + 1) == 0
+        assert capi.get_tuning(capi.KNOB_SWAP_WORKGROUPS) == base + 5
+    assert capi.get_tuning(capi.KNOB_SWAP_WORKGROUPS) == base + 1
+    assert capi.set_tuning(capi.KNOB_SWAP_WORKGROUPS, base) == 0
+    assert capi.get_tuning(capi.KNOB_UNROLL) == 1
+
+
 def test_argument_errors_are_reported_before_any_gpu_work():
     # None of these reach a launch, so they are safe without a device.
     assert capi.gather_rows(0, 0, 0, True, 0, 16) == 0                 # n_ids == 0: no-op

@@ -476,24 +476,19 @@ def test_paced_swap_ends_when_its_rate_is_unreachably_low(memory):
     src_ids, dst_ids = W.block_table(cfg, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
     pairs = W.pairs_tensor(src_ids, dst_ids).to(DEV)
     dtab = ptr_table(dev)
-    try:
-        for what, knob, value in (("1 MB/s", capi.KNOB_SWAP_PACE_MBPS, 1), ("unknown link", capi.KNOB_LINK_MBPS, 0)):
-            announce("paced swap, %s: %d planes x %d blocks" % (what, cfg.planes, src_ids.numel()))
-            assert capi.set_tuning(knob, value) == 0
-            pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0x11)
+    for what, knob, value in (("1 MB/s", capi.KNOB_SWAP_PACE_MBPS, 1), ("unknown link", capi.KNOB_LINK_MBPS, 0)):
+        announce("paced swap, %s: %d planes x %d blocks" % (what, cfg.planes, src_ids.numel()))
+        pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0x11)
+        with capi.thread_tuning({knob: value}):      # this thread's calls only; the process-wide knobs stay
             capi.check(capi.swap_blocks(host_ptr_table(host).data_ptr(), dtab.data_ptr(), pairs.data_ptr(), cfg.planes,
                                         src_ids.numel(), bb, bb, bb, cfg.dev_blocks, cfg.host_blocks, 0, stream_handle(),
                                         capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE))
-            torch.cuda.synchronize()
-            for p in range(cfg.planes):
-                want = torch.full((cfg.host_blocks, bb), 0x11, dtype=torch.uint8)
-                O.torch_swap_blocks(want, cpu[p], src_ids, dst_ids)
-                assert torch.equal(host[p], want), "%s plane %d" % (what, p)
-            assert capi.set_tuning(capi.KNOB_SWAP_PACE_MBPS, 0) == 0
-            assert capi.set_tuning(capi.KNOB_LINK_MBPS, -1) == 0
-    finally:
-        capi.set_tuning(capi.KNOB_SWAP_PACE_MBPS, 0)
-        capi.set_tuning(capi.KNOB_LINK_MBPS, -1)
+        torch.cuda.synchronize()
+        for p in range(cfg.planes):
+            want = torch.full((cfg.host_blocks, bb), 0x11, dtype=torch.uint8)
+            O.torch_swap_blocks(want, cpu[p], src_ids, dst_ids)
+            assert torch.equal(host[p], want), "%s plane %d" % (what, p)
+    assert capi.get_tuning(capi.KNOB_SWAP_PACE_MBPS) == 0
     announce("PCIe link rate read from sysfs: %d MB/s (0 = unreadable: paced swaps run unpaced)" % capi.get_tuning(capi.KNOB_LINK_MBPS))
 
 
@@ -549,21 +544,16 @@ def test_results_independent_of_tuning_and_grid():
         w = torch.zeros(16, cfg.block_bytes, dtype=torch.uint8)
         O.torch_swap_blocks(w, W.as_bytes(cpu[p]), src_ids, dst_ids)
         want.append(w)
-    saved = [capi.get_tuning(k) for k in range(3)]
-    try:
-        for unroll in (1, 2, 4, 8, 16):
-            for nt in (0, 1, 2, 3):
-                for wgs in (0, 1, 5, 100000):
-                    assert capi.set_tuning(capi.KNOB_UNROLL, unroll) == 0
-                    assert capi.set_tuning(capi.KNOB_NONTEMPORAL, nt) == 0
-                    out = [torch.zeros(16, cfg.block_bytes, dtype=torch.uint8, device=DEV) for _ in range(cfg.planes)]
+    for unroll in (1, 2, 4, 8, 16):
+        for nt in (0, 1, 2, 3):
+            for wgs in (0, 1, 5, 100000):
+                out = [torch.zeros(16, cfg.block_bytes, dtype=torch.uint8, device=DEV) for _ in range(cfg.planes)]
+                with capi.thread_tuning({capi.KNOB_SWAP_UNROLL: unroll, capi.KNOB_UNROLL: unroll, capi.KNOB_NONTEMPORAL: nt}):
                     swap(ptr_table(out), ptr_table(dev), pairs, cfg.planes, cfg.block_bytes, workgroups=wgs)
-                    torch.cuda.synchronize()
-                    for p in range(cfg.planes):
-                        assert torch.equal(out[p].cpu(), want[p]), (unroll, nt, wgs, p)
-    finally:
-        for k, v in enumerate(saved):
-            capi.set_tuning(k, v)
+                torch.cuda.synchronize()
+                for p in range(cfg.planes):
+                    assert torch.equal(out[p].cpu(), want[p]), (unroll, nt, wgs, p)
+    assert capi.get_tuning(capi.KNOB_NONTEMPORAL) == 3
 
 
 def test_strided_planes():
