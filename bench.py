@@ -31,7 +31,8 @@ if ROOT not in sys.path:
 
 PCIE5_X16_GBPS = 32.0 * 16 * (128.0 / 130.0) / 8.0   # 63.0 GB/s per direction, before packet overheads
 HBM_PEAK_GBPS = 8000.0                               # MI355X HBM3E
-ALL_SECTIONS = ("swap_out", "swap_in", "gather", "duplex", "staged", "hbm_ceiling", "tables")
+ALL_SECTIONS = ("swap_out", "swap_in", "gather", "gather_orders", "duplex", "staged", "hbm_ceiling", "tables", "repeat",
+                "reference_ops")
 
 
 def log(msg):
@@ -624,6 +625,118 @@ def section_tables(b, w, steps):
             "two planes verified per table and shape" % max(4, steps // 2)}
 
 
+def section_gather_orders(b, w, steps):
+    """The block gather on the workload's own cache under different orders of the same kind of work: which
+    blocks are read (in sequence, random, random but sorted, random within 2 MiB neighbourhoods) and in
+    which order the destination is written (in sequence, or at random with the source in sequence). Every
+    launch reads and writes the same number of bytes with the same kernel shape; what differs is locality in
+    DRAM rows and in address translation. Verified on every plane before a figure is kept."""
+    torch, capi, cfg = b.torch, b.capi, w.cfg
+    planes, bb, n = cfg.planes, cfg.block_bytes, cfg.n_blocks
+    gen = torch.Generator().manual_seed(cfg.base_seed + 7)
+    own = w.src_ids
+    per_2mib = max(1, (2 << 20) // bb)
+    groups = torch.randperm(cfg.dev_blocks // per_2mib, generator=gen)[:max(1, n // per_2mib)]
+    grouped = torch.cat([g * per_2mib + torch.randperm(per_2mib, generator=gen) for g in groups.tolist()])[:n]
+    orders = {
+        "the_workloads_own_random": own,
+        "sequential": torch.arange(n) + 7,
+        "random_sorted": torch.sort(own).values,
+        "random_within_2MiB_groups": grouped,
+    }
+    out = {}
+    iters = max(steps, 200)
+    for name, ids in orders.items():
+        if ids.numel() != n or int(ids.max()) >= cfg.dev_blocks:
+            continue
+        ids_dev = ids.to(b.dev)
+
+        def launch():
+            capi.check(capi.gather_blocks(w.prefill_tab.data_ptr(), w.dev_tab.data_ptr(), ids_dev.data_ptr(), planes, n, bb, bb,
+                                          cfg.dev_blocks, 0, b.stream), "hfk_gather_blocks")
+        w.prefill.zero_()
+        _, ms = b.timed(launch, iters, 3)
+        for p in range(planes):
+            assert torch.equal(w.prefill[p], w.dev_bytes[p].index_select(0, ids_dev)), "gather mismatch (%s, plane %d)" % (name, p)
+        out[name] = round(w.gather_alg_bytes / (ms * 1e6), 1)
+    # the same bytes with the source in sequence and the destination at random: a device-to-device swap through the
+    # same block-copy body, one vector per lane and one workgroup per chunk like the gather
+    perm = torch.randperm(n, generator=gen)
+    pairs = b.W.pairs_tensor(torch.arange(n) + 7, perm).to(b.dev)
+    with capi.thread_tuning({capi.KNOB_SWAP_UNROLL: capi.get_tuning(capi.KNOB_UNROLL)}):
+        def scatter():
+            capi.check(capi.swap_blocks(w.prefill_tab.data_ptr(), w.dev_tab.data_ptr(), pairs.data_ptr(), planes, n, bb, bb, bb,
+                                        cfg.dev_blocks, n, 1 << 20, b.stream, 0), "hfk_swap_blocks(device to device)")
+        w.prefill.zero_()
+        _, ms = b.timed(scatter, iters, 3)
+    seq_dev, perm_dev = (torch.arange(n) + 7).to(b.dev), perm.to(b.dev)
+    for p in range(planes):
+        assert torch.equal(w.prefill[p].index_select(0, perm_dev), w.dev_bytes[p].index_select(0, seq_dev)), "scatter mismatch %d" % p
+    out["sequential_source_random_destination"] = round(w.gather_alg_bytes / (ms * 1e6), 1)
+    log("gather by order of work, GB/s of HBM traffic: " + ", ".join("%s %.0f" % kv for kv in out.items()))
+    return {"traffic_GBps": out, "launches_timed": iters, "frac_of_hbm_peak": {k: round(v / HBM_PEAK_GBPS, 4) for k, v in out.items()}}
+
+
+def section_repeat(b, w, steps, warmup, flags, first_value):
+    """The timed step once more, as the last thing done on the headline workload: the same launch on the same
+    table and pool after everything else has run. Also what a paced launch of the same swap does with its
+    schedule (hfk's pace report): a launch that holds its pace ends with ran <= allotted."""
+    torch, capi, cfg = b.torch, b.capi, w.cfg
+    for p in range(cfg.planes):
+        w.host_planes[p][w.dst_ids] = 0
+    spread = b.launch_spread(lambda: w.swap_out(flags), min(steps, 10))
+    wall, ms = b.timed(lambda: w.swap_out(flags), steps, warmup)
+    for p in range(cfg.planes):
+        want = w.dev_bytes[p].index_select(0, w.ids_dev).cpu()
+        assert torch.equal(w.host_planes[p].index_select(0, w.dst_ids), want), "repeated swap-out mismatch in plane %d" % p
+    gbps = steps * w.payload / wall / 1e9
+    iso = {k: round(w.payload / (spread[k] * 1e6), 2) for k in ("median_ms", "min_ms", "max_ms")}
+    out = {"GBps": gbps, "kernel_GBps": w.payload / (ms * 1e6),
+           "isolated_launches_GBps": {"median": iso["median_ms"], "slowest": iso["max_ms"], "fastest": iso["min_ms"]},
+           "first_measurement_GBps": first_value,
+           "last_over_first": None if not first_value else gbps / first_value}
+    log("swap-out repeated at the end: %.2f GB/s (first measurement %s), isolated launches %.2f / %.2f / %.2f "
+        "(slowest / median / fastest)" % (gbps, "%.2f" % first_value if first_value else "-", iso["max_ms"],
+                                           iso["median_ms"], iso["min_ms"]))
+    # a paced launch of the same swap and how it kept its schedule
+    report = torch.zeros(64 * 8, dtype=torch.int64, device=b.dev)
+    paced = {}
+    for permille in (890, 900):
+        with capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: permille, capi.KNOB_PACE_REPORT: report.data_ptr()}):
+            _, pms = b.timed(lambda: w.swap_out(capi.SWAP_DST_HOST), max(4, steps // 2), 1)
+            grid = capi.get_tuning(capi.KNOB_PACED_WORKGROUPS)
+        rows = report.cpu().view(64, 8)[:grid]
+        ran, allotted, turns, late, worst = (rows[:, i].double() for i in range(5))
+        paced["at_0.%d_of_link" % (permille // 10)] = {
+            "GBps": round(w.payload / (pms * 1e6), 2), "workgroups": grid,
+            "ran_over_allotted": round(float((ran / allotted.clamp(min=1)).max()), 4),
+            "late_turns_pct": round(100 * float(late.sum() / turns.sum().clamp(min=1)), 2),
+            "largest_delay_us": round(float(worst.max()) / 100.0, 1)}
+    out["paced_launch_of_the_same_swap"] = paced
+    log("paced launches of the same swap: %s" % json.dumps(paced))
+    return out
+
+
+def section_reference_ops(b):
+    """The reference's own three ops on the shapes its README quotes (pcieThrough/tests/README.md:34-42,70-75):
+    gather out of a registered host table of [4 000 000, 512] fp16 rows, one call per batch and ten batches per
+    call, and the layout-converting transfer of one block, direct and staged, on four shapes; next to them
+    the block-table transfer of eight blocks in one launch, both directions, and the row gather out of a
+    table in device memory. Every figure is printed only after its bytes were compared."""
+    from heterofusedkernels_amd import reference_shapes_bench as R
+    t0 = time.time()
+    out = {"gather": [], "transfer": [], "rows": 4000000, "runs": 60}
+    R.config1_latency(out, runs=200)
+    R.gather_table(out["rows"], out["runs"], out, fill="bytes")
+    R.gather_hbm_table(out)
+    R.transfer_table(out)
+    out["seconds"] = round(time.time() - t0, 1)
+    out["how"] = ("gather: host wall time per call over %d calls, as pcieThrough/tests/test_gather.py:50-61; transfer: mean of "
+                  "per-op HIP event times, as tests/test_transfer_kernel.py:51-52,86-88; table_in / table_out: 8 blocks "
+                  "in one launch, one event pair around 5 launches" % out["runs"])
+    return out
+
+
 def section_hbm_ceiling(b, steps, warmup):
     """What HBM gives a kernel of the gather's shape (256-lane workgroups, one workgroup per chunk, 16-byte
     non-temporal accesses) that only reads, only writes, or copies 512 MiB of contiguous device memory.
@@ -796,7 +909,8 @@ def main():
                          "always runs unless a profile of one other kernel alone is wanted")
     ap.add_argument("--tune", default="", help="comma list of library knobs for experiments, e.g. unroll=4,nt=0 "
                     "(unroll, nt, wg_per_cu, swap_wgs, swap_unroll, duplex_unroll, duplex_wgs, pace_mbps, link_mbps, "
-                    "throughput_pace, hbm_lds, paced_unroll, paced_wgs); defaults are the shipped ones")
+                    "throughput_pace, hbm_lds, paced_unroll, paced_wgs, transfer_pace); defaults are "
+                    "the shipped ones")
     ap.add_argument("--out-flags", type=int, default=1, help="flags of the timed swap-out (default HFK_SWAP_DST_HOST = 1: "
                     "the caller knows its destination is host memory; 0 = say nothing)")
     ap.add_argument("--skip-cpu-baseline", action="store_true")
@@ -815,7 +929,8 @@ def main():
              "swap_unroll": capi.KNOB_SWAP_UNROLL, "pace_mbps": capi.KNOB_SWAP_PACE_MBPS, "link_mbps": capi.KNOB_LINK_MBPS,
              "duplex_wgs": capi.KNOB_DUPLEX_WORKGROUPS, "throughput_pace": capi.KNOB_THROUGHPUT_PACE_PERMILLE,
              "hbm_lds": capi.KNOB_HBM_LDS_BYTES, "paced_unroll": capi.KNOB_PACED_UNROLL,
-             "paced_wgs": capi.KNOB_PACED_WORKGROUPS}
+             "paced_wgs": capi.KNOB_PACED_WORKGROUPS,
+             "transfer_pace": capi.KNOB_TRANSFER_PACE_PERMILLE}
     tuned = {}
     for item in filter(None, args.tune.split(",")):
         key, val = item.split("=")
@@ -855,6 +970,8 @@ def main():
         torch_gather_gbps = 2 * cfg.n_blocks * cfg.block_bytes / (ms_t * 1e6)
         log("torch.index_select on one plane: %.1f GB/s" % torch_gather_gbps)
 
+    gather_orders = section_gather_orders(b, w, args.steps) if "gather_orders" in sections else None
+
     duplex = None
     if "duplex" in sections:
         duplex, _keep = section_duplex(b, w, args.steps, args.warmup)
@@ -879,6 +996,7 @@ def main():
     memcpy_loop = None if args.skip_memcpy_loop else section_memcpy_loop(b, w)
     cpu_baseline = None if args.skip_cpu_baseline else section_cpu_baseline(b, w)
     tables = section_tables(b, w, args.steps) if "tables" in sections else None
+    repeat = section_repeat(b, w, args.steps, args.warmup, args.out_flags, value) if "repeat" in sections else None
     headline_config = config_summary(w, {"tuning_overrides": tuned})
     link_known = capi.get_tuning(capi.KNOB_LINK_MBPS) > 0
     gather_unroll = capi.get_tuning(capi.KNOB_UNROLL)
@@ -890,6 +1008,8 @@ def main():
     configs = {}
     for key in others:
         configs[key] = measure_other_config(b, key, by_key[key], args.steps, args.warmup, d2h_peak, h2d_peak)
+
+    reference_ops = section_reference_ops(b) if "reference_ops" in sections else None
 
     # ---- HBM traffic measured offline with rocprofv3 --pmc, if recorded -------------
     traffic = {}
@@ -903,7 +1023,14 @@ def main():
     out_kernel_gbps = rate(w_payload, kernel_ms_out)
     in_kernel_gbps = rate(w_payload, kernel_ms_in)
     gather_alg_bytes = 2 * w_payload + 8 * headline_config["blocks_per_launch"]
-    paced = (args.out_flags & capi.SWAP_DST_HOST) and link_known and w_payload >= (64 << 20) and pace_permille > 0
+    long_out = (args.out_flags & capi.SWAP_DST_HOST) and w_payload >= (64 << 20)
+    paced = long_out and link_known and pace_permille > 0
+    if paced:
+        out_kernel = "swap_blocks_kernel<%d, 3>, %d workgroups, paced at 0.%d of the link" % (paced_unroll, paced_wgs, pace_permille // 10)
+    elif long_out:
+        out_kernel = "swap_blocks_kernel<8, 1>, 12 workgroups (non-temporal loads, plain stores), unpaced"
+    else:
+        out_kernel = "swap_blocks_kernel<8, 3>, 16 workgroups"
     result = {
         "metric": "KV swap GB/s (% of PCIe5 x16 peak); block gather GB/s (% of HBM peak)",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -914,12 +1041,12 @@ def main():
         # PCIe Gen5 x16 link, so that is the roofline it is priced against (theoretical link rate as
         # `peak`, the rate one large pinned hipMemcpyAsync reaches in this run as `peak_measured`).
         "roofline": {
-            "kernel": ("swap_blocks_kernel<%d, 3>, %d workgroups, paced at 0.%d of the link" %
-                       (paced_unroll, paced_wgs, pace_permille // 10) if paced else "swap_blocks_kernel<8, 3>, 16 workgroups") +
-                      " via hfk_swap_blocks (swap-out, HBM -> pinned host)", "bound": "pcie",
+            "kernel": out_kernel + " via hfk_swap_blocks (swap-out, HBM -> pinned host)", "bound": "pcie",
             "achieved": out_kernel_gbps, "peak": PCIE5_X16_GBPS, "unit": "GB/s",
             "frac": frac(out_kernel_gbps, PCIE5_X16_GBPS),
             "traffic": traffic.get("swap_out_hbm_bytes_per_launch"),
+            "traffic_source": "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this launch, collected "
+                              "in a run of its own; this run does not measure it)",
             "peak_measured": d2h_peak, "frac_of_measured": frac(out_kernel_gbps, d2h_peak),
             "algorithmic_bytes_per_launch": w_payload, "avg_launch_ms": kernel_ms_out,
         },
@@ -946,10 +1073,13 @@ def main():
         "staged": staged,
         "fragmented_host_slots": fragmented,
         "swap_out_by_block_table": tables,
+        "swap_out_repeat": repeat,
+        "gather_by_order_of_work": gather_orders,
+        "reference_ops": reference_ops,
         "beside_compute": beside,
         "memcpy_block_loop": memcpy_loop,
         "cpu_baseline": cpu_baseline,
-        "verified": "bit-exact on every plane: " + ", ".join(sorted(sections - {"hbm_ceiling", "tables"})),
+        "verified": "bit-exact on every plane: " + ", ".join(sorted(sections - {"hbm_ceiling", "tables", "reference_ops"})),
     }
     print(json.dumps(result), flush=True)
 

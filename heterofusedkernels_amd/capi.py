@@ -28,6 +28,8 @@ KNOB_PACE_REPORT = 13
 KNOB_DUPLEX_PACE_PERMILLE = 14
 KNOB_TRANSFER_PACE_PERMILLE = 15
 KNOB_TRANSFER_UNROLL = 16
+KNOB_CHECK_HOST_COLUMN = 17
+KNOB_TRANSFER_TILED = 18
 SWAP_DST_HOST = 1
 SWAP_SRC_HOST = 2
 SWAP_BESIDE_COMPUTE = 4
@@ -35,6 +37,7 @@ SWAP_SRC_DEVICE = 8
 SWAP_DST_DEVICE = 16
 STATIC_STAGING_BYTES = 64 << 20
 ERR_STAGING_TOO_SMALL = -7
+ERR_TABLE_MISMATCH = -8
 
 
 class KnobValue(ctypes.Structure):

@@ -376,13 +376,17 @@ HFK_HD void zero_chunk(uint64_t d_addr, uint64_t block_bytes, uint32_t chunk, ui
 
 // SPLIT: the launch moves only the pairs its run filter selects (a.run_mode must then be
 // kLongRunsOnly or kShortRunsOnly); without it a.run_mode must be kAllPairs.
-template <typename IdT, int UNROLL, int NT, bool SPLIT = false>
+// PACED: the launch may be paced (a.pace_q8); kernels that never are (everything HBM-bound) are built
+// without it and carry none of the pacer's code: one workgroup per 4 KiB chunk pays for every
+// instruction of its prologue.
+template <typename IdT, int UNROLL, int NT, bool SPLIT = false, bool PACED = true>
 HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
-    Pacer pacer(a.pace_q8, bid, nb);
-    uint64_t w = bid;                   // 64-bit so that w + nb cannot wrap
+    Pacer pacer(PACED ? a.pace_q8 : 0u, bid, nb);
+    uint64_t id = bid;                  // 64-bit so that id + nb cannot wrap
     uint32_t judged_pair = 0xffffffffu; // SPLIT: the pair the filter was last evaluated for, and its verdict
     bool judged_selected = false;       // (a workgroup's consecutive items mostly belong to one pair)
-    while (w < a.n_work) {
+    while (id < a.n_work) {
+        const uint64_t w = id;
         uint64_t s_addr = 0, d_addr = 0;
         uint32_t chunk = 0;
         if constexpr (SPLIT) {
@@ -392,24 +396,24 @@ HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t 
                 judged_selected = pair_selected(a, pair);
             }
             if (!judged_selected) {
-                w = next_pair_item(a, w, bid, nb);
+                id = next_pair_item(a, w, bid, nb);
                 continue;
             }
         }
         const ChunkAction what = resolve_chunk<IdT, SPLIT>(a, (uint32_t)w, s_addr, d_addr, chunk);
         if (what == kSkip) {            // moves nothing, so it takes no turn on the link either
-            w = SPLIT ? next_pair_item(a, w, bid, nb) : w + nb;
+            id = SPLIT ? next_pair_item(a, w, bid, nb) : id + nb;
             continue;
         }
-        pacer.wait_turn();
+        if constexpr (PACED) pacer.wait_turn();
         if (what == kCopy) {
             copy_chunk<UNROLL, NT>(s_addr, d_addr, a.block_bytes, chunk, tid);
         } else {
             zero_chunk<UNROLL, NT>(d_addr, a.block_bytes, chunk, tid);
         }
-        w += nb;
+        id += nb;
     }
-    pacer.report(a.pace_report, bid, tid);
+    if constexpr (PACED) pacer.report(a.pace_report, bid, tid);
 }
 
 // ---------------------------------------------------------------------------
@@ -563,6 +567,8 @@ struct TransposeArgs {
     uint32_t total_units;        // T * L * H * row_units, per block
     uint32_t n_work;             // n_pairs * chunks_per_block
     uint32_t pace_q8;            // see Pacer; 0 = unpaced
+    uint32_t tile_tokens;        // tiled form only (plan_transpose_tiles): tokens and packed rows per tile;
+    uint32_t tile_rows;          // chunks_per_block is then the number of tiles per block
 };
 
 // Where the body finds layer l's address. The layer differs from lane to lane (a 128-byte row is 8
@@ -590,81 +596,192 @@ HFK_HD void unit_from_bytes(const HFK_GLOBAL uint8_t* p, vec16& v) {
     v.w = w[3];
 }
 
-template <typename V, int UNROLL, int NT, bool TO_PACKED, typename LayerTable>
-HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid, const LayerTable& layer_address) {
-    constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
+// One work item of the transfer: chunk `chunk` of the pair's packed block.
+struct TransposeItem {
+    uint64_t packed_addr;   // address of the pair's packed block
+    uint64_t layered_off;   // byte offset of the pair's block inside every layer's cache
+    uint64_t g0;            // this lane's first unit within the packed block
+};
+
+// Where work item w lives; false when the pair's block indices are out of range.
+HFK_HD bool transpose_item(const TransposeArgs& a, uint64_t w64, uint32_t tid, uint32_t chunk_units, TransposeItem& it) {
+    const uint32_t w = (uint32_t)w64;
+    const uint32_t chunk = w % a.chunks_per_block;
+    const uint32_t pair = w / a.chunks_per_block;
+    const uint64_t pb = a.pairs ? (uint64_t)table_entry(a.pairs, 2 * (uint64_t)pair) : 0;
+    const uint64_t db = a.pairs ? (uint64_t)table_entry(a.pairs, 2 * (uint64_t)pair + 1) : 0;
+    if (pb >= a.packed_limit || db >= a.layered_limit) {
+        return false;
+    }
+    it.packed_addr = a.packed + pb * a.packed_stride;
+    it.layered_off = db * a.layered_stride;
+    it.g0 = (uint64_t)chunk * chunk_units + tid;
+    return true;
+}
+
+// The layered-side address of each of the lane's UNROLL units (0 past the end of the block).
+template <typename V, int UNROLL, typename LayerTable>
+HFK_HD void transpose_addresses(const TransposeArgs& a, const TransposeItem& it, const LayerTable& layer_address,
+                                uint64_t (&layered_addr)[UNROLL]) {
     const uint32_t LH = a.L * a.H;
-    Pacer pacer(a.pace_q8, bid, nb);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t g64 = it.g0 + (uint64_t)u * kWorkgroupLanes;
+        layered_addr[u] = 0;
+        if (g64 < a.total_units) {
+            const uint32_t g = (uint32_t)g64;
+            const uint32_t r = g / a.row_units;      // packed row = (t*L + l)*H + h
+            const uint32_t col = g - r * a.row_units;
+            const uint32_t t = r / LH;
+            const uint32_t lh = r - t * LH;
+            const uint32_t l = lh / a.H;
+            const uint32_t h = lh - l * a.H;
+            const uint64_t unit = ((uint64_t)h * a.T + t) * a.row_units + col;
+            layered_addr[u] = layer_address(l) + it.layered_off + unit * sizeof(V);
+        }
+    }
+}
 
-    for (uint64_t w64 = bid; w64 < a.n_work; w64 += nb) {
-        const uint32_t w = (uint32_t)w64;
-        const uint32_t chunk = w % a.chunks_per_block;
-        const uint32_t pair = w / a.chunks_per_block;
-        const uint64_t pb = a.pairs ? (uint64_t)table_entry(a.pairs, 2 * (uint64_t)pair) : 0;
-        const uint64_t db = a.pairs ? (uint64_t)table_entry(a.pairs, 2 * (uint64_t)pair + 1) : 0;
-        if (pb >= a.packed_limit || db >= a.layered_limit) {
-            continue;
-        }
-        pacer.wait_turn();
-        const uint64_t packed_addr = a.packed + pb * a.packed_stride;
-        const uint64_t layered_off = db * a.layered_stride;
-        const uint64_t g0 = (uint64_t)chunk * kChunkUnits + tid;
-
-        V v[UNROLL];
-        uint64_t layered_addr[UNROLL];
+// Loads the lane's units of one work item from the layered side (TO_PACKED) or the packed side.
+template <typename V, int UNROLL, int NT, bool TO_PACKED>
+HFK_HD void transpose_load(const TransposeArgs& a, const TransposeItem& it, const uint64_t (&layered_addr)[UNROLL], V (&v)[UNROLL]) {
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const uint64_t g64 = g0 + (uint64_t)u * kWorkgroupLanes;
-            layered_addr[u] = 0;
-            if (g64 < a.total_units) {
-                const uint32_t g = (uint32_t)g64;
-                const uint32_t r = g / a.row_units;      // packed row = (t*L + l)*H + h
-                const uint32_t col = g - r * a.row_units;
-                const uint32_t t = r / LH;
-                const uint32_t lh = r - t * LH;
-                const uint32_t l = lh / a.H;
-                const uint32_t h = lh - l * a.H;
-                const uint64_t unit = ((uint64_t)h * a.T + t) * a.row_units + col;
-                layered_addr[u] = layer_address(l) + layered_off + unit * sizeof(V);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const uint64_t g64 = g0 + (uint64_t)u * kWorkgroupLanes;
-            if (g64 < a.total_units) {
-                if constexpr (TO_PACKED) {
-                    if ((layered_addr[u] & (sizeof(V) - 1)) == 0) {
-                        v[u] = load_unit<NT>(global_in<V>(layered_addr[u]));
-                    } else {  // layer cache not aligned to the unit: byte loads keep it correct
-                        unit_from_bytes(global_in<uint8_t>(layered_addr[u]), v[u]);
-                    }
-                } else {
-                    v[u] = load_unit<NT>(global_in<V>(packed_addr) + g64);
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t g64 = it.g0 + (uint64_t)u * kWorkgroupLanes;
+        if (g64 < a.total_units) {
+            if constexpr (TO_PACKED) {
+                if ((layered_addr[u] & (sizeof(V) - 1)) == 0) {
+                    v[u] = load_unit<NT>(global_in<V>(layered_addr[u]));
+                } else {  // layer cache not aligned to the unit: byte loads keep it correct
+                    unit_from_bytes(global_in<uint8_t>(layered_addr[u]), v[u]);
                 }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const uint64_t g64 = g0 + (uint64_t)u * kWorkgroupLanes;
-            if (g64 < a.total_units) {
-                if constexpr (TO_PACKED) {
-                    store_unit<NT>(global_out<V>(packed_addr) + g64, v[u]);
-                } else if ((layered_addr[u] & (sizeof(V) - 1)) == 0) {
-                    store_unit<NT>(global_out<V>(layered_addr[u]), v[u]);
-                } else {  // byte stores for a misaligned layer cache
-                    HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(layered_addr[u]);
-                    for (uint32_t k = 0; k < sizeof(V); ++k) {
-                        d1[k] = unit_byte(v[u], k);
-                    }
-                }
+            } else {
+                v[u] = load_unit<NT>(global_in<V>(it.packed_addr) + g64);
             }
         }
     }
 }
 
 template <typename V, int UNROLL, int NT, bool TO_PACKED>
+HFK_HD void transpose_store(const TransposeArgs& a, const TransposeItem& it, const uint64_t (&layered_addr)[UNROLL], const V (&v)[UNROLL]) {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t g64 = it.g0 + (uint64_t)u * kWorkgroupLanes;
+        if (g64 < a.total_units) {
+            if constexpr (TO_PACKED) {
+                store_unit<NT>(global_out<V>(it.packed_addr) + g64, v[u]);
+            } else if ((layered_addr[u] & (sizeof(V) - 1)) == 0) {
+                store_unit<NT>(global_out<V>(layered_addr[u]), v[u]);
+            } else {  // byte stores for a misaligned layer cache
+                HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(layered_addr[u]);
+                for (uint32_t k = 0; k < sizeof(V); ++k) {
+                    d1[k] = unit_byte(v[u], k);
+                }
+            }
+        }
+    }
+}
+
+template <typename V, int UNROLL, int NT, bool TO_PACKED, typename LayerTable>
+HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid, const LayerTable& layer_address) {
+    constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
+    Pacer pacer(a.pace_q8, bid, nb);
+    for (uint64_t w64 = bid; w64 < a.n_work; w64 += nb) {
+        TransposeItem it;
+        if (!transpose_item(a, w64, tid, kChunkUnits, it)) {
+            continue;
+        }
+        pacer.wait_turn();
+        V v[UNROLL];
+        uint64_t layered_addr[UNROLL];
+        transpose_addresses<V, UNROLL>(a, it, layer_address, layered_addr);
+        transpose_load<V, UNROLL, NT, TO_PACKED>(a, it, layered_addr, v);
+        transpose_store<V, UNROLL, NT, TO_PACKED>(a, it, layered_addr, v);
+    }
+}
+
+template <typename V, int UNROLL, int NT, bool TO_PACKED>
 HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid) {
     transpose_body<V, UNROLL, NT, TO_PACKED>(a, bid, nb, tid, LayerTableInMemory{a.layer_ptrs});
+}
+
+// ---------------------------------------------------------------------------
+// The transfer toward the packed side, tiled through LDS. The direct body above reads the layered
+// side in rows: with 128-byte rows a wavefront's load touches eight different (layer, head) places,
+// and toward a packed pool in host memory that form stays 2-3 GB/s under what the link takes from a
+// kernel that reads long runs. Here a work item is a tile of 64 / row_units tokens x 4 * U packed rows:
+// each wavefront load reads ONE (layer, head) run of 64 units (1 KiB: the tile's tokens are
+// consecutive on the layered side), the tile is laid out in LDS in packed order, and each wavefront
+// store writes 1 KiB of that order; per token the tile's rows are contiguous on the packed side
+// (4 * U rows). Nothing here is indexed per lane by division: layer and head are uniform over a
+// wavefront. Needs: 16-byte units, row_units a power of two <= 64, T a multiple of 64 / row_units,
+// L * H a multiple of 4 * U (plan_transpose_tiles checks). A workgroup runs load phase, barrier, store
+// phase, barrier per tile; the two phases are separate functions so that a CPU walk can do the same.
+struct TransposeTile {
+    uint64_t packed_addr;   // address of the pair's packed block
+    uint64_t layered_off;   // byte offset of the pair's block inside every layer's cache
+    uint32_t t0;            // first token of the tile
+    uint32_t r0;            // first packed row (l * H + h) of the tile
+};
+
+HFK_HD bool transpose_tile_item(const TransposeArgs& a, uint64_t w64, TransposeTile& it) {
+    const uint32_t w = (uint32_t)w64;
+    const uint32_t pair = w / a.chunks_per_block;
+    const uint32_t rem = w - pair * a.chunks_per_block;
+    const uint64_t pb = a.pairs ? (uint64_t)table_entry(a.pairs, 2 * (uint64_t)pair) : 0;
+    const uint64_t db = a.pairs ? (uint64_t)table_entry(a.pairs, 2 * (uint64_t)pair + 1) : 0;
+    if (pb >= a.packed_limit || db >= a.layered_limit) {
+        return false;
+    }
+    const uint32_t row_groups = (a.L * a.H) / a.tile_rows;   // row group fastest: a token group's tiles are neighbours
+    const uint32_t tg = rem / row_groups;
+    it.packed_addr = a.packed + pb * a.packed_stride;
+    it.layered_off = db * a.layered_stride;
+    it.t0 = tg * a.tile_tokens;
+    it.r0 = (rem - tg * row_groups) * a.tile_rows;
+    return true;
+}
+
+// Load phase: the lane's U units of the tile, from the layered side into `tile` (64 * 4 * U units, packed order).
+template <int U, int NT, typename LayerTable>
+HFK_HD void transpose_tile_load(const TransposeArgs& a, const TransposeTile& it, uint32_t tid, const LayerTable& layer_address,
+                                vec16* tile) {
+    constexpr uint32_t R = 4 * U;
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t tt = lane / a.row_units, col = lane - tt * a.row_units;
+    vec16 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t r = it.r0 + wave * U + u;     // uniform over the wavefront
+        const uint32_t l = r / a.H;
+        const uint32_t h = r - l * a.H;
+        const uint64_t addr = layer_address(l) + it.layered_off + (((uint64_t)h * a.T + it.t0) * a.row_units + lane) * sizeof(vec16);
+        if ((addr & (sizeof(vec16) - 1)) == 0) {
+            v[u] = load_unit<NT>(global_in<vec16>(addr));
+        } else {  // layer cache not aligned to the unit: byte loads keep it correct
+            unit_from_bytes(global_in<uint8_t>(addr), v[u]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        tile[(tt * R + wave * U + u) * a.row_units + col] = v[u];
+    }
+}
+
+// Store phase: the tile, in packed order, to the packed side: 1 KiB per wavefront store.
+template <int U, int NT>
+HFK_HD void transpose_tile_store(const TransposeArgs& a, const TransposeTile& it, uint32_t tid, const vec16* tile) {
+    const uint32_t wave = tid >> 6, lane = tid & 63u;
+    const uint32_t LH = a.L * a.H;
+    const uint32_t segment = 4 * U * a.row_units;   // units the tile holds per token, contiguous on the packed side
+    HFK_GLOBAL vec16* packed = global_out<vec16>(it.packed_addr);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t lin = (wave * U + u) * 64u + lane;
+        const uint32_t tt = lin / segment;
+        const uint32_t within = lin - tt * segment;
+        store_unit<NT>(packed + (((uint64_t)(it.t0 + tt) * LH + it.r0) * a.row_units + within), tile[lin]);
+    }
 }
 
 }  // namespace hfk

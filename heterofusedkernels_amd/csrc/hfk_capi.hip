@@ -16,6 +16,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <vector>
 #include <cctype>
 #include <cstdint>
 #include <cstdio>
@@ -49,12 +50,12 @@ __global__ __launch_bounds__(256) void swap_short_runs_kernel(const BlockCopyArg
 
 template <int UNROLL, int NT>
 __global__ __launch_bounds__(256) void gather_long_runs_kernel(const BlockCopyArgs<int64_t> a) {
-    hfk::block_copy_body<int64_t, UNROLL, NT, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    hfk::block_copy_body<int64_t, UNROLL, NT, true, false>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
 template <int UNROLL, int NT>
 __global__ __launch_bounds__(256) void scatter_long_runs_kernel(const BlockCopyArgs<int64_t> a) {
-    hfk::block_copy_body<int64_t, UNROLL, NT, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    hfk::block_copy_body<int64_t, UNROLL, NT, true, false>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
 template <int UNROLL, int NT>
@@ -64,17 +65,17 @@ __global__ __launch_bounds__(256) void swap_blocks_kernel(const BlockCopyArgs<in
 
 template <int UNROLL, int NT>
 __global__ __launch_bounds__(256) void gather_blocks_kernel(const BlockCopyArgs<int64_t> a) {
-    hfk::block_copy_body<int64_t, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    hfk::block_copy_body<int64_t, UNROLL, NT, false, false>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
 template <int UNROLL, int NT>
 __global__ __launch_bounds__(256) void scatter_blocks_kernel(const BlockCopyArgs<int64_t> a) {
-    hfk::block_copy_body<int64_t, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    hfk::block_copy_body<int64_t, UNROLL, NT, false, false>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
 template <typename IdT, int UNROLL, int NT>
 __global__ __launch_bounds__(256) void gather_rows_wide_kernel(const BlockCopyArgs<IdT> a) {
-    hfk::block_copy_body<IdT, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
+    hfk::block_copy_body<IdT, UNROLL, NT, false, false>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
 template <int UNROLL, int NT>
@@ -119,6 +120,26 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
     transpose_with_layer_table<V, UNROLL, NT, true>(a);
 }
 
+// The same toward the packed side, tiled through LDS (see transpose_tile_load): 1 KiB runs on both sides.
+template <int U, int NT>
+__global__ __launch_bounds__(256) void transpose_to_packed_tiled_kernel(const TransposeArgs a) {
+    __shared__ uint64_t layer_table[kLayerTableLdsEntries];
+    __shared__ vec16 tile[64 * 4 * U];
+    for (uint32_t l = threadIdx.x; l < a.L; l += 256) layer_table[l] = hfk::table_entry(a.layer_ptrs, l);
+    __syncthreads();
+    const LayerTableInLds layer_address{layer_table};
+    hfk::Pacer pacer(a.pace_q8, blockIdx.x, gridDim.x);
+    for (uint64_t w = blockIdx.x; w < a.n_work; w += gridDim.x) {
+        hfk::TransposeTile it;
+        if (!hfk::transpose_tile_item(a, w, it)) continue;   // uniform over the workgroup
+        pacer.wait_turn();
+        hfk::transpose_tile_load<U, NT>(a, it, threadIdx.x, layer_address, tile);
+        __syncthreads();
+        hfk::transpose_tile_store<U, NT>(a, it, threadIdx.x, tile);
+        __syncthreads();
+    }
+}
+
 // ---- tuning state ---------------------------------------------------------
 // Defaults are the measured best on MI355X:
 //  * HBM-bound launches (gathers, the staged swap's kernel): ONE 16-byte vector per lane, i.e. 4 KiB
@@ -140,7 +161,7 @@ __global__ __launch_bounds__(256) void transpose_to_packed_kernel(const Transpos
 // Every knob has a process-wide value (hfk_set_tuning) and, per thread, an optional override that
 // lasts from hfk_thread_tuning_begin to hfk_thread_tuning_end: a caller that wants a launch shape
 // of its own for a few calls changes nothing another thread can see.
-constexpr int kKnobCount = 17;
+constexpr int kKnobCount = 19;
 std::atomic<int64_t> g_knob[kKnobCount] = {
     1,       // HFK_KNOB_UNROLL
     3,       // HFK_KNOB_NONTEMPORAL
@@ -159,6 +180,8 @@ std::atomic<int64_t> g_knob[kKnobCount] = {
     890,     // HFK_KNOB_DUPLEX_PACE_PERMILLE
     0,       // HFK_KNOB_TRANSFER_PACE_PERMILLE
     8,       // HFK_KNOB_TRANSFER_UNROLL
+    0,       // HFK_KNOB_CHECK_HOST_COLUMN
+    1,       // HFK_KNOB_TRANSFER_TILED
 };
 
 struct ThreadTuning {
@@ -192,6 +215,8 @@ bool knob_value_valid(int k, int64_t v) {
         case HFK_KNOB_DUPLEX_PACE_PERMILLE:
         case HFK_KNOB_TRANSFER_PACE_PERMILLE: return v >= 0 && v <= 2000;
         case HFK_KNOB_TRANSFER_UNROLL: return v == 2 || v == 8;
+        case HFK_KNOB_CHECK_HOST_COLUMN:
+        case HFK_KNOB_TRANSFER_TILED: return v == 0 || v == 1;
         default: return false;
     }
 }
@@ -526,7 +551,24 @@ void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, bool to_p
         default: launch_transpose_u<V, hfk::kTransposeUnrollToHost>(a, grid, nt, to_packed, s); break;
     }
 }
+template <int U>
+void launch_transpose_tiled_u(const TransposeArgs& a, uint32_t grid, int nt, hipStream_t s) {
+    switch (nt & 3) {
+        case 0: hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 0>), dim3(grid), dim3(256), 0, s, a); break;
+        case 1: hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 1>), dim3(grid), dim3(256), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 2>), dim3(grid), dim3(256), 0, s, a); break;
+        default: hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 3>), dim3(grid), dim3(256), 0, s, a); break;
+    }
+}
 
+void launch_transpose_tiled(const TransposeArgs& a, uint32_t grid, int nt, int U, hipStream_t s) {
+    switch (U) {
+        case 8: launch_transpose_tiled_u<8>(a, grid, nt, s); break;
+        case 4: launch_transpose_tiled_u<4>(a, grid, nt, s); break;
+        case 2: launch_transpose_tiled_u<2>(a, grid, nt, s); break;
+        default: launch_transpose_tiled_u<1>(a, grid, nt, s); break;
+    }
+}
 
 // Where an address lives: 1 = host memory (pinned, device-mapped), 0 = device memory, -1 = the
 // runtime does not know the pointer.
@@ -567,6 +609,10 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
                                  packed_blocks, layered_blocks, T, L, H, D, elem_bytes, unroll);
     if (rc != 0) return rc;
     if (a.n_work == 0) return HFK_OK;  // nothing to move
+    int tiled_unroll = 0;
+    if (to_packed && side != 0 && knob_value(HFK_KNOB_TRANSFER_TILED) != 0) {
+        tiled_unroll = hfk::plan_transpose_tiles(a, unit, kLayerTableLdsEntries);
+    }
     if (workgroups == 0 && side != 0) {
         // One block (the reference's op: 4-64 MiB, over in 0.1-1.2 ms) is sized for speed alone; a
         // block table may run for many milliseconds beside other kernels and gets the smaller grid.
@@ -583,7 +629,8 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
         if (pace_mbps != 0) a.pace_q8 = pace_interval_q8((double)a.total_units * unit / a.chunks_per_block, grid, pace_mbps);
     }
     const int nt = (int)knob_value(HFK_KNOB_NONTEMPORAL);
-    if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, to_packed, unroll, s);
+    if (tiled_unroll != 0) launch_transpose_tiled(a, grid, nt, tiled_unroll, s);
+    else if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, to_packed, unroll, s);
     else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, to_packed, unroll, s);
     else launch_transpose_v<uint8_t>(a, grid, nt, to_packed, unroll, s);
     return finish_launch();
@@ -612,7 +659,7 @@ int launch_swap(const BlockCopyArgs<int64_t>& a, uint32_t flags, uint32_t workgr
                                  (uint32_t)knob_value(HFK_KNOB_THROUGHPUT_PACE_PERMILLE),
                                  (uint32_t)knob_value(HFK_KNOB_SWAP_PACE_MBPS)};
     const hfk::SwapShape shape =
-        hfk::choose_swap_shape(flags, bytes, wants_pace ? (uint32_t)current_link_mbps() : 0u, workgroups, tuning);
+        hfk::choose_swap_shape(flags, bytes, a.block_bytes, wants_pace ? (uint32_t)current_link_mbps() : 0u, workgroups, tuning);
     return launch_block_copy<Role::kSwapBlocks, int64_t>(a, shape.workgroups, s, shape.unroll, shape.pace_mbps,
                                                          shape.plain_stores);
 }
@@ -794,6 +841,7 @@ const char* hfk_status_string(int status) {
         case HFK_ERR_BAD_FLAGS: return "hfk: unknown flag bits";
         case HFK_ERR_STAGING_TOO_SMALL:
             return "hfk: transfer exceeds the library's static staging buffer (HFK_STATIC_STAGING_BYTES)";
+        case HFK_ERR_TABLE_MISMATCH: return "hfk: host_block_ids differs from the host column of block_pairs";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -972,6 +1020,16 @@ int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs
     if (n_planes == 0 || n_pairs == 0) return HFK_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool out = to_host != 0;
+    if (host_block_ids != nullptr && block_pairs != nullptr && knob_value(HFK_KNOB_CHECK_HOST_COLUMN) != 0) {
+        // Debugging aid: the two movers read the host column from two places; make sure they agree.
+        hipError_t e = hipStreamSynchronize(s);   // whatever uploads the table on this stream has finished
+        std::vector<int64_t> table(2 * n_pairs);
+        if (e == hipSuccess) e = hipMemcpy(table.data(), block_pairs, 2 * n_pairs * sizeof(int64_t), hipMemcpyDefault);
+        if (e != hipSuccess) return (int)e;
+        for (uint64_t j = 0; j < n_pairs; ++j) {
+            if (table[2 * j + (out ? 1 : 0)] != host_block_ids[j]) return HFK_ERR_TABLE_MISMATCH;
+        }
+    }
     const uint32_t side_flags = flags | (out ? HFK_SWAP_DST_HOST : HFK_SWAP_SRC_HOST);
     // The direct mover over the whole table: (src, dst) = (device, host) on the way out, (host, device) back.
     BlockCopyArgs<int64_t> direct;

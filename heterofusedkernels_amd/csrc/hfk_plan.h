@@ -28,14 +28,32 @@ constexpr int kFlatUnrollHost = 4;
 constexpr int kTransposeUnroll = 2;
 constexpr int kTransposeUnrollToHost = 8;
 
+// A block smaller than 256 * unroll vectors would leave lanes idle, so the unroll
+// is halved until one chunk fits inside the block (down to 1).
+inline int fit_unroll(uint64_t block_bytes, int unroll) {
+    while (unroll > 1 && (uint64_t)kWorkgroupLanes * 16u * (uint64_t)unroll > block_bytes) {
+        unroll >>= 1;
+    }
+    return unroll;
+}
+
 // ---- launch shape of a block-table swap -------------------------------------
 // What a swap launch looks like follows from what the caller says about it (flags), how much it
 // moves, and the link's rate; the rules live here, apart from the launching code, so that a CPU
 // test can pin them. Workgroups x 16-byte vectors per lane, the rate offered toward the host
 // (0 = unpaced), and whether the stores are plain (through the L2) or non-temporal (streamed). The
 // measurements behind each shape stand beside the tunables in hfk_capi.hip.
-constexpr uint32_t kToHostWorkgroups = 12;         // toward the host, throughput mode: 12 x 8, plain stores
+// Toward the host, throughput mode: unpaced, plain stores, 96 vectors per lane in flight over the grid.
+// Measured for blocks of 4 KiB to 128 KiB (256 MiB per launch): 12 x 8 56.6 GB/s, 24 x 4 56.5, 48 x 2
+// 56.2-56.5, 96 x 1 56.5, whichever of them the block size allows; half as much in flight 54.6-55.0,
+// twice as much no more. A block that does not divide into whole chunks gets 32 x 4 (72 KiB blocks:
+// 56.6 against 54.8 on 12 x 8), and no grid may be a multiple of the chunks per block when the last
+// chunk is short: the same workgroups would then draw the short chunks every time (12 workgroups,
+// chunks of 32 + 32 + 8 KiB: four of them idle most of the time).
+constexpr uint32_t kToHostVectorsInFlight = 96;
 constexpr int kToHostUnroll = 8;
+constexpr uint32_t kToHostRaggedWorkgroups = 32;
+constexpr int kToHostRaggedUnroll = 4;
 constexpr uint32_t kBesidePacedWorkgroups = 12;    // toward the host, beside compute: 12 x 1 paced at 0.84
 constexpr uint32_t kFromHostWorkgroups = 40;       // from the host: 40 x 1
 constexpr uint32_t kBesideFromHostWorkgroups = 24; // from the host, beside compute: 24 x 1
@@ -63,9 +81,26 @@ struct SwapShape {
     bool plain_stores;
 };
 
-// `workgroups` != 0 is the caller's own grid bound and is kept; `link_mbps` 0 = unknown.
-inline SwapShape choose_swap_shape(uint32_t flags, uint64_t bytes, uint32_t link_mbps, uint32_t workgroups,
-                                   const SwapTuning& t) {
+inline SwapShape to_host_shape(uint64_t block_bytes) {
+    int unroll = fit_unroll(block_bytes, kToHostUnroll);
+    uint32_t grid = kToHostVectorsInFlight / (uint32_t)unroll;
+    uint64_t chunk_bytes = (uint64_t)kWorkgroupLanes * 16u * (uint64_t)unroll;
+    if (block_bytes > chunk_bytes && block_bytes % chunk_bytes != 0) {
+        if (unroll > kToHostRaggedUnroll) {
+            unroll = kToHostRaggedUnroll;
+            grid = kToHostRaggedWorkgroups;
+            chunk_bytes = (uint64_t)kWorkgroupLanes * 16u * (uint64_t)unroll;
+        }
+        const uint64_t chunks = (block_bytes + chunk_bytes - 1) / chunk_bytes;
+        if (grid % chunks == 0) ++grid;
+    }
+    return SwapShape{grid, unroll, 0, true};
+}
+
+// `workgroups` != 0 is the caller's own grid bound and is kept; `link_mbps` 0 = unknown; `bytes` is what
+// the launch moves in all, `block_bytes` the size of one block.
+inline SwapShape choose_swap_shape(uint32_t flags, uint64_t bytes, uint64_t block_bytes, uint32_t link_mbps,
+                                   uint32_t workgroups, const SwapTuning& t) {
     const bool beside = (flags & HFK_SWAP_BESIDE_COMPUTE) != 0;
     if ((flags & HFK_SWAP_DST_HOST) != 0 && (beside || bytes >= kLongSwapBytes)) {
         uint32_t pace = 0;
@@ -75,7 +110,11 @@ inline SwapShape choose_swap_shape(uint32_t flags, uint64_t bytes, uint32_t link
             const uint32_t grid = beside ? kBesidePacedWorkgroups : t.paced_workgroups;
             return SwapShape{workgroups ? workgroups : grid, beside ? kFineUnroll : t.paced_unroll, pace, false};
         }
-        if (!beside) return SwapShape{workgroups ? workgroups : kToHostWorkgroups, kToHostUnroll, 0, true};
+        if (!beside) {
+            SwapShape shape = to_host_shape(block_bytes);
+            if (workgroups != 0) shape.workgroups = workgroups;
+            return shape;
+        }
     }
     if ((flags & HFK_SWAP_SRC_HOST) != 0) {
         const uint32_t grid = beside ? kBesideFromHostWorkgroups : kFromHostWorkgroups;
@@ -97,15 +136,6 @@ inline int link_mbps_from_sysfs(const char* speed_text, const char* width_text) 
     if (end == width_text || width <= 0 || width > 32) return -1;
     const double encoding = gts >= 8.0 ? 128.0 / 130.0 : 0.8;
     return (int)(gts * 1000.0 * (double)width * encoding / 8.0);
-}
-
-// A block smaller than 256 * unroll vectors would leave lanes idle, so the unroll
-// is halved until one chunk fits inside the block (down to 1).
-inline int fit_unroll(uint64_t block_bytes, int unroll) {
-    while (unroll > 1 && (uint64_t)kWorkgroupLanes * 16u * (uint64_t)unroll > block_bytes) {
-        unroll >>= 1;
-    }
-    return unroll;
 }
 
 // For launches with one workgroup per chunk (the HBM-bound gathers): the largest unroll of at
@@ -207,6 +237,29 @@ inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_
     a.n_work = (uint32_t)(chunks * n_pairs);
     *unit_out = unit;
     return HFK_OK;
+}
+
+// Turns a planned transfer (plan_transpose, 16-byte units) into its tiled form when the geometry allows
+// (see transpose_tile_load): picks the largest U of 8, 4, 2, 1 with L * H a multiple of 4 * U, sets the
+// tile fields, chunks_per_block (tiles per block) and n_work. Returns U, or 0 when the transfer has to
+// go the direct way (a is then unchanged). `max_layers`: what the kernel's layer table holds.
+inline int plan_transpose_tiles(TransposeArgs& a, uint32_t unit, uint32_t max_layers) {
+    if (unit != 16u || a.n_work == 0 || a.L > max_layers) return 0;
+    const uint32_t ru = a.row_units;
+    if (ru == 0 || ru > 64u || (ru & (ru - 1)) != 0) return 0;
+    const uint32_t tile_tokens = 64u / ru;
+    if (a.T % tile_tokens != 0) return 0;
+    const uint64_t LH = (uint64_t)a.L * a.H;
+    int U = 8;
+    while (U >= 1 && LH % (4u * (uint32_t)U) != 0) U >>= 1;
+    if (U < 1) return 0;
+    const uint64_t tiles = (uint64_t)(a.T / tile_tokens) * (LH / (4u * (uint32_t)U));
+    if (tiles * a.n_pairs > kU32Max) return 0;
+    a.tile_tokens = tile_tokens;
+    a.tile_rows = 4u * (uint32_t)U;
+    a.chunks_per_block = (uint32_t)tiles;
+    a.n_work = (uint32_t)(tiles * a.n_pairs);
+    return U;
 }
 
 // Argument checks + struct fill for the public block-table entry points.

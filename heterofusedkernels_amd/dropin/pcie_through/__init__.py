@@ -1,10 +1,11 @@
-import weakref
-
 from ._load import _load_opextension_so
 
 _load_opextension_so()
 
-_table_in_host = {}   # data_ptr of a plane pointer table -> whether its planes are host memory
+# plane_pointer_table() notes on the table it returns whether its planes are host memory, as an attribute
+# of that tensor object: the note lives and dies with the object, and a tensor that merely sits at the
+# same address later (or another view of the same storage) carries none.
+_SIDE_ATTR = "hfk_planes_in_host"
 
 # flags of torch.ops.pcie_through.swap_blocks (hfk.h: HFK_SWAP_*)
 SWAP_DST_HOST = 1        # the destination planes are host memory (swap-out)
@@ -41,10 +42,8 @@ def plane_pointer_table(planes, device):
             addrs.append(dev)
     table = torch.tensor(addrs, dtype=torch.int64).to(device)
     kinds = {bool(t.is_cuda) for t in planes}
-    if len(kinds) == 1:   # remembered for swap_blocks() below, for as long as the table lives
-        key = table.data_ptr()
-        _table_in_host[key] = not kinds.pop()
-        weakref.finalize(table, _table_in_host.pop, key, None)
+    if len(kinds) == 1:   # remembered for swap_blocks() below, on the table itself
+        setattr(table, _SIDE_ATTR, not kinds.pop())
     return table
 
 
@@ -56,9 +55,9 @@ def swap_blocks(dst_table, src_table, block_pairs, block_bytes, src_block_stride
     import torch
     if flags is None:
         flags = SWAP_BESIDE_COMPUTE if beside_compute else 0
-        if _table_in_host.get(dst_table.data_ptr()):
+        if getattr(dst_table, _SIDE_ATTR, None) is True:     # a table that carries no note names no side
             flags |= SWAP_DST_HOST
-        if _table_in_host.get(src_table.data_ptr()):
+        if getattr(src_table, _SIDE_ATTR, None) is True:
             flags |= SWAP_SRC_HOST
     torch.ops.pcie_through.swap_blocks(dst_table, src_table, block_pairs, block_bytes, src_block_stride,
                                        dst_block_stride, src_blocks, dst_blocks, workgroups, flags)

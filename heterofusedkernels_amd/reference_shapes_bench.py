@@ -24,7 +24,12 @@ import pcie_through  # noqa: F401
 from heterofusedkernels import memory
 
 
-def gather_table(rows, runs, out):
+PCIE5_X16_GBPS = 32.0 * 16 * (128.0 / 130.0) / 8.0
+
+
+def gather_table(rows, runs, out, batch_sizes=(16, 32, 64, 128, 256, 512, 1024), fill="randn"):
+    """fill: "randn" = N(0,1) rows like the reference's test; "bytes" = random 16-bit patterns, which fill
+    a 4 GiB table in seconds (rows are compared as bytes either way)."""
     dev = "cuda"
     dim = 512
     embed = memory.alloc_numa_pinned_tensor(rows * dim * 2).view(torch.float16).view(rows, dim)
@@ -32,8 +37,11 @@ def gather_table(rows, runs, out):
     chunk = 1 << 16
     for r0 in range(0, rows, chunk):        # every row distinct and non-zero
         r1 = min(rows, r0 + chunk)
-        embed[r0:r1] = torch.randn(r1 - r0, dim, generator=gen).to(torch.float16)
-    for bs in (16, 32, 64, 128, 256, 512, 1024):
+        if fill == "randn":
+            embed[r0:r1] = torch.randn(r1 - r0, dim, generator=gen).to(torch.float16)
+        else:
+            embed[r0:r1].view(torch.int16).random_(1, 32767, generator=gen)
+    for bs in batch_sizes:
         row = {"bs": bs}
         # torch CPU advanced index + H2D copy (tests/test_memcpy.py:18,23)
         ids = torch.randint(0, rows, (runs, bs), dtype=torch.int64, generator=gen)
@@ -77,11 +85,39 @@ def gather_table(rows, runs, out):
         assert torch.equal(dst10.cpu().view(torch.int16), embed[ids10[runs - 1]].view(torch.int16)), "gather mismatch"
         row["gather_combined_ms_per_batch"] = dt * 1e3 / 10
         row["gather_combined_GBps"] = bs * 10 * dim * 2 / dt / 1e9
+        row["gather_combined_frac_of_pcie5_x16"] = row["gather_combined_GBps"] / PCIE5_X16_GBPS
         out["gather"].append(row)
         print("gather bs=%4d: cpu+h2d %.3f ms (%.2f GB/s) | gather %.4f ms (%.2f GB/s) | combined %.4f ms/batch "
               "(%.2f GB/s)" % (bs, row["torch_cpu_index_h2d_ms"], row["torch_cpu_index_h2d_GBps"], row["gather_ms"],
                                row["gather_GBps"], row["gather_combined_ms_per_batch"], row["gather_combined_GBps"]),
               file=sys.stderr, flush=True)
+
+
+def gather_hbm_table(out, rows=1 << 20, n_ids=1 << 18, launches=50):
+    """The same row gather with the table in device memory: [rows, 512] fp16, n_ids random rows per call,
+    timed by one HIP event pair around `launches` calls; GB/s of HBM traffic (rows read + rows written + ids)."""
+    dev = "cuda"
+    dim = 512
+    gen = torch.Generator().manual_seed(1)
+    table = torch.randint(1, 32767, (rows, dim), dtype=torch.int16, device=dev).view(torch.float16)
+    ids = torch.randint(0, rows, (n_ids,), dtype=torch.int64, generator=gen).to(dev)
+    dst = torch.empty(n_ids, dim, dtype=torch.float16, device=dev)
+    for _ in range(3):
+        torch.ops.pcie_through.gather(table, dst, ids)
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(launches):
+        torch.ops.pcie_through.gather(table, dst, ids)
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / launches
+    assert torch.equal(dst.view(torch.int16), table.view(torch.int16).index_select(0, ids)), "gather mismatch"
+    traffic = 2 * n_ids * dim * 2 + 8 * n_ids
+    out["gather_hbm_table"] = {"rows": rows, "ids_per_call": n_ids, "row_bytes": dim * 2, "ms": ms,
+                               "traffic_GBps": traffic / (ms * 1e6), "frac_of_hbm_peak": traffic / (ms * 1e6) / 8000.0}
+    print("gather from an HBM table [%d, %d] fp16, %d ids per call: %.4f ms, %.0f GB/s of HBM traffic" %
+          (rows, dim, n_ids, ms, traffic / (ms * 1e6)), file=sys.stderr, flush=True)
 
 
 README_TRANSFER_SHAPES = ((1024, 32, 1, 128), (1024, 32, 8, 128), (1024, 64, 1, 128), (1024, 64, 8, 128))
@@ -131,6 +167,7 @@ def transfer_table(out, blocks=8, shapes=README_TRANSFER_SHAPES):
                 dev_blocks.zero_()   # the next leg must move the bytes itself
             row[name + "_ms"] = ms
             row[name + "_GBps"] = nbytes / (ms * 1e6)
+            row[name + "_frac_of_pcie5_x16"] = row[name + "_GBps"] / PCIE5_X16_GBPS
         # all blocks in one launch through the block table, host -> device and device -> host
         caches = torch.zeros(L, blocks, H, T, D, dtype=torch.int8, device=dev)
         lptrs = torch.tensor([caches[l].data_ptr() for l in range(L)], dtype=torch.int64).to(dev)
@@ -151,6 +188,7 @@ def transfer_table(out, blocks=8, shapes=README_TRANSFER_SHAPES):
             ms = s.elapsed_time(e) / 5
             row[name + "_ms"] = ms
             row[name + "_GBps"] = blocks * nbytes / (ms * 1e6)
+            row[name + "_frac_of_pcie5_x16"] = row[name + "_GBps"] / PCIE5_X16_GBPS
         got = caches.cpu()
         for b in range(blocks):
             assert torch.equal(got[:, blocks - 1 - b].permute(2, 0, 1, 3), host_blocks[b]), "table transfer mismatch"
@@ -216,18 +254,22 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--rows", type=int, default=4000000, help="embedding rows (reference: 4 000 000)")
     ap.add_argument("--runs", type=int, default=200)
-    ap.add_argument("--only", default="config1,gather,transfer", help="comma list of: config1, gather, transfer")
+    ap.add_argument("--only", default="config1,gather,gather_hbm,transfer",
+                    help="comma list of: config1, gather, gather_hbm, transfer")
+    ap.add_argument("--fill", default="randn", choices=["randn", "bytes"], help="how the gather's host table is filled")
     ap.add_argument("--transfer-shape", default=None,
                     help="one T,L,H,D instead of the README's four shapes (e.g. 1024,64,8,128), for profiling")
     args = ap.parse_args()
     assert torch.cuda.is_available()
     parts = set(args.only.split(","))
-    assert parts <= {"config1", "gather", "transfer"}, "unknown part in --only"
+    assert parts <= {"config1", "gather", "gather_hbm", "transfer"}, "unknown part in --only"
     out = {"gather": [], "transfer": [], "rows": args.rows, "runs": args.runs}
     if "config1" in parts:
         config1_latency(out)
     if "gather" in parts:
-        gather_table(args.rows, args.runs, out)
+        gather_table(args.rows, args.runs, out, fill=args.fill)
+    if "gather_hbm" in parts:
+        gather_hbm_table(out)
     if "transfer" in parts:
         shapes = README_TRANSFER_SHAPES
         if args.transfer_shape:

@@ -43,7 +43,8 @@ enum hfk_status {
     HFK_ERR_BAD_KNOB = -4,     /* unknown tuning knob or value out of range      */
     HFK_ERR_OUT_OF_RANGE = -5, /* an index passed in host memory is out of range */
     HFK_ERR_BAD_FLAGS = -6,    /* a flags argument has unknown bits set            */
-    HFK_ERR_STAGING_TOO_SMALL = -7 /* the transfer does not fit the library's static staging buffer */
+    HFK_ERR_STAGING_TOO_SMALL = -7, /* the transfer does not fit the library's static staging buffer */
+    HFK_ERR_TABLE_MISMATCH = -8 /* two forms of the same block table disagree (HFK_KNOB_CHECK_HOST_COLUMN) */
 };
 
 /* HFK_VERSION_MAJOR * 1000 + HFK_VERSION_MINOR of the loaded library. */
@@ -346,7 +347,8 @@ HFK_API int hfk_swap_blocks_staged_static(const void* dev_plane_ptrs, void* cons
  *   - Everything else goes the direct way, in one launch of the block-swap kernel that steps over
  *     the pairs the copy engines took.
  *   - With no staging buffer (NULL, or smaller than n_planes * n_pairs * block_bytes), or no host
- *     arrays, the whole table goes the direct way: exactly hfk_swap_blocks with the host side named.
+ *     arrays, the whole table goes the direct way: as hfk_swap_blocks with the host side named,
+ *     except that a device id out of range zero-fills its host slot on the way out.
  * k = min_run_blocks, or when that is 0 the smallest run whose single copy moves 16 MiB, with
  * HFK_SWAP_BESIDE_COMPUTE 4 MiB. A copy costs the DMA engines about 9.5 us before its first byte, the
  * link time of 0.5 MiB: runs of 16 MiB move at 97 % of the link rate, runs of 4 MiB at 88 %, single
@@ -361,9 +363,15 @@ HFK_API int hfk_swap_blocks_staged_static(const void* dev_plane_ptrs, void* cons
  *   block_pairs       device-visible int64 [n_pairs, 2] = (src_block, dst_block):
  *                     (device, host) when to_host != 0, (host, device) otherwise
  *   host_block_ids    HOST int64 [n_pairs]: the host column of block_pairs, read before the call
- *                     returns; may be NULL. It must equal that column: where the two disagree
- *                     blocks end up unmoved or moved twice (never outside the pools: both
- *                     copies are range-checked).
+ *                     returns; may be NULL. It must equal that column. The copy engines pick their
+ *                     runs from this array, the kernels theirs from block_pairs: where the two
+ *                     disagree blocks end up unmoved or moved twice, and a pair the array calls part
+ *                     of a long run but the table does not is copied from a staging slot this call
+ *                     never filled, so stale bytes of an earlier transfer reach the named host slot
+ *                     (never anything outside the pools: both movers are range-checked). Setting
+ *                     HFK_KNOB_CHECK_HOST_COLUMN makes the call compare the two first (it waits for
+ *                     `stream` and reads the table back: for debugging, not for production) and
+ *                     return HFK_ERR_TABLE_MISMATCH, with nothing enqueued, if they differ.
  *   dev_blocks / host_blocks  blocks per plane; 0 = unchecked. With host arrays present, a host id
  *                     out of range rejects the call (HFK_ERR_OUT_OF_RANGE) before anything is
  *                     enqueued. A device id out of range: skipped on the way in; on the way out
@@ -445,7 +453,13 @@ enum hfk_knob {
                                        HFK_SWAP_BESIDE_COMPUTE; 0 = unpaced; default 890                        */
     HFK_KNOB_TRANSFER_PACE_PERMILLE = 15, /* the same for a block-table transfer into a packed pool in host
                                        memory; 0 (default) = unpaced                                            */
-    HFK_KNOB_TRANSFER_UNROLL = 16   /* 16-byte units per lane of that transfer, 2 or 8 (default 8)              */
+    HFK_KNOB_TRANSFER_UNROLL = 16,  /* 16-byte units per lane of that transfer, 2 or 8 (default 8)              */
+    HFK_KNOB_TRANSFER_TILED = 18,   /* 1 (default): a block-table transfer into a packed pool in host memory goes through
+                                       LDS tiles where its geometry allows (1 KiB runs on both sides); 0: always
+                                       row by row                                                               */
+    HFK_KNOB_CHECK_HOST_COLUMN = 17 /* debugging aid, default 0: hfk_swap_blocks_auto first waits for its stream,
+                                       reads block_pairs back and compares its host column with host_block_ids;
+                                       a difference rejects the call with HFK_ERR_TABLE_MISMATCH                */
 };
 HFK_API int hfk_set_tuning(int knob, int64_t value);
 HFK_API int64_t hfk_get_tuning(int knob);

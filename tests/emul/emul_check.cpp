@@ -477,6 +477,34 @@ void walk_transpose(const TransposeArgs& a, uint32_t unit, uint32_t grid_cap) {
     else walk(a, grid, transpose_body<uint8_t, UNROLL, 0, TO_PACKED>);
 }
 
+// The tiled form toward the packed side: per tile every lane's load phase, then every lane's store phase,
+// with a host array standing in for LDS: what the kernel's two barriers order.
+template <int U>
+void walk_transpose_tiles_u(const TransposeArgs& a, uint32_t grid) {
+    std::vector<vec16> tile(64 * 4 * U);
+    for (uint32_t bid = 0; bid < grid; ++bid) {
+        for (uint64_t w = bid; w < a.n_work; w += grid) {
+            TransposeTile it;
+            if (!transpose_tile_item(a, w, it)) continue;
+            for (uint32_t tid = 0; tid < kWorkgroupLanes; ++tid)
+                transpose_tile_load<U, 3>(a, it, tid, LayerTableInMemory{a.layer_ptrs}, tile.data());
+            for (uint32_t tid = 0; tid < kWorkgroupLanes; ++tid) transpose_tile_store<U, 3>(a, it, tid, tile.data());
+        }
+    }
+}
+
+int g_tiled_walks = 0;
+void walk_transpose_tiles(const TransposeArgs& a, int U, uint32_t grid_cap) {
+    const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+    ++g_tiled_walks;
+    switch (U) {
+        case 8: walk_transpose_tiles_u<8>(a, grid); break;
+        case 4: walk_transpose_tiles_u<4>(a, grid); break;
+        case 2: walk_transpose_tiles_u<2>(a, grid); break;
+        default: walk_transpose_tiles_u<1>(a, grid); break;
+    }
+}
+
 // single block, the reference's op
 void case_transpose(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem, size_t s_mis, size_t l_mis,
                     uint32_t grid_cap) {
@@ -551,7 +579,10 @@ void case_transpose_table(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32
     const bool to_host_shape = to_packed && (to_packed_cases++ % 2 == 1);
     int rc = plan_transpose(a, &unit, lp.data(), packed.p, pairs.data(), n_pairs, ps, ls, packed_blocks, dev_blocks, T,
                             L, H, D, elem, to_host_shape ? kTransposeUnrollToHost : kTransposeUnroll);
+    // a pool in host memory goes through LDS tiles where the geometry allows
+    const int tiled = rc == HFK_OK && to_host_shape ? plan_transpose_tiles(a, unit, 512) : 0;
     if (rc != HFK_OK) { ++g_failures; std::printf("plan_transpose(table) rc=%d\n", rc); }
+    else if (tiled != 0) walk_transpose_tiles(a, tiled, grid_cap);
     else if (to_host_shape) walk_transpose<true, kTransposeUnrollToHost>(a, unit, grid_cap);
     else if (to_packed) walk_transpose<true>(a, unit, grid_cap);
     else walk_transpose<false>(a, unit, grid_cap);
@@ -577,6 +608,7 @@ void case_swap_shape() {
     paced.throughput_pace_permille = 890;         // ... unless the knob says so
     const uint32_t link = 63015, out = HFK_SWAP_DST_HOST, in = HFK_SWAP_SRC_HOST, beside = HFK_SWAP_BESIDE_COMPUTE;
     const uint64_t big = 512ull << 20, small = 2ull << 20;
+    const uint64_t bb = 32768;
     struct { const SwapTuning* tuning; uint32_t flags; uint64_t bytes; uint32_t link; uint32_t asked;
              uint32_t wg; int unroll; uint32_t pace; bool plain; const char* what; } rows[] = {
         {&t, 0, big, link, 0, 16, 8, 0, false, "nothing known: 16 x 8 unpaced"},
@@ -600,7 +632,7 @@ void case_swap_shape() {
         {&paced, out, big, link, 20, 20, 4, 56083, false, "pacing switched on, the caller's grid bound is kept"},
     };
     for (const auto& r : rows) {
-        const SwapShape got = choose_swap_shape(r.flags, r.bytes, r.link, r.asked, *r.tuning);
+        const SwapShape got = choose_swap_shape(r.flags, r.bytes, bb, r.link, r.asked, *r.tuning);
         ++g_cases;
         if (got.workgroups != r.wg || got.unroll != r.unroll || got.pace_mbps != r.pace || got.plain_stores != r.plain) {
             ++g_failures;
@@ -608,9 +640,29 @@ void case_swap_shape() {
                         got.workgroups, got.unroll, got.pace_mbps, (int)got.plain_stores, r.wg, r.unroll, r.pace, (int)r.plain);
         }
     }
+    // the unpaced shape toward the host by block size: 96 vectors per lane in flight, whole chunks or 32 x 4,
+    // never a grid that divides evenly into chunks of unequal size
+    struct { uint64_t block; uint32_t wg; int unroll; } by_block[] = {
+        {4096, 96, 1}, {8192, 48, 2}, {16384, 24, 4}, {32768, 12, 8}, {65536, 12, 8}, {131072, 12, 8},
+        {73728, 32, 4},          // 72 KiB: 16 + 16 + 16 + 16 + 8
+        {69632, 32, 4},          // 68 KiB
+        {20480, 25, 4},          // 20 KiB = 16 + 4: two chunks, and 24 workgroups would split evenly over them
+        {12288, 49, 2},          // 12 KiB = 8 + 4 on 48 x 2
+        {4112, 97, 1},           // 4 KiB + 16 B
+        {1024, 96, 1},           // smaller than one chunk
+    };
+    for (const auto& r : by_block) {
+        const SwapShape got = choose_swap_shape(out, big, r.block, link, 0, t);
+        ++g_cases;
+        if (got.workgroups != r.wg || got.unroll != r.unroll || got.pace_mbps != 0 || !got.plain_stores) {
+            ++g_failures;
+            std::printf("swap shape for %llu-byte blocks: got %u x %d, want %u x %d\n", (unsigned long long)r.block,
+                        got.workgroups, got.unroll, r.wg, r.unroll);
+        }
+    }
     SwapTuning forced = t;
     forced.beside_pace_mbps = 1;      // an explicit pace (the test of the bounded wait uses 1 MB/s)
-    const SwapShape s1 = choose_swap_shape(out | beside, small, 0, 0, forced);
+    const SwapShape s1 = choose_swap_shape(out | beside, small, bb, 0, 0, forced);
     ++g_cases;
     if (s1.workgroups != 12 || s1.unroll != 1 || s1.pace_mbps != 1) { ++g_failures; std::printf("swap shape: explicit pace\n"); }
 }
@@ -749,6 +801,21 @@ int main() {
         case_transpose_table(6, 2, 2, 16, 1, 3, 3, 2, 3, 5, 1, 3, to_packed, false, 5);        // everything odd
         case_transpose_table(64, 2, 1, 128, 1, 3, 3, 3, 0, 0, 0, 0, to_packed, false, 2);      // one-head blocks
     }
+    // toward the packed side twice each, so that both launch shapes meet every geometry: the second one
+    // goes through LDS tiles where T, L * H and the row size allow (rows of 16 B ... 1 KiB, 4 to 32 rows per tile)
+    for (int rep = 0; rep < 2; ++rep) {
+        case_transpose_table(16, 4, 8, 128, 1, 6, 5, 4, 0, 0, 0, 0, true, false, 7);       // 128-byte rows, L * H = 32: tiles of 8 tokens x 32 rows
+        case_transpose_table(16, 4, 2, 128, 1, 6, 5, 4, 0, 0, 0, 0, true, true, 1000);     // L * H = 8: 8 rows per tile, bad pairs
+        case_transpose_table(8, 3, 4, 64, 2, 5, 7, 5, 32, 64, 0, 0, true, false, 3);       // L * H = 12: 4 rows per tile, padded strides
+        case_transpose_table(128, 2, 2, 16, 1, 4, 4, 3, 0, 0, 0, 0, true, false, 5);       // 16-byte rows: 64 tokens per tile
+        case_transpose_table(3, 8, 2, 512, 2, 4, 4, 4, 0, 0, 0, 0, true, true, 9);         // 1 KiB rows: one token per tile, 16 rows
+        case_transpose_table(4, 2, 8, 256, 1, 3, 3, 3, 0, 0, 0, 4, true, false, 4);        // 256-byte rows, layer caches 4-byte aligned
+        case_transpose_table(12, 2, 2, 128, 1, 3, 3, 2, 0, 0, 0, 0, true, false, 5);       // T no multiple of 8: not tiled
+        case_transpose_table(16, 3, 1, 128, 1, 3, 3, 2, 0, 0, 0, 0, true, false, 5);       // L * H = 3: not tiled
+        case_transpose_table(16, 2, 2, 48, 1, 3, 3, 2, 0, 0, 0, 0, true, false, 5);        // 48-byte rows: not tiled
+    }
+    ++g_cases;
+    if (g_tiled_walks < 6) { ++g_failures; std::printf("only %d tiled walks: the tiled cases did not tile\n", g_tiled_walks); }
 
     // seeded random shapes on top of the hand-picked ones
     auto pick = [&](std::initializer_list<uint64_t> v) { return *(v.begin() + rng() % v.size()); };

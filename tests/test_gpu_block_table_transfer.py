@@ -184,3 +184,36 @@ def test_block_table_transfer_with_token_major_layer_caches(T, L, H, D, dtype):
     untouched = torch.ones(host_blocks, dtype=torch.bool)
     untouched[hb2] = False
     assert int(pool2.view(host_blocks, block_bytes)[untouched].abs().max()) == 0
+
+
+def test_more_layers_than_the_lds_copy_of_the_layer_table_holds():
+    """L = 513: one layer more than the kernels copy into LDS, so they read the layer addresses from the
+    device array instead. Both directions against the oracle, on a tiny geometry."""
+    T, L, H, D, e = 1, 513, 1, 48, 1
+    host_blocks, dev_blocks, n = 5, 6, 4
+    announce("block-table transfer with L=%d layers (layer table read from memory), both directions" % L)
+    block_bytes = T * L * H * D * e
+    stride = H * T * D * e
+    gen = torch.Generator().manual_seed(513)
+    pool = memory.alloc_numa_pinned_tensor(host_blocks * block_bytes)
+    pool.copy_(torch.randint(-128, 128, (host_blocks * block_bytes,), dtype=torch.int8, generator=gen))
+    host_pool = pool.view(host_blocks, T, L, H, D)
+    caches = torch.zeros(L, dev_blocks, H, T, D, dtype=torch.int8, device=DEV)
+    ptrs = torch.tensor([caches[l].data_ptr() for l in range(L)], dtype=torch.int64).to(DEV)
+    pairs = torch.stack([torch.randperm(host_blocks, generator=gen)[:n], torch.randperm(dev_blocks, generator=gen)[:n]], 1).contiguous()
+    torch.ops.pcie_through.multi_layer_block_table_transfer(ptrs, host_pool, pairs.to(DEV), stride, dev_blocks)
+    torch.cuda.synchronize()
+    want = np.zeros((L, dev_blocks, stride), dtype=np.uint8)
+    O.c_multi_layer_block_table_transfer(want, pool.view(torch.uint8).numpy().reshape(host_blocks, block_bytes),
+                                         pairs.numpy(), T, L, H, D, e, False)
+    assert np.array_equal(caches.cpu().view(torch.uint8).numpy().reshape(L, dev_blocks, stride), want)
+    # and back out, to other host slots
+    pool2 = memory.alloc_numa_pinned_tensor(host_blocks * block_bytes)
+    pool2.fill_(0x55)
+    pairs2 = torch.stack([torch.randperm(host_blocks, generator=gen)[:n], pairs[:, 1]], 1).contiguous()
+    torch.ops.pcie_through.multi_layer_block_table_transfer(ptrs, pool2.view(host_blocks, T, L, H, D), pairs2.to(DEV), stride,
+                                                            dev_blocks, True)
+    torch.cuda.synchronize()
+    want2 = np.full((host_blocks, block_bytes), 0x55, dtype=np.uint8)
+    O.c_multi_layer_block_table_transfer(want, want2, pairs2.numpy(), T, L, H, D, e, True)
+    assert np.array_equal(pool2.view(torch.uint8).numpy().reshape(host_blocks, block_bytes), want2)

@@ -572,7 +572,6 @@ def test_strided_planes():
 
 def test_python_swap_wrapper_names_the_host_side_by_itself(memory):
     """pcie_through.swap_blocks: the op with its flags read off tables that plane_pointer_table built."""
-    import gc
     announce("pcie_through.swap_blocks wrapper: out and back, flags inferred from the tables")
     planes, blocks, bb, n = 3, 40, 32768, 12
     gen = torch.Generator().manual_seed(321)
@@ -580,7 +579,7 @@ def test_python_swap_wrapper_names_the_host_side_by_itself(memory):
     pool = memory.alloc_numa_pinned_tensor(planes * blocks * bb)
     host = list(pool.view(torch.uint8).view(planes, blocks, bb).unbind(0))
     dtab, htab = pcie_through.plane_pointer_table(dev, DEV), pcie_through.plane_pointer_table(host, DEV)
-    assert pcie_through._table_in_host[htab.data_ptr()] is True and pcie_through._table_in_host[dtab.data_ptr()] is False
+    assert htab.hfk_planes_in_host is True and dtab.hfk_planes_in_host is False
     src, dst = torch.randperm(blocks, generator=gen)[:n], torch.randperm(blocks, generator=gen)[:n]
     before = [d.cpu() for d in dev]
     pcie_through.swap_blocks(htab, dtab, torch.stack([src, dst], 1).to(DEV), bb, bb, bb, blocks, blocks)
@@ -593,10 +592,15 @@ def test_python_swap_wrapper_names_the_host_side_by_itself(memory):
         want = before[p].clone()
         want[back] = before[p][src]
         assert torch.equal(dev[p].cpu(), want), "swap-in through the wrapper"
-    key = htab.data_ptr()
-    del htab
-    gc.collect()
-    assert key not in pcie_through._table_in_host          # the note goes when the table goes
+    # the note belongs to the table object: another tensor over the same storage carries none, and names no side
+    alias = htab.view(-1)
+    assert getattr(alias, "hfk_planes_in_host", None) is None
+    for p in range(planes):
+        host[p][dst] = 0
+    pcie_through.swap_blocks(alias, dtab, torch.stack([back, dst], 1).to(DEV), bb, bb, bb, blocks, blocks)
+    torch.cuda.synchronize()
+    for p in range(planes):
+        assert torch.equal(host[p][dst], dev[p].cpu()[back]), "swap-out through a table without a note"
 
 
 @pytest.mark.parametrize("args", [(), ("3", "40", "4112", "20"), ("64", "128", "32768", "64")],
