@@ -38,6 +38,7 @@ SWAP_DST_DEVICE = 16
 STATIC_STAGING_BYTES = 64 << 20
 ERR_STAGING_TOO_SMALL = -7
 ERR_TABLE_MISMATCH = -8
+ERR_STAGING_BUSY = -9
 
 
 class KnobValue(ctypes.Structure):

@@ -16,6 +16,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <mutex>
 #include <vector>
 #include <cctype>
 #include <cstdint>
@@ -225,6 +226,8 @@ constexpr uint32_t kBesideDuplexWorkgroups = 16;
 constexpr int kBesideDuplexUnroll = 2;
 constexpr uint32_t kBesideTransferWorkgroups = 16;
 constexpr uint32_t kTransferToHostWorkgroups = 32;
+constexpr uint32_t kShortTransferToHostWorkgroups = 64;
+constexpr uint64_t kShortTransferBytes = 128ull << 20;
 constexpr uint32_t kTransferFromHostWorkgroups = 24;
 constexpr uint32_t kSingleBlockTransferWorkgroups = 32;
 constexpr uint32_t kHostGatherWorkgroups = 64;
@@ -551,22 +554,19 @@ void launch_transpose_v(const TransposeArgs& a, uint32_t grid, int nt, bool to_p
         default: launch_transpose_u<V, hfk::kTransposeUnrollToHost>(a, grid, nt, to_packed, s); break;
     }
 }
+// The tiled kernel stores plainly (through the L2, which hands the link whole lines); `nt_loads` picks its loads.
 template <int U>
-void launch_transpose_tiled_u(const TransposeArgs& a, uint32_t grid, int nt, hipStream_t s) {
-    switch (nt & 3) {
-        case 0: hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 0>), dim3(grid), dim3(256), 0, s, a); break;
-        case 1: hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 1>), dim3(grid), dim3(256), 0, s, a); break;
-        case 2: hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 2>), dim3(grid), dim3(256), 0, s, a); break;
-        default: hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 3>), dim3(grid), dim3(256), 0, s, a); break;
-    }
+void launch_transpose_tiled_u(const TransposeArgs& a, uint32_t grid, bool nt_loads, hipStream_t s) {
+    if (nt_loads) hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 1>), dim3(grid), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((transpose_to_packed_tiled_kernel<U, 0>), dim3(grid), dim3(256), 0, s, a);
 }
 
-void launch_transpose_tiled(const TransposeArgs& a, uint32_t grid, int nt, int U, hipStream_t s) {
+void launch_transpose_tiled(const TransposeArgs& a, uint32_t grid, bool nt_loads, int U, hipStream_t s) {
     switch (U) {
-        case 8: launch_transpose_tiled_u<8>(a, grid, nt, s); break;
-        case 4: launch_transpose_tiled_u<4>(a, grid, nt, s); break;
-        case 2: launch_transpose_tiled_u<2>(a, grid, nt, s); break;
-        default: launch_transpose_tiled_u<1>(a, grid, nt, s); break;
+        case 8: launch_transpose_tiled_u<8>(a, grid, nt_loads, s); break;
+        case 4: launch_transpose_tiled_u<4>(a, grid, nt_loads, s); break;
+        case 2: launch_transpose_tiled_u<2>(a, grid, nt_loads, s); break;
+        default: launch_transpose_tiled_u<1>(a, grid, nt_loads, s); break;
     }
 }
 
@@ -595,12 +595,17 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     // With the packed side in host memory the PCIe link is the bound and a small grid does; an
     // unknown pointer gets the small grid too. Measured on the reference's four shapes, 8 blocks per
     // launch: host -> device (two units per lane) 56.0-57.0 GB/s on 16 workgroups, 57.1-57.6 on 24-36,
-    // 54.1-54.6 on 48-56 (a dip that repeats), 56.6-57.5 on 80-96; device -> host 52.2-53.2 on 48
-    // workgroups of two units per lane (49.9 on one shape in one run), 53.2-53.9 on 32 of eight: toward
-    // the host a workgroup that moves more per turn is offered to the link more evenly, as for the
-    // swap-out. (Pacing, which gains a swap-out 1-2 %, does not pay here: it gains 0.8 GB/s on the
-    // eight-head shapes and loses up to 3.5 on the one-head shapes, whose 128-byte rows come from 64
-    // different layer caches per chunk and fall behind any schedule.)
+    // 54.1-54.6 on 48-56 (a dip that repeats), 56.6-57.5 on 80-96.
+    // Device -> host, row by row (eight units per lane): 53.2-54.0 GB/s on 32 or more workgroups,
+    // whatever the store kind, against 55.3-56.9 when the rows are 256 bytes or longer: a wavefront
+    // load that fetches eight 128-byte rows from eight places makes the same kernel 2-3 GB/s slower
+    // on the link, although HBM serves either pattern five times faster than the link drains it (the
+    // link then takes 2 % more 64-byte write requests than the payload has lines, against 1.4 %; no
+    // difference in address translation: 0.05 % of the lookups miss either way). Through LDS tiles
+    // (1 KiB runs on both sides) with plain stores: 56.5-56.6 GB/s on 32 workgroups for transfers of
+    // 256 MiB and more (55.4 with non-temporal stores, 56.1 on 64 workgroups); short transfers want
+    // more workgroups to be over sooner (32 MiB: 54.2 on 32, 55.3 on 64; 64 MiB: 55.4 and 55.6).
+    // Pacing does not pay: at 0.895 of the link 55.3-55.9 on the long shapes and 50-52 on the short.
     const int side = packed_side == kAskRuntime ? memory_side(packed) : packed_side;
     const int unroll = to_packed && side != 0 ? (int)knob_value(HFK_KNOB_TRANSFER_UNROLL) : hfk::kTransposeUnroll;
     TransposeArgs a;
@@ -618,7 +623,8 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
         // block table may run for many milliseconds beside other kernels and gets the smaller grid.
         workgroups = pairs == nullptr ? kSingleBlockTransferWorkgroups
                      : beside_compute ? kBesideTransferWorkgroups
-                     : to_packed      ? kTransferToHostWorkgroups
+                     : to_packed      ? ((uint64_t)a.total_units * unit * n_pairs < kShortTransferBytes ? kShortTransferToHostWorkgroups
+                                                                                                       : kTransferToHostWorkgroups)
                                       : kTransferFromHostWorkgroups;
     }
     uint32_t grid = 0;
@@ -629,7 +635,7 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
         if (pace_mbps != 0) a.pace_q8 = pace_interval_q8((double)a.total_units * unit / a.chunks_per_block, grid, pace_mbps);
     }
     const int nt = (int)knob_value(HFK_KNOB_NONTEMPORAL);
-    if (tiled_unroll != 0) launch_transpose_tiled(a, grid, nt, tiled_unroll, s);
+    if (tiled_unroll != 0) launch_transpose_tiled(a, grid, (nt & 1) != 0, tiled_unroll, s);
     else if (unit == 16u) launch_transpose_v<vec16>(a, grid, nt, to_packed, unroll, s);
     else if (unit == 4u) launch_transpose_v<uint32_t>(a, grid, nt, to_packed, unroll, s);
     else launch_transpose_v<uint8_t>(a, grid, nt, to_packed, unroll, s);
@@ -804,6 +810,65 @@ int static_staging(void** out) {
     return HFK_OK;
 }
 
+// Every static call on a device shares that device's array, and two that overlap in time corrupt each
+// other's blocks without either noticing. Calls on one stream are ordered by the stream. For calls on
+// different streams the library remembers, per device, the stream of the last static call and an event
+// recorded behind it: a call that arrives on another stream while that event is still pending is
+// refused (HFK_ERR_STAGING_BUSY) instead of racing. A stream under capture is left alone (an event
+// recorded there belongs to the graph): callers that replay graphs order them themselves.
+struct StaticUse {
+    std::mutex lock;
+    hipEvent_t done = nullptr;     // created on the device's first static call, never destroyed
+    hipStream_t last_stream = nullptr;
+    bool pending = false;          // `done` was recorded and not yet seen complete
+};
+StaticUse g_static_use[kMaxDevices];
+
+// Before a static call enqueues anything. `*guarded` tells static_release whether to record.
+int static_acquire(hipStream_t s, int* dev_out, bool* guarded) {
+    *guarded = false;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return HFK_ERR_TOO_LARGE;
+    *dev_out = dev;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        return HFK_OK;
+    }
+    if (capture != hipStreamCaptureStatusNone) return HFK_OK;
+    StaticUse& u = g_static_use[dev];
+    std::lock_guard<std::mutex> hold(u.lock);
+    if (u.done == nullptr) {
+        e = hipEventCreateWithFlags(&u.done, hipEventDisableTiming);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (u.pending && u.last_stream != s) {
+        e = hipEventQuery(u.done);
+        if (e == hipErrorNotReady) {
+            (void)hipGetLastError();
+            return HFK_ERR_STAGING_BUSY;
+        }
+        if (e != hipSuccess) return (int)e;
+        u.pending = false;
+    }
+    *guarded = true;
+    return HFK_OK;
+}
+
+void static_release(hipStream_t s, int dev, bool guarded) {
+    if (!guarded) return;
+    StaticUse& u = g_static_use[dev];
+    std::lock_guard<std::mutex> hold(u.lock);
+    if (hipEventRecord(u.done, s) == hipSuccess) {
+        u.last_stream = s;
+        u.pending = true;
+    } else {
+        (void)hipGetLastError();
+    }
+}
+
 // A run of host slots is worth a DMA copy when one copy of it moves at least this much.
 constexpr uint64_t kDmaRunBytes = 16ull << 20;
 constexpr uint64_t kDmaRunBytesBesideCompute = 4ull << 20;
@@ -841,6 +906,8 @@ const char* hfk_status_string(int status) {
         case HFK_ERR_BAD_FLAGS: return "hfk: unknown flag bits";
         case HFK_ERR_STAGING_TOO_SMALL:
             return "hfk: transfer exceeds the library's static staging buffer (HFK_STATIC_STAGING_BYTES)";
+        case HFK_ERR_STAGING_BUSY:
+            return "hfk: the library's static staging buffer is still in use by a call on another stream";
         case HFK_ERR_TABLE_MISMATCH: return "hfk: host_block_ids differs from the host column of block_pairs";
         default: break;
     }
@@ -1005,9 +1072,15 @@ int hfk_swap_blocks_staged_static(const void* dev_plane_ptrs, void* const* host_
     void* staging = nullptr;
     int rc = static_staging(&staging);
     if (rc != 0) return rc;
-    return staged_swap(dev_plane_ptrs, host_plane_addrs, dev_block_ids, host_block_ids, n_planes, n_blocks, block_bytes,
-                       dev_block_stride, host_block_stride, dev_blocks, host_blocks, staging, to_host, workgroups,
-                       static_cast<hipStream_t>(stream));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int dev = 0;
+    bool guarded = false;
+    rc = static_acquire(s, &dev, &guarded);
+    if (rc != 0) return rc;
+    rc = staged_swap(dev_plane_ptrs, host_plane_addrs, dev_block_ids, host_block_ids, n_planes, n_blocks, block_bytes,
+                     dev_block_stride, host_block_stride, dev_blocks, host_blocks, staging, to_host, workgroups, s);
+    static_release(s, dev, guarded);   // also after a failure: part of the work may be enqueued
+    return rc;
 }
 
 int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs, void* const* host_plane_addrs,

@@ -44,6 +44,7 @@ enum hfk_status {
     HFK_ERR_OUT_OF_RANGE = -5, /* an index passed in host memory is out of range */
     HFK_ERR_BAD_FLAGS = -6,    /* a flags argument has unknown bits set            */
     HFK_ERR_STAGING_TOO_SMALL = -7, /* the transfer does not fit the library's static staging buffer */
+    HFK_ERR_STAGING_BUSY = -9,  /* the library's static staging buffer is in use by a call on another stream */
     HFK_ERR_TABLE_MISMATCH = -8 /* two forms of the same block table disagree (HFK_KNOB_CHECK_HOST_COLUMN) */
 };
 
@@ -320,7 +321,14 @@ HFK_API int hfk_swap_blocks_staged(const void* dev_plane_ptrs, void* const* host
  *   - n_planes * n_blocks * block_bytes must not exceed HFK_STATIC_STAGING_BYTES, else
  *     HFK_ERR_STAGING_TOO_SMALL and nothing is enqueued.
  *   - Every call on one GPU uses the same array: calls that overlap in time on one GPU (two
- *     streams, two threads) race on it. Calls on one stream are ordered and safe.
+ *     streams, two threads) would race on it. Calls on one stream are ordered and safe. A call that
+ *     arrives on another stream while the previous static call's work is still pending is refused
+ *     with HFK_ERR_STAGING_BUSY and enqueues nothing (the library keeps one event per device for
+ *     this, created on the first call: no device memory). What the library cannot see it cannot
+ *     refuse: replays of a captured graph that holds a static call, and calls from other processes'
+ *     copies of the library (each process has its own array), are the caller's to order.
+ *   - The array is part of the library's device image: every process that loads the library holds
+ *     HFK_STATIC_STAGING_BYTES of device memory on every GPU it uses, whether or not it ever calls this.
  *   - The array keeps the last call's blocks; nothing needs clearing between calls (every staging
  *     byte that reaches a destination was written by the same call first).
  *   - The first call on a device asks the runtime for that device's address of the array; make it

@@ -142,7 +142,9 @@ def test_gather_from_registered_host_table(memory, bs, id_dtype):
 def test_gather_from_reference_scale_host_table(memory):
     """The reference's own table: [4 000 000, 512] fp16 (4 GB) in registered host memory, int64 ids on
     the device, aiv=4 and default (pcieThrough/tests/test_gather.py:35-58), at batch sizes from its loop
-    (8 .. 2040 in steps of 8) and with random rows instead of its all-zero table."""
+    (8 .. 2040 in steps of 8), at the size of its combined call (ten batches of 2040 ids in one call,
+    default aiv: pcieThrough/tests/test_gather_combine.py:47-56; 20 MiB per call, which takes the grid
+    bound of a long gather out of host memory) and with random rows instead of its all-zero table."""
     rows, dim = 4000000, 512
     announce("host-table gather out of the reference's 4 000 000 x 512 fp16 table")
     embed = _pinned(memory, rows * dim * 2).view(torch.float16).view(rows, dim)
@@ -152,10 +154,10 @@ def test_gather_from_reference_scale_host_table(memory):
                               generator=torch.Generator(device=DEV).manual_seed(first))
         embed[first:first + part].view(torch.uint8).copy_(chunk)
     gen = torch.Generator().manual_seed(4000000)
-    for bs in (8, 16, 128, 1024, 2040):
+    for bs in (8, 16, 128, 1024, 2040, 20400):
         ids = torch.randint(0, rows, (bs,), generator=gen, dtype=torch.int64)
         ids[0], ids[-1] = 0, rows - 1                           # both ends of the table
-        for aiv in (4, None):
+        for aiv in ((None,) if bs == 20400 else (4, None)):
             dst = torch.zeros(bs, dim, dtype=torch.float16, device=DEV)
             torch.ops.pcie_through.gather(embed, dst, ids.to(DEV), aiv=aiv)
             torch.cuda.synchronize()

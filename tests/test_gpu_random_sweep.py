@@ -361,11 +361,13 @@ def test_random_swap_blocks_auto(seed):
         pairs_d = torch.from_numpy(pairs).to(DEV)
         staging = torch.full((max(n_planes * n * bb, 1),), 0xC3, dtype=torch.uint8, device=DEV)
         staging_bytes = staging.numel() if how != 2 else max(staging.numel() - 1, 0)
-        capi.check(capi.swap_blocks_auto(dtab.data_ptr(), htab.data_ptr(), host_addrs if how != 3 else None,
-                                         pairs_d.data_ptr(), host_ids.ctypes.data if how != 3 else None, n_planes, n, bb,
-                                         dstride, hstride, dev_blocks, host_blocks,
-                                         staging.data_ptr() if how != 1 else None, staging_bytes if how != 1 else 0,
-                                         int(to_host), min_run, flags, stream_handle()), "hfk_swap_blocks_auto")
+        # every other case with the debugging check that compares the table's host column with the host array
+        with capi.thread_tuning({capi.KNOB_CHECK_HOST_COLUMN: case % 2}):
+            capi.check(capi.swap_blocks_auto(dtab.data_ptr(), htab.data_ptr(), host_addrs if how != 3 else None,
+                                             pairs_d.data_ptr(), host_ids.ctypes.data if how != 3 else None, n_planes, n, bb,
+                                             dstride, hstride, dev_blocks, host_blocks,
+                                             staging.data_ptr() if how != 1 else None, staging_bytes if how != 1 else 0,
+                                             int(to_host), min_run, flags, stream_handle()), "hfk_swap_blocks_auto")
         torch.cuda.synchronize()
 
         def host_view(buf, p):
@@ -394,3 +396,40 @@ def test_random_swap_blocks_auto(seed):
                 assert np.array_equal(chk, _view(want_dev, doff, p, dev_blocks, dstride, bb))
         assert np.array_equal(host.now(), want_host), "host side"
         assert np.array_equal(dev.now(), want_dev), "device side"
+
+
+@pytest.mark.parametrize("to_host", [True, False])
+def test_auto_swap_refuses_a_host_array_that_differs_from_the_table(to_host):
+    """HFK_KNOB_CHECK_HOST_COLUMN: the host array of host slots and the device table's host column are two
+    copies of one thing; with the check on, a call whose copies differ returns HFK_ERR_TABLE_MISMATCH and
+    moves nothing; with it off (the default) the same call is accepted."""
+    rng = np.random.default_rng(99)
+    n_planes, dev_blocks, host_blocks, bb, n = 2, 12, 16, 4096, 8
+    announce("auto swap with the host-column check, to_host %s" % to_host)
+    dev = Arena(n_planes * dev_blocks * bb, False, rng)
+    host = Arena(n_planes * host_blocks * bb, True, rng)
+    dtab = _table(_planes(dev.addr, 0, n_planes, dev_blocks, bb))
+    htab = _table(_planes(host.addr, 0, n_planes, host_blocks, bb))
+    host_addrs = (ctypes.c_void_p * n_planes)(*[host.host_addr + p * host_blocks * bb for p in range(n_planes)])
+    host_ids = np.arange(4, 4 + n, dtype=np.int64)
+    dev_ids = rng.permutation(dev_blocks)[:n].astype(np.int64)
+    pairs_d = torch.from_numpy(np.stack([dev_ids, host_ids] if to_host else [host_ids, dev_ids], 1).astype(np.int64)).to(DEV)
+    staging = torch.zeros(n_planes * n * bb, dtype=torch.uint8, device=DEV)
+    wrong = host_ids.copy()
+    wrong[3] = 0                    # breaks the run the copy engines would take
+
+    def call(ids):
+        return capi.swap_blocks_auto(dtab.data_ptr(), htab.data_ptr(), host_addrs, pairs_d.data_ptr(), ids.ctypes.data, n_planes,
+                                     n, bb, bb, bb, dev_blocks, host_blocks, staging.data_ptr(), staging.numel(), int(to_host),
+                                     2, 0, stream_handle())
+
+    with capi.thread_tuning({capi.KNOB_CHECK_HOST_COLUMN: 1}):
+        rc = call(wrong)
+        assert rc == capi.ERR_TABLE_MISMATCH, rc
+        assert "host_block_ids" in capi.status_string(rc)
+        torch.cuda.synchronize()
+        assert np.array_equal(host.now(), host.before) and np.array_equal(dev.now(), dev.before), "a refused call moved bytes"
+        assert call(host_ids) == 0
+    torch.cuda.synchronize()
+    moved = dev.now() if not to_host else host.now()
+    assert not np.array_equal(moved, dev.before if not to_host else host.before)
