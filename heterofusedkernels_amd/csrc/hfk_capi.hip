@@ -141,6 +141,34 @@ __global__ __launch_bounds__(256) void transpose_to_packed_tiled_kernel(const Tr
     }
 }
 
+// Staging slots of a split table whose staging buffer holds only the long runs (see
+// hfk::fill_stage_slots, which states the result): one workgroup walks the table 256 pairs at a time,
+// marks the pairs in long runs, and numbers them with a running prefix sum.
+__global__ __launch_bounds__(256) void stage_slots_kernel(const int64_t* ids, uint32_t stride, uint32_t n, uint32_t min_run,
+                                                          int64_t* slots) {
+    __shared__ uint32_t scan[256];
+    __shared__ uint32_t carried;
+    const uint32_t tid = threadIdx.x;
+    if (tid == 0) carried = 0;
+    __syncthreads();
+    for (uint32_t base = 0; base < n; base += 256) {
+        const uint32_t j = base + tid;
+        const uint32_t is_long = j < n && hfk::run_length_capped(ids, stride, n, j, min_run) >= min_run ? 1u : 0u;
+        scan[tid] = is_long;
+        __syncthreads();
+        for (uint32_t step = 1; step < 256; step <<= 1) {     // inclusive scan over the workgroup
+            const uint32_t add = tid >= step ? scan[tid - step] : 0u;
+            __syncthreads();
+            scan[tid] += add;
+            __syncthreads();
+        }
+        if (j < n) slots[(uint64_t)j * stride] = is_long ? (int64_t)(carried + scan[tid] - 1u) : 0;
+        __syncthreads();
+        if (tid == 255) carried += scan[255];
+        __syncthreads();
+    }
+}
+
 // ---- tuning state ---------------------------------------------------------
 // Defaults are the measured best on MI355X:
 //  * HBM-bound launches (gathers, the staged swap's kernel): ONE 16-byte vector per lane, i.e. 4 KiB
@@ -152,12 +180,12 @@ __global__ __launch_bounds__(256) void transpose_to_packed_tiled_kernel(const Tr
 //    and stays below this one). A grid-stride loop over fewer workgroups loses 5-10 %, so the grid
 //    bound is high enough to stay inactive (CUs x 65536 workgroups).
 //  * non-temporal accesses: +15-20 % over plain ones (the data is touched once).
-//  * PCIe-bound swaps are flat from 16 to 128 workgroups (55.4-55.7 GB/s out, 57.0-57.4 in);
-//    what grows with the grid is the harm to kernels on other streams (a memory-bound
-//    neighbour runs 2.3-3x slower beside 16 workgroups, 4-5.7x beside 64), so a swap
-//    defaults to 16. For the same reason the duplex swap defaults to 32 workgroups (98.2 GB/s
+//  * PCIe-bound swaps about which nothing is known are flat from 16 to 128 workgroups (55.4-56.0
+//    GB/s out, 57.0-57.4 in); what grows with the grid is the harm to kernels on other streams (a
+//    memory-bound neighbour runs 2.3-3x slower beside 16 workgroups, 4-5.7x beside 64), so such a
+//    swap defaults to 16. For the same reason the duplex swap defaults to 32 workgroups (98.2 GB/s
 //    summed against 99.1 at 128, neighbours 1.1-1.6x slower instead of 2.8-2.9x), a block-table
-//    transfer out of host memory to 24 and one into host memory to 48 (see launch_transpose).
+//    transfer out of host memory to 24 and one into host memory to 32 (see launch_transpose).
 //
 // Every knob has a process-wide value (hfk_set_tuning) and, per thread, an optional override that
 // lasts from hfk_thread_tuning_begin to hfk_thread_tuning_end: a caller that wants a launch shape
@@ -236,10 +264,6 @@ constexpr uint64_t kAskTableSideBytes = 64ull << 10;
 // The duplex swap wants little in flight per workgroup: one vector per lane and direction
 // (unroll 8 loses 6 %). 32 workgroups reach 98.1-98.4 GB/s summed for 16, 32 and 72 KiB
 // blocks; 40-64 dip to 89-94, 96-192 are a flat 98-99.
-// Share of the link's raw rate, in thousandths, that a long throughput-mode launch offers toward the
-// host (0 = unpaced).
-// Explicit offered rate of a swap that runs beside compute, MB/s; 0 = derive it from the link.
-// PCIe link rate override, MB/s; -1 = read each device's link from sysfs on first use.
 
 // Launch shapes of a swap whose host side the caller has named. What a host-facing launch keeps in
 // flight beyond the link's bandwidth-delay product (about 64 KiB toward the host, 128 KiB from it)
@@ -256,23 +280,27 @@ constexpr uint64_t kAskTableSideBytes = 64ull << 10;
 //      24 x 1: 55.9 GB/s / 1.30x / 1.58x     40 x 1: 57.4 / 1.95x / 1.59x     16 x 4: 57.4 / 3.4x / 1.58x
 //    the copy's slowdown follows what is in flight, the GEMM's (1.5-1.6x) is what any resident kernel
 //    costs it (one wavefront that only sleeps: 1.50x).
-// Toward the host, throughput mode (HFK_KNOB_PACED_WORKGROUPS x HFK_KNOB_PACED_UNROLL, at
-// HFK_KNOB_THROUGHPUT_PACE_PERMILLE of the link). A paced launch has to hold its pace whatever the
-// block table looks like and whatever ran before it. A workgroup that is late starts its next item
-// at once, so a launch that has fallen behind offers more than its pace until it has caught up; at
-// 0.90 of the link, the most it accepts, it never does, and a link that is offered more than it
-// takes accepts less. Measured over eight address patterns (consecutive, strided, descending, runs
-// of 8, random; 12 launches each) and, in a process of their own, the four benchmark configurations:
+// Toward the host, throughput mode: unpaced by default, 96 vectors per lane in flight over the grid
+// (12 workgroups x 8 for blocks of 32 KiB and more, see hfk::to_host_shape) with non-temporal loads
+// and PLAIN stores: 56.6-56.7 GB/s on every kind of block table, 0.899 of the link's raw rate and 99 %
+// of what hipMemcpy reaches, against 55.9-56.2 with non-temporal stores (which reach the link as
+// 1.4 % more write requests than the payload has lines; plain ones go through the L2, which hands the
+// link whole lines). It is the fast shape, not the gentle one: a device copy / SDPA / GEMM on another
+// stream runs 5.9x / 2.9x / 4.0x slower meanwhile.
+// Paced (HFK_KNOB_THROUGHPUT_PACE_PERMILLE != 0: HFK_KNOB_PACED_WORKGROUPS x HFK_KNOB_PACED_UNROLL
+// with non-temporal stores) the same swap is gentler, 1.35x / 1.32x / 2.5x at 0.89 of the link on
+// 6 x 4, and was the default until its rate turned out to follow the machine: a paced launch holds
+// its schedule to 0.01 % (ran / allotted ticks in its pace report, on every machine tried), so it
+// delivers its offered rate times whatever that machine's 100 MHz counter really runs at, and 0.89
+// was 55.9 GB/s on one box, 55.5 on a second and 54.9 on a third, while the link's knee (0.905: 13 %
+// of the turns begin late, against 2 % at 0.89) leaves no room to offer more. An unpaced launch
+// depends on no clock. Measured while pacing was the default, over eight address patterns
+// (consecutive, strided, descending, runs of 8, random; 12 launches each):
 //   0.90: 16 x 1 53.2-56.5 GB/s by pattern, single launches down to 52.6; 6 x 4 56.4-56.6, single
 //         launches down to 50.7 and one benchmark run at 49.8; 32 x 1 55.6-56.6;
-//   0.89: every shape within 55.5-56.0 on every pattern; 6 x 4 56.0 on all eight (slowest launch
-//         55.95) and 55.5 / 56.0 / 55.5 / 56.0 on the configurations in every run; 16 x 1 55.5-56.0
-//         but 53.4 in one of three runs of configuration 2.
-// One percent of headroom is what makes the pace holdable, and 96 KiB in flight hold it where 64 KiB
-// do not always. What the steadier shape costs the kernels beside it (device copy / SDPA / GEMM):
-// 1.35x / 1.32x / 2.5x against 1.07x / 1.21x / 2.3x for 16 x 1; a swap that should be gentle says so
-// (HFK_SWAP_BESIDE_COMPUTE) and gets the fine shape at 0.84, which it holds on every pattern
-// (52.7-52.8 GB/s).
+//   0.89: every shape within 55.5-56.0 on every pattern; 6 x 4 56.0 on all eight.
+// A swap that should be gentle says so (HFK_SWAP_BESIDE_COMPUTE) and gets the fine shape at 0.84,
+// which it holds on every pattern (52.3-52.8 GB/s; 1.05x / 1.08x / 1.6x).
 // Share of the link's raw rate offered to host writes when pacing. 256-byte transaction payloads
 // cap the link at 0.90 of raw (56.8 of 63.0 GB/s measured, reached only by a paced grid); from 0.92
 // on throughput collapses to 0.84 and the neighbours' slowdown doubles. The closer to the cap, the
@@ -648,15 +676,17 @@ constexpr uint32_t kSwapFlagMask = HFK_SWAP_DST_HOST | HFK_SWAP_SRC_HOST | HFK_S
 
 int launch_swap(const BlockCopyArgs<int64_t>& a, uint32_t flags, uint32_t workgroups, uint64_t bytes, hipStream_t s) {
     // Toward the host the link accepts the most when it is offered what it can take (offering 1.5-2x
-    // its rate lowers what it accepts to 47-49 GB/s). A swap that shares the GPU offers 0.84 of the raw
-    // rate, one that owns it 0.89; should the link take less than assumed the launch degrades to an
-    // unpaced one. A paced launch starts its workgroups staggered over one interval and ends behind
-    // its schedule, which only a long one amortises (2 MiB: 71 us paced, 51 us unpaced; 32 MiB: 52.6
-    // against 54.5 GB/s; 64 MiB: 55.1 against 55.0; 128 MiB: 55.9 against 55.5), so a short
-    // throughput-mode swap stays unpaced. Without a usable pace (no host side named, or the link's rate
-    // unknown) a beside-compute swap gets a small unpaced grid (49.8 GB/s toward the host), and a swap
-    // about which nothing is known the shape that saturates the link either way (16 workgroups x 8
-    // vectors per lane: 55.4-56.0 GB/s out, 57.0-57.4 in).
+    // its rate lowers what it accepts to 47-49 GB/s). A swap that shares the GPU is paced at 0.84 of the
+    // raw rate; one that owns it runs unpaced on the shape that offers just enough (hfk::to_host_shape)
+    // unless pacing is switched on for it; should the link's rate be unknown a paced launch degrades
+    // to an unpaced one. A paced launch starts its workgroups staggered over one interval and ends
+    // behind its schedule, and the plain stores of the long unpaced shape only pay once the launch
+    // lasts (2 MiB: 50.5 us on 16 x 8 with non-temporal stores, 53.9 on 12 x 8 with plain ones; 32 MiB:
+    // 619 against 624 us; from 64 MiB on the plain-store shape wins, 256 MiB: 4816 against 4767 us), so
+    // a short throughput-mode swap runs as one about which nothing is known: the shape that saturates
+    // the link either way (16 workgroups x 8 vectors per lane: 55.4-56.0 GB/s out, 57.0-57.4 in).
+    // Without a usable pace (no host side named, or the link's rate unknown) a beside-compute swap gets
+    // a small unpaced grid (49.8 GB/s toward the host).
     const bool wants_pace = (flags & HFK_SWAP_DST_HOST) != 0;
     const hfk::SwapTuning tuning{(uint32_t)knob_value(HFK_KNOB_SWAP_WORKGROUPS),
                                  (int)knob_value(HFK_KNOB_SWAP_UNROLL),
@@ -679,8 +709,10 @@ struct HostLeg {
     uint64_t n_blocks;
     uint64_t block_bytes;
     uint64_t host_block_stride;
-    void* staging;                   // [n_planes][n_blocks][block_bytes] in device memory
+    void* staging;                   // [n_planes][n_blocks][block_bytes] in device memory, or, when compact,
     bool to_host;
+    bool compact = false;            // [n_planes][stage_plane_blocks][block_bytes]: the long runs only, in table order
+    uint64_t stage_plane_blocks = 0;
 };
 
 int check_host_leg(const HostLeg& h, uint64_t host_blocks) {
@@ -706,7 +738,8 @@ int check_host_leg(const HostLeg& h, uint64_t host_blocks) {
 // streams gains nothing (same-direction copies are executed one after the other: 45.1 GB/s either
 // way for 111 runs of 2-14 MiB; a copy costs its engine about 9.5 us before the first byte moves).
 int copy_host_runs(const HostLeg& h, uint64_t min_run, hipStream_t s) {
-    const uint64_t stage_pitch = h.n_blocks * h.block_bytes;
+    const uint64_t stage_pitch = (h.compact ? h.stage_plane_blocks : h.n_blocks) * h.block_bytes;
+    uint64_t staged_before = 0;      // pairs in long runs before the current run (compact staging: its first slot)
     hipError_t e = hipSuccess;
     // Copies `run_bytes` at host_off / stage_off for planes [p0, p0 + count), which are evenly spaced
     // by `pitch` bytes on the host (count == 1: a plain copy).
@@ -727,7 +760,8 @@ int copy_host_runs(const HostLeg& h, uint64_t min_run, hipStream_t s) {
         if (len < min_run || e != hipSuccess) return;
         hipStream_t cs = s;
         const uint64_t host_off = (uint64_t)h.host_block_ids[first] * h.host_block_stride;
-        const uint64_t stage_off = first * h.block_bytes;
+        const uint64_t stage_off = (h.compact ? staged_before : first) * h.block_bytes;
+        staged_before += len;
         const uint64_t run_bytes = len * h.block_bytes;
         if (h.host_block_stride == h.block_bytes) {
             // maximal groups of evenly spaced planes: one 2-D copy each
@@ -1113,11 +1147,14 @@ int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs
     if (rc != 0) return rc;
     direct.zero_skipped = out ? 1u : 0u;   // one rule for the whole table, whichever mover takes a pair
     const uint64_t total_bytes = (uint64_t)n_planes * n_pairs * block_bytes;
-    const bool can_stage = staging != nullptr && host_plane_addrs != nullptr && host_block_ids != nullptr &&
-                           staging_bytes / block_bytes / n_pairs >= n_planes;
+    // Staging the copy engines' share takes the host arrays and a buffer. One that holds the whole table
+    // ([n_planes][n_pairs] blocks) is used with pair j in slot j. A smaller one is used compactly if it
+    // holds the blocks of the long runs and, behind them, a table of their slots (16 bytes per pair).
+    const bool have_arrays = staging != nullptr && host_plane_addrs != nullptr && host_block_ids != nullptr;
+    const bool holds_table = have_arrays && staging_bytes / block_bytes / n_pairs >= n_planes;
     uint64_t min_run = min_run_blocks;
     uint64_t long_blocks = 0;
-    if (can_stage) {
+    if (have_arrays) {
         const HostLeg probe{host_plane_addrs, host_block_ids, n_planes, n_pairs, block_bytes, host_block_stride, staging,
                             out};
         rc = check_host_leg(probe, host_blocks);
@@ -1134,17 +1171,35 @@ int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs
         }
         if (min_run <= kMaxRunFilter) long_blocks = hfk::blocks_in_long_runs(host_block_ids, n_pairs, min_run);
     }
+    bool compact = false;
+    uint64_t slots_offset = 0;
+    if (long_blocks != 0 && !holds_table) {
+        if (long_blocks < n_pairs && long_blocks <= staging_bytes / block_bytes / n_planes) {
+            slots_offset = (n_planes * long_blocks * block_bytes + 255u) & ~(uint64_t)255u;
+            compact = slots_offset <= staging_bytes && n_pairs <= (staging_bytes - slots_offset) / (2 * sizeof(int64_t));
+        }
+        if (!compact) long_blocks = 0;   // the buffer is too small for this table's long runs: everything goes direct
+    }
     if (long_blocks == 0) {   // nothing for the copy engines (or no staging to give them): one direct launch
         return launch_swap(direct, side_flags, 0, total_bytes, s);
     }
-    const HostLeg leg{host_plane_addrs, host_block_ids, n_planes, n_pairs, block_bytes, host_block_stride, staging, out};
+    HostLeg leg{host_plane_addrs, host_block_ids, n_planes, n_pairs, block_bytes, host_block_stride, staging, out};
+    leg.compact = compact;
+    leg.stage_plane_blocks = long_blocks;
     const int64_t* host_column = block_pairs + (out ? 1 : 0);
     const int64_t* dev_column = block_pairs + (out ? 0 : 1);
+    int64_t* slots = compact ? reinterpret_cast<int64_t*>(static_cast<char*>(staging) + slots_offset) : nullptr;
     BlockCopyArgs<int64_t> hbm;   // long runs: device planes <-> staging, the copy engines do the rest
     rc = hfk::plan_stage_blocks(hbm, dev_plane_ptrs, staging, dev_column, n_planes, n_pairs, block_bytes,
-                                dev_block_stride, dev_blocks, out);
+                                dev_block_stride, dev_blocks, out, slots, long_blocks);
     if (rc != 0) return rc;
     hbm.id_stride = 2;
+    if (compact) {   // the slot table, with the block table's stride, computed on the device from the device's table
+        hipLaunchKernelGGL(stage_slots_kernel, dim3(1), dim3(256), 0, s, host_column, 2u, (uint32_t)n_pairs, (uint32_t)min_run,
+                           slots);
+        rc = finish_launch();
+        if (rc != 0) return rc;
+    }
     const bool split = long_blocks < n_pairs;
     if (split) {
         hfk::filter_runs(hbm, hfk::kLongRunsOnly, host_column, (uint32_t)min_run);

@@ -43,17 +43,19 @@ inline int fit_unroll(uint64_t block_bytes, int unroll) {
 // test can pin them. Workgroups x 16-byte vectors per lane, the rate offered toward the host
 // (0 = unpaced), and whether the stores are plain (through the L2) or non-temporal (streamed). The
 // measurements behind each shape stand beside the tunables in hfk_capi.hip.
-// Toward the host, throughput mode: unpaced, plain stores, 96 vectors per lane in flight over the grid.
-// Measured for blocks of 4 KiB to 128 KiB (256 MiB per launch): 12 x 8 56.6 GB/s, 24 x 4 56.5, 48 x 2
-// 56.2-56.5, 96 x 1 56.5, whichever of them the block size allows; half as much in flight 54.6-55.0,
-// twice as much no more. A block that does not divide into whole chunks gets 32 x 4 (72 KiB blocks:
-// 56.6 against 54.8 on 12 x 8), and no grid may be a multiple of the chunks per block when the last
-// chunk is short: the same workgroups would then draw the short chunks every time (12 workgroups,
-// chunks of 32 + 32 + 8 KiB: four of them idle most of the time).
-constexpr uint32_t kToHostVectorsInFlight = 96;
+// Toward the host, throughput mode: unpaced, plain stores, and a grid that keeps 96-128 vectors per lane
+// in flight: 12 x 8 for blocks of 32 KiB and more, 32 x 4, 64 x 2 or 96 x 1 for smaller ones. Measured
+// for blocks of 4 KiB to 128 KiB on random tables (256 MiB per launch): 12 x 8 56.6 GB/s, 32 x 4
+// 56.5-56.6 (24 x 4 56.3-56.5, and 55.9 against 56.6 on a table of fragmented runs of 16 KiB blocks),
+// 64 x 2 56.4-56.6, 96 x 1 56.5; half as much in flight 54.6-55.5, twice as much no more. A block that
+// does not divide into whole chunks gets 32 x 4 (72 KiB blocks: 56.6 against 54.8 on 12 x 8), and no
+// grid may be a multiple of the chunks per block when the last chunk is short: the same workgroups
+// would then draw the short chunks every time (12 workgroups, chunks of 32 + 32 + 8 KiB: four of them
+// idle most of the time).
 constexpr int kToHostUnroll = 8;
 constexpr uint32_t kToHostRaggedWorkgroups = 32;
 constexpr int kToHostRaggedUnroll = 4;
+inline uint32_t to_host_workgroups(int unroll) { return unroll >= 8 ? 12u : unroll == 4 ? 32u : unroll == 2 ? 64u : 96u; }
 constexpr uint32_t kBesidePacedWorkgroups = 12;    // toward the host, beside compute: 12 x 1 paced at 0.84
 constexpr uint32_t kFromHostWorkgroups = 40;       // from the host: 40 x 1
 constexpr uint32_t kBesideFromHostWorkgroups = 24; // from the host, beside compute: 24 x 1
@@ -83,7 +85,7 @@ struct SwapShape {
 
 inline SwapShape to_host_shape(uint64_t block_bytes) {
     int unroll = fit_unroll(block_bytes, kToHostUnroll);
-    uint32_t grid = kToHostVectorsInFlight / (uint32_t)unroll;
+    uint32_t grid = to_host_workgroups(unroll);
     uint64_t chunk_bytes = (uint64_t)kWorkgroupLanes * 16u * (uint64_t)unroll;
     if (block_bytes > chunk_bytes && block_bytes % chunk_bytes != 0) {
         if (unroll > kToHostRaggedUnroll) {
@@ -337,9 +339,14 @@ inline int plan_gather_blocks(BlockCopyArgs<int64_t>& a, const void* dst_plane_p
 // The kernel half of a staged swap: blocks between the device planes and a
 // contiguous staging buffer [n_planes][n_blocks][block_bytes] in device memory.
 // to_staging: staging[p][i] = plane_p[ids[i]]  (gather);  else  plane_p[ids[i]] = staging[p][i]  (scatter).
+// `stage_slots` null: pair j's blocks live in staging slot j and a plane of the staging buffer holds
+// n_blocks slots. Otherwise pair j's slot is stage_slots[j * stride] (the caller sets a.id_stride: the
+// slot table is laid out with the stride of the block table it belongs to) and a plane holds
+// `stage_plane_blocks` slots: a staging buffer that holds only the share of the table that is staged.
 inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_ptrs, void* staging,
                              const int64_t* dev_block_ids, uint32_t n_planes, uint64_t n_blocks, uint64_t block_bytes,
-                             uint64_t dev_block_stride, uint64_t dev_blocks, bool to_staging) {
+                             uint64_t dev_block_stride, uint64_t dev_blocks, bool to_staging,
+                             const int64_t* stage_slots = nullptr, uint64_t stage_plane_blocks = 0) {
     if (dev_plane_ptrs == nullptr || staging == nullptr || dev_block_ids == nullptr) return HFK_ERR_NULL_POINTER;
     if (block_bytes == 0 || dev_block_stride < block_bytes) return HFK_ERR_BAD_SIZE;
     if (n_blocks > kU32Max) return HFK_ERR_TOO_LARGE;
@@ -355,7 +362,8 @@ inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_pt
         a.src_stride = dev_block_stride;
         a.src_limit = limit;
         a.dst_base = (uint64_t)(uintptr_t)staging;
-        a.dst_plane_stride = n_blocks * block_bytes;
+        a.dst_ids = stage_slots;
+        a.dst_plane_stride = (stage_slots ? stage_plane_blocks : n_blocks) * block_bytes;
         a.dst_stride = block_bytes;
         a.dst_limit = kUnchecked;
         // The copies that follow move staging[p][i] to the host whatever ids[i] was (the ids live on the
@@ -368,7 +376,8 @@ inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_pt
         a.dst_stride = dev_block_stride;
         a.dst_limit = limit;
         a.src_base = (uint64_t)(uintptr_t)staging;
-        a.src_plane_stride = n_blocks * block_bytes;
+        a.src_ids = stage_slots;
+        a.src_plane_stride = (stage_slots ? stage_plane_blocks : n_blocks) * block_bytes;
         a.src_stride = block_bytes;
         a.src_limit = kUnchecked;
     }
@@ -398,6 +407,22 @@ inline uint64_t blocks_in_long_runs(const int64_t* ids, uint64_t n, uint64_t min
         if (len >= min_run) total += len;
     });
     return total;
+}
+
+// Staging slots of a split table whose staging buffer holds only the long runs: pair j of a long run
+// gets slot (number of pairs in long runs before j), written to slots[j * stride]; the entries of
+// other pairs are set to 0 and never used. The sequential statement of what stage_slots_kernel
+// computes in parallel; the copy engines' leg counts the same way as it walks the runs.
+inline void fill_stage_slots(const int64_t* ids, uint32_t stride, uint64_t n, uint64_t min_run, int64_t* slots) {
+    uint64_t next = 0;
+    uint64_t first = 0;
+    while (first < n) {
+        uint64_t len = 1;
+        while (first + len < n && ids[(first + len) * stride] == ids[(first + len - 1) * stride] + 1) ++len;
+        for (uint64_t i = 0; i < len; ++i) slots[(first + i) * stride] = len >= min_run ? (int64_t)(next + i) : 0;
+        if (len >= min_run) next += len;
+        first += len;
+    }
 }
 
 // Restricts a planned block copy to the pairs in long (or short) runs of `run_ids`

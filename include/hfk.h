@@ -354,9 +354,9 @@ HFK_API int hfk_swap_blocks_staged_static(const void* dev_plane_ptrs, void* cons
  *     one 2-D DMA copy per run. Kernels on other streams do not notice them.
  *   - Everything else goes the direct way, in one launch of the block-swap kernel that steps over
  *     the pairs the copy engines took.
- *   - With no staging buffer (NULL, or smaller than n_planes * n_pairs * block_bytes), or no host
- *     arrays, the whole table goes the direct way: as hfk_swap_blocks with the host side named,
- *     except that a device id out of range zero-fills its host slot on the way out.
+ *   - With no staging buffer, no host arrays, or a buffer too small for what would be staged, the
+ *     whole table goes the direct way: as hfk_swap_blocks with the host side named, except that a
+ *     device id out of range zero-fills its host slot on the way out.
  * k = min_run_blocks, or when that is 0 the smallest run whose single copy moves 16 MiB, with
  * HFK_SWAP_BESIDE_COMPUTE 4 MiB. A copy costs the DMA engines about 9.5 us before its first byte, the
  * link time of 0.5 MiB: runs of 16 MiB move at 97 % of the link rate, runs of 4 MiB at 88 %, single
@@ -384,7 +384,11 @@ HFK_API int hfk_swap_blocks_staged_static(const void* dev_plane_ptrs, void* cons
  *                     out of range rejects the call (HFK_ERR_OUT_OF_RANGE) before anything is
  *                     enqueued. A device id out of range: skipped on the way in; on the way out
  *                     its host slot receives zeros, whichever mover had the pair.
- *   staging           device buffer, or NULL; staging_bytes its size
+ *   staging           device buffer (256-byte aligned), or NULL; staging_bytes its size.
+ *                     n_planes * n_pairs * block_bytes always suffices. A smaller buffer is used when
+ *                     it holds the staged share alone: n_planes * (blocks in runs of k or more) *
+ *                     block_bytes, rounded up to 256, plus 16 bytes per pair for the table of staging
+ *                     slots, which a one-workgroup kernel of the same call fills from block_pairs
  *   flags             0 or HFK_SWAP_BESIDE_COMPUTE (shape of the direct launch, see hfk_swap_blocks;
  *                     the host side is named by to_host)
  * All work is enqueued on `stream` in order. Destination blocks must be distinct.

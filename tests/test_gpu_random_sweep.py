@@ -324,8 +324,8 @@ def _run_table(rng, n, blocks):
 @pytest.mark.parametrize("seed", range(3))
 def test_random_swap_blocks_auto(seed):
     """The run-splitting swap against the oracle: fragmented host slots, every threshold from "stage
-    everything" to "stage nothing", with and without a staging buffer, padded strides (2-D copies per
-    plane), planes that are not evenly spaced on the host, bad device ids."""
+    everything" to "stage nothing", with and without a staging buffer, with a buffer that holds the long runs
+    only, padded strides (2-D copies per plane), planes that are not evenly spaced on the host, bad device ids."""
     rng = np.random.default_rng(5000 + seed + 17 * SEED_OFFSET)
     for case in range(CASES):
         n_planes = int(rng.integers(1, 7))
@@ -342,7 +342,11 @@ def test_random_swap_blocks_auto(seed):
             dev_ids[rng.integers(0, n, 2)] = np.array([-1, dev_blocks], dtype=np.int64)[rng.integers(0, 2, 2)]
         ok = (dev_ids >= 0) & (dev_ids < dev_blocks)
         min_run = int(rng.choice([0, 1, 2, 3, 4, 7, 5000]))
-        how = int(rng.integers(0, 4))       # 0: full arguments, 1: no staging, 2: staging too small, 3: no host arrays
+        # 0: full arguments, 1: no staging, 2: staging one byte short of the whole table (used compactly if the long
+        # runs and their slot table fit), 3: no host arrays, 4: staging of exactly the compact size
+        how = int(rng.integers(0, 5))
+        if how == 4:
+            min_run = int(rng.choice([2, 3, 4]))
         flags = int(rng.choice([0, capi.SWAP_BESIDE_COMPUTE]))
         plane_gap = int(rng.choice([0, 0, 64]))       # != 0: the last plane sits off the even spacing
         announce("random auto seed %d case %d: %d planes, blocks %d/%d, %d B (strides %d/%d, offsets %d/%d), %d pairs, "
@@ -359,8 +363,16 @@ def test_random_swap_blocks_auto(seed):
         host_addrs = (ctypes.c_void_p * n_planes)(*[host.host_addr + o for o in host_offsets])
         pairs = np.stack([dev_ids, host_ids] if to_host else [host_ids, dev_ids], 1).astype(np.int64)
         pairs_d = torch.from_numpy(pairs).to(DEV)
-        staging = torch.full((max(n_planes * n * bb, 1),), 0xC3, dtype=torch.uint8, device=DEV)
-        staging_bytes = staging.numel() if how != 2 else max(staging.numel() - 1, 0)
+        guard = 4096
+        staging = torch.full((max(n_planes * n * bb, 1) + 16 * n + 256 + guard,), 0xC3, dtype=torch.uint8, device=DEV)
+        staging_bytes = n_planes * n * bb if how != 2 else max(n_planes * n * bb - 1, 0)
+        if how == 4:      # the blocks of the long runs, rounded up to 256 bytes, and 16 bytes per pair for their slots
+            run_len = np.ones(n, dtype=np.int64)
+            starts = np.flatnonzero(np.r_[True, host_ids[1:] != host_ids[:-1] + 1])
+            for first, last in zip(starts, np.r_[starts[1:], n]):
+                run_len[first:last] = last - first
+            long_blocks = int((run_len >= min_run).sum())
+            staging_bytes = (n_planes * long_blocks * bb + 255) // 256 * 256 + 16 * n
         # every other case with the debugging check that compares the table's host column with the host array
         with capi.thread_tuning({capi.KNOB_CHECK_HOST_COLUMN: case % 2}):
             capi.check(capi.swap_blocks_auto(dtab.data_ptr(), htab.data_ptr(), host_addrs if how != 3 else None,
@@ -369,6 +381,9 @@ def test_random_swap_blocks_auto(seed):
                                              staging.data_ptr() if how != 1 else None, staging_bytes if how != 1 else 0,
                                              int(to_host), min_run, flags, stream_handle()), "hfk_swap_blocks_auto")
         torch.cuda.synchronize()
+        assert bool((staging[staging_bytes:] == 0xC3).all()), "staging was written beyond the size given"
+        if how == 4 and 0 < long_blocks < n:      # the compact buffer was used, not passed over for the direct way
+            assert not bool((staging[:n_planes * long_blocks * bb] == 0xC3).all()), "compact staging went unused"
 
         def host_view(buf, p):
             return np.lib.stride_tricks.as_strided(buf[host_offsets[p]:], shape=(host_blocks, bb), strides=(hstride, 1),
