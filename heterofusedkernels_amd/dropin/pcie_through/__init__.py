@@ -51,7 +51,7 @@ def swap_blocks(dst_table, src_table, block_pairs, block_bytes, src_block_stride
                 dst_blocks=0, workgroups=None, flags=None, beside_compute=False):
     """``torch.ops.pcie_through.swap_blocks`` with the flags filled in: for tables that came from
     ``plane_pointer_table`` the side that is host memory is known and named, so the launch is sized
-    and paced for the PCIe link instead of guessing. ``flags`` given explicitly are passed through."""
+    for the PCIe link instead of guessing. ``flags`` given explicitly are passed through."""
     import torch
     if flags is None:
         flags = SWAP_BESIDE_COMPUTE if beside_compute else 0
@@ -65,7 +65,7 @@ def swap_blocks(dst_table, src_table, block_pairs, block_bytes, src_block_stride
 
 def swap_flags(dst_planes, src_planes, beside_compute=False):
     """The ``flags`` argument of ``swap_blocks`` for these two plane lists: names the side that is
-    host memory (so the launch is sized and paced for the PCIe link instead of guessing) and, with
+    host memory (so the launch is sized for the PCIe link instead of guessing) and, with
     ``beside_compute``, says that other kernels run meanwhile and matter. Planes of one side must all
     live on the same kind of memory."""
     def side(planes, what):

@@ -1,6 +1,7 @@
 """The benchmark configurations at their full sizes, launched exactly as the benchmark
-launches them (the caller names the host side, so a swap-out of 64 MiB or more runs
-paced and a swap-in keeps half as much in flight), and checked two ways:
+launches them (the caller names the host side, so a swap-out of 64 MiB or more runs on
+the link-sized grid with plain stores and a swap-in on 40 workgroups of one vector per
+lane), and checked two ways:
 
 * four planes of every case against the C oracle, whole destination planes compared
   (moved blocks and every untouched block alike);
@@ -156,8 +157,8 @@ def test_config4_mla_round_trip_full(named):
     dev_before = [dev_bytes[p].cpu() for p in ids]
     dtab, htab = ptr_table(planes), host_ptr_table(host)
     out_pairs, in_pairs = W.pairs_tensor(out_src, host_slots), W.pairs_tensor(host_slots, in_dst)
-    # 549 MiB each way: with the host side named the swap-out is paced, the swap-in moves 72 KiB blocks
-    # in 4.5 chunks of 16 KiB (the tail-chunk path)
+    # 549 MiB each way: with the host side named the swap-out runs on 32 workgroups of four vectors per lane
+    # (72 KiB blocks in 4.5 chunks of 16 KiB: the tail-chunk path), the swap-in on 40 of one
     swap(htab, dtab, out_pairs.to(DEV), cfg.planes, cfg.block_bytes, src_blocks=cfg.dev_blocks,
          dst_blocks=cfg.host_blocks, flags=capi.SWAP_DST_HOST if named else 0)
     swap(dtab, htab, in_pairs.to(DEV), cfg.planes, cfg.block_bytes, src_blocks=cfg.host_blocks,
@@ -190,7 +191,8 @@ def test_config5_fp8_fragmented_full():
         assert torch.equal(prefill[p], dev_bytes[p].index_select(0, ids_dev)), "plane %d gather" % p
     pool, host = _host_cache(cfg, host_blocks)
     pairs = W.pairs_tensor(ids, torch.arange(cfg.n_blocks))
-    # 4 GiB toward the host, the host side named: the paced launch the benchmark times for this configuration
+    # 4 GiB toward the host, the host side named: the launch the benchmark times for this configuration
+    # (16 KiB blocks: 32 workgroups of four vectors per lane, plain stores)
     swap(host_ptr_table(host), ptr_table(planes), pairs.to(DEV), cfg.planes, cfg.block_bytes, src_blocks=cfg.dev_blocks,
          dst_blocks=host_blocks, flags=capi.SWAP_DST_HOST)
     torch.cuda.synchronize()
@@ -207,7 +209,7 @@ def test_config5_fp8_fragmented_full():
             "plane %d gather differs from the oracle" % p
 
     # The same fragmented device blocks onto fragmented HOST slots through the mover that chooses per run of host
-    # slots (long runs: staging + copy engines; the rest: the small paced kernel), 4 GiB out and back.
+    # slots (long runs: staging + copy engines; the rest: the direct kernel over the short runs), 4 GiB out and back.
     host_ids = W.fragmented_ids(host_blocks, cfg.n_blocks, seed=11)
     for h in host:
         h.zero_()
@@ -287,9 +289,10 @@ def _verify_swap_out(c2, src_ids, dst_ids, what):
 
 
 @pytest.mark.parametrize("flags", [capi.SWAP_DST_HOST, 0, capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE],
-                         ids=["dst_host_paced", "no_flags", "beside_compute"])
+                         ids=["dst_host", "no_flags", "beside_compute"])
 def test_config2_llama8b_swap_out_full(c2, flags):
-    """flags = HFK_SWAP_DST_HOST is the launch the benchmark times: 512 MiB >= 64 MiB, so it is paced."""
+    """flags = HFK_SWAP_DST_HOST is the launch the benchmark times: 512 MiB >= 64 MiB, so 12 workgroups of eight
+    vectors per lane, unpaced, non-temporal loads and plain stores."""
     cfg = c2["cfg"]
     announce("config 2 full, swap-out of 256 pairs x 64 planes in one launch, flags %d" % flags)
     _clear_host(c2["host"])
