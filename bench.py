@@ -913,7 +913,7 @@ def main():
                          "always runs unless a profile of one other kernel alone is wanted")
     ap.add_argument("--tune", default="", help="comma list of library knobs for experiments, e.g. unroll=4,nt=0 "
                     "(unroll, nt, wg_per_cu, swap_wgs, swap_unroll, duplex_unroll, duplex_wgs, pace_mbps, link_mbps, "
-                    "throughput_pace, hbm_lds, paced_unroll, paced_wgs, transfer_pace, transfer_tiled); defaults are "
+                    "throughput_pace, hbm_lds, paced_unroll, paced_wgs, transfer_pace, transfer_tiled, duplex_pace); defaults are "
                     "the shipped ones")
     ap.add_argument("--out-flags", type=int, default=1, help="flags of the timed swap-out (default HFK_SWAP_DST_HOST = 1: "
                     "the caller knows its destination is host memory; 0 = say nothing)")
@@ -934,7 +934,8 @@ def main():
              "duplex_wgs": capi.KNOB_DUPLEX_WORKGROUPS, "throughput_pace": capi.KNOB_THROUGHPUT_PACE_PERMILLE,
              "hbm_lds": capi.KNOB_HBM_LDS_BYTES, "paced_unroll": capi.KNOB_PACED_UNROLL,
              "paced_wgs": capi.KNOB_PACED_WORKGROUPS,
-             "transfer_pace": capi.KNOB_TRANSFER_PACE_PERMILLE, "transfer_tiled": capi.KNOB_TRANSFER_TILED}
+             "transfer_pace": capi.KNOB_TRANSFER_PACE_PERMILLE, "transfer_tiled": capi.KNOB_TRANSFER_TILED,
+             "duplex_pace": capi.KNOB_DUPLEX_PACE_PERMILLE}
     tuned = {}
     for item in filter(None, args.tune.split(",")):
         key, val = item.split("=")

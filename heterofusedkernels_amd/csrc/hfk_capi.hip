@@ -254,8 +254,10 @@ constexpr uint32_t kBesideDuplexWorkgroups = 16;
 constexpr int kBesideDuplexUnroll = 2;
 constexpr uint32_t kBesideTransferWorkgroups = 16;
 constexpr uint32_t kTransferToHostWorkgroups = 32;
-constexpr uint32_t kShortTransferToHostWorkgroups = 64;
+constexpr uint32_t kShortTransferToHostWorkgroups = 64;     // under 128 MiB
 constexpr uint64_t kShortTransferBytes = 128ull << 20;
+constexpr uint32_t kShorterTransferToHostWorkgroups = 128;  // under 64 MiB
+constexpr uint64_t kShorterTransferBytes = 64ull << 20;
 constexpr uint32_t kTransferFromHostWorkgroups = 24;
 constexpr uint32_t kSingleBlockTransferWorkgroups = 32;
 constexpr uint32_t kHostGatherWorkgroups = 64;
@@ -611,6 +613,13 @@ int memory_side(const void* p) {
     return -1;
 }
 
+// A transfer toward the host that is over in a millisecond wants to be over sooner rather than gentler.
+uint32_t transfer_to_host_workgroups(uint64_t bytes) {
+    return bytes < kShorterTransferBytes ? kShorterTransferToHostWorkgroups
+           : bytes < kShortTransferBytes ? kShortTransferToHostWorkgroups
+                                         : kTransferToHostWorkgroups;
+}
+
 // `packed_side` is what the caller knows about the packed pool (1 host memory, 0 device memory);
 // kAskRuntime: the runtime is asked where it lives.
 constexpr int kAskRuntime = -2;
@@ -632,7 +641,7 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     // difference in address translation: 0.05 % of the lookups miss either way). Through LDS tiles
     // (1 KiB runs on both sides) with plain stores: 56.5-56.6 GB/s on 32 workgroups for transfers of
     // 256 MiB and more (55.4 with non-temporal stores, 56.1 on 64 workgroups); short transfers want
-    // more workgroups to be over sooner (32 MiB: 54.2 on 32, 55.3 on 64; 64 MiB: 55.4 and 55.6).
+    // more workgroups to be over sooner (32 MiB: 54.2 on 32, 55.3 on 64, 55.8 on 128; 64 MiB: 55.4, 55.6, 55.6).
     // Pacing does not pay: at 0.895 of the link 55.3-55.9 on the long shapes and 50-52 on the short.
     const int side = packed_side == kAskRuntime ? memory_side(packed) : packed_side;
     const int unroll = to_packed && side != 0 ? (int)knob_value(HFK_KNOB_TRANSFER_UNROLL) : hfk::kTransposeUnroll;
@@ -651,8 +660,7 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
         // block table may run for many milliseconds beside other kernels and gets the smaller grid.
         workgroups = pairs == nullptr ? kSingleBlockTransferWorkgroups
                      : beside_compute ? kBesideTransferWorkgroups
-                     : to_packed      ? ((uint64_t)a.total_units * unit * n_pairs < kShortTransferBytes ? kShortTransferToHostWorkgroups
-                                                                                                       : kTransferToHostWorkgroups)
+                     : to_packed      ? transfer_to_host_workgroups((uint64_t)a.total_units * unit * n_pairs)
                                       : kTransferFromHostWorkgroups;
     }
     uint32_t grid = 0;
