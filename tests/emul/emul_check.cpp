@@ -414,6 +414,44 @@ void case_auto(uint32_t n_planes, uint32_t n_pairs, uint64_t block_bytes, uint32
     for (auto* b : host_exp) delete b;
 }
 
+// What the run-splitting swap does when its two copies of the host column disagree (the header documents it;
+// HFK_KNOB_CHECK_HOST_COLUMN exists to catch it): the copy engines take their runs from the host array, the
+// kernels theirs from the table. Here the array calls all four pairs one long run, the table calls them four
+// single slots. On the way out the staging kernel therefore fills nothing, the copies send the four staging
+// slots as they are to the array's slots, and the direct kernel then moves every pair to the table's slots: a
+// slot both name ends up right, a slot only the array names holds what staging held before the call.
+void case_auto_with_disagreeing_columns() {
+    const uint64_t bb = 4096;
+    const uint32_t n = 4, dev_blocks = 8, host_blocks = 40, min_run = 2;
+    Buf dev(dev_blocks * bb), host(host_blocks * bb), staging(n * bb);
+    dev.randomize();
+    host.fill(0x11);
+    staging.fill(0xEE);                                   // "an earlier transfer's bytes"
+    const int64_t array_ids[n] = {10, 11, 12, 13}, table_ids[n] = {10, 20, 12, 30}, dev_ids[n] = {3, 1, 7, 5};
+    std::vector<int64_t> pairs;
+    for (uint32_t j = 0; j < n; ++j) { pairs.push_back(dev_ids[j]); pairs.push_back(table_ids[j]); }
+    uint64_t dp[1] = {(uint64_t)(uintptr_t)dev.p}, hp[1] = {(uint64_t)(uintptr_t)host.p};
+    BlockCopyArgs<int64_t> direct, hbm;
+    int rc = plan_swap_blocks(direct, hp, dp, pairs.data(), 1, n, bb, bb, bb, dev_blocks, host_blocks);
+    if (rc == HFK_OK) rc = plan_stage_blocks(hbm, dp, staging.p, pairs.data(), 1, n, bb, bb, dev_blocks, true);
+    if (rc != HFK_OK) { ++g_failures; std::printf("disagreeing columns: plan rc=%d\n", rc); return; }
+    direct.zero_skipped = 1;
+    hbm.id_stride = 2;
+    filter_runs(hbm, kLongRunsOnly, pairs.data() + 1, min_run);
+    filter_runs(direct, kShortRunsOnly, pairs.data() + 1, min_run);
+    run_block_copy<int64_t, 3>(hbm, 1, 4, true);                                     // the table has no long run: nothing staged
+    for_each_host_run(array_ids, n, [&](uint64_t first, uint64_t len) {              // the array has one: four slots copied
+        if (len >= min_run) std::memcpy(host.p + (uint64_t)array_ids[first] * bb, staging.p + first * bb, len * bb);
+    });
+    run_block_copy<int64_t, 3>(direct, 1, 4);                                        // every pair is short for the table
+    Buf want(host_blocks * bb);
+    want.fill(0x11);
+    std::memset(want.p + 11 * bb, 0xEE, bb);              // named by the array only: stale staging bytes
+    std::memset(want.p + 13 * bb, 0xEE, bb);
+    for (uint32_t j = 0; j < n; ++j) std::memcpy(want.p + (uint64_t)table_ids[j] * bb, dev.p + (uint64_t)dev_ids[j] * bb, bb);
+    expect_equal(host.p, want.p, host.n, "run-splitting swap with disagreeing host columns");
+}
+
 // ---- gather_blocks (multi-plane, shared ids) -------------------------------
 void case_gather_blocks(uint32_t n_planes, uint32_t n_ids, uint64_t block_bytes, uint64_t src_blocks, int unroll,
                         uint32_t grid_cap) {
@@ -799,6 +837,8 @@ int main() {
                 case_auto(2, 11, 73728, 12, 30, to_host, min_run, unroll, 16, true);
                 case_auto(1, 9, 4100, 10, 20, to_host, min_run, unroll, 3, false);
             }
+
+    case_auto_with_disagreeing_columns();
 
     // block-table transfer, both directions
     for (bool to_packed : {false, true}) {

@@ -494,6 +494,44 @@ def test_paced_swap_ends_when_its_rate_is_unreachably_low(memory):
     announce("PCIe link rate read from sysfs: %d MB/s (0 = unreadable: paced swaps run unpaced)" % capi.get_tuning(capi.KNOB_LINK_MBPS))
 
 
+def test_pace_report_accounts_for_every_turn(memory):
+    """HFK_KNOB_PACE_REPORT: every workgroup of a paced swap leaves its account (ticks run, ticks allotted, turns,
+    late turns, largest delay, interval). The turns add up to the launch's work items, the interval is the same
+    in every row and matches the offered rate, and a launch paced far below the link's rate keeps its schedule:
+    it runs no longer than allotted (plus its last item) and almost no turn begins late."""
+    cfg = W.C2_LLAMA8B_SWAP_OUT.scaled(layers=4, dev_blocks=64, host_blocks=64, n_blocks=48)
+    bb = cfg.block_bytes
+    cpu = [W.as_bytes(p).clone() for p in _cpu_planes(cfg, cfg.dev_blocks)]
+    dev = [p.to(DEV) for p in cpu]
+    src_ids, dst_ids = W.block_table(cfg, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    pairs = W.pairs_tensor(src_ids, dst_ids).to(DEV)
+    dtab = ptr_table(dev)
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0x22)
+    grid, pace_mbps = 12, 20000                       # the beside-compute shape: 12 workgroups x 1 vector per lane, at 20 GB/s
+    report = torch.full((grid, 8), -1, dtype=torch.int64, device=DEV)
+    announce("pace report: %d planes x %d blocks paced at %d MB/s" % (cfg.planes, src_ids.numel(), pace_mbps))
+    with capi.thread_tuning({capi.KNOB_SWAP_PACE_MBPS: pace_mbps, capi.KNOB_PACE_REPORT: report.data_ptr()}):
+        capi.check(capi.swap_blocks(host_ptr_table(host).data_ptr(), dtab.data_ptr(), pairs.data_ptr(), cfg.planes,
+                                    src_ids.numel(), bb, bb, bb, cfg.dev_blocks, cfg.host_blocks, 0, stream_handle(),
+                                    capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE))
+    torch.cuda.synchronize()
+    for p in range(cfg.planes):
+        want = torch.full((cfg.host_blocks, bb), 0x22, dtype=torch.uint8)
+        O.torch_swap_blocks(want, cpu[p], src_ids, dst_ids)
+        assert torch.equal(host[p], want), "plane %d" % p
+    rows = report.cpu()
+    ran, allotted, turns, late, worst, interval_q8 = (rows[:, i] for i in range(6))
+    items = cfg.planes * src_ids.numel() * (bb // 4096)            # one 4 KiB chunk per work item
+    assert int(turns.sum()) == items, (int(turns.sum()), items)
+    assert bool((rows[:, 6:] == 0).all())
+    assert int(interval_q8.min()) == int(interval_q8.max()) > 0
+    ticks_per_item = float(interval_q8[0]) / 256.0 / grid          # 100 MHz ticks the launch allots to one item
+    assert abs(ticks_per_item - 4096 / (pace_mbps * 1e6) * 1e8) < 0.05 * ticks_per_item, ticks_per_item
+    assert bool((ran <= allotted + 2 * interval_q8 // 256).all()), (ran.tolist(), allotted.tolist())
+    assert int(late.sum()) <= items // 20, (int(late.sum()), items)
+    assert capi.get_tuning(capi.KNOB_PACE_REPORT) == 0             # the override ended with the block
+
+
 # ---------------------------------------------------------------------------
 # edge cases
 # ---------------------------------------------------------------------------
