@@ -1138,7 +1138,12 @@ int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs
     if (host_block_ids != nullptr && block_pairs != nullptr && knob_value(HFK_KNOB_CHECK_HOST_COLUMN) != 0) {
         // Debugging aid: the two movers read the host column from two places; make sure they agree.
         hipError_t e = hipStreamSynchronize(s);   // whatever uploads the table on this stream has finished
-        std::vector<int64_t> table(2 * n_pairs);
+        std::vector<int64_t> table;
+        try {
+            table.resize(2 * n_pairs);
+        } catch (...) {                           // nothing may be thrown across this interface
+            return HFK_ERR_TOO_LARGE;
+        }
         if (e == hipSuccess) e = hipMemcpy(table.data(), block_pairs, 2 * n_pairs * sizeof(int64_t), hipMemcpyDefault);
         if (e != hipSuccess) return (int)e;
         for (uint64_t j = 0; j < n_pairs; ++j) {
@@ -1182,7 +1187,7 @@ int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs
     bool compact = false;
     uint64_t slots_offset = 0;
     if (long_blocks != 0 && !holds_table) {
-        if (long_blocks < n_pairs && long_blocks <= staging_bytes / block_bytes / n_planes) {
+        if (long_blocks < n_pairs && n_pairs <= 0x7fffffffu && long_blocks <= staging_bytes / block_bytes / n_planes) {
             slots_offset = (n_planes * long_blocks * block_bytes + 255u) & ~(uint64_t)255u;
             compact = slots_offset <= staging_bytes && n_pairs <= (staging_bytes - slots_offset) / (2 * sizeof(int64_t));
         }

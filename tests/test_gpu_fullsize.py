@@ -377,3 +377,37 @@ def test_config2_staged_and_auto_full(c2, mover):
                    "hfk_swap_blocks_auto")
     torch.cuda.synchronize()
     _verify_swap_out(c2, src_ids, host_ids, mover)
+
+
+@pytest.mark.parametrize("bb", [4096, 8192, 12288, 20480, 69632, 131072 + 16])
+def test_long_swap_out_shapes_by_block_size(bb):
+    """A swap-out of 64 MiB or more toward a named host side picks its grid and its vectors per lane from the
+    block size (96 x 1, 64 x 2, 32 x 4, 12 x 8; one workgroup more where the grid would split evenly over chunks
+    of unequal size) and stores plainly. One launch of 64-66 MiB per block size, among them sizes with a short
+    last chunk and one that is not a multiple of 256 bytes; two planes against the C oracle, all planes against
+    torch indexing."""
+    n_planes = 8
+    n = (64 << 20) // (n_planes * bb) + 1
+    dev_blocks, host_blocks = n + 7, n + 11
+    announce("long swap-out, blocks of %d B: %d planes x %d blocks = %.1f MiB" % (bb, n_planes, n, n_planes * n * bb / 2**20))
+    gen = torch.Generator().manual_seed(bb)
+    dev = [torch.randint(0, 256, (dev_blocks, bb), dtype=torch.uint8, device=DEV,
+                         generator=torch.Generator(device=DEV).manual_seed(bb + p)) for p in range(n_planes)]
+    pool = memory.alloc_numa_pinned_tensor(n_planes * host_blocks * bb).view(torch.uint8)
+    pool.fill_(0x6B)
+    host = list(pool.view(n_planes, host_blocks, bb).unbind(0))
+    src, dst = torch.randperm(dev_blocks, generator=gen)[:n], torch.randperm(host_blocks, generator=gen)[:n]
+    pairs = W.pairs_tensor(src, dst)
+    assert n_planes * n * bb >= 64 << 20
+    swap(host_ptr_table(host), ptr_table(dev), pairs.to(DEV), n_planes, bb, src_blocks=dev_blocks, dst_blocks=host_blocks,
+         flags=capi.SWAP_DST_HOST)
+    torch.cuda.synchronize()
+    ids = [0, n_planes - 1]
+    before = [torch.full((host_blocks, bb), 0x6B, dtype=torch.uint8) for _ in ids]
+    _check_against_oracle([host[p] for p in ids], before, [dev[p].cpu() for p in ids], pairs, ids, "blocks of %d B" % bb)
+    src_dev = src.to(DEV)
+    untouched = torch.ones(host_blocks, dtype=torch.bool)
+    untouched[dst] = False
+    for p in range(n_planes):
+        assert torch.equal(host[p].index_select(0, dst), dev[p].index_select(0, src_dev).cpu()), "plane %d" % p
+        assert bool((host[p][untouched] == 0x6B).all()), "plane %d: wrote outside its slots" % p
