@@ -482,7 +482,8 @@ HFK_API int64_t hfk_get_tuning(int knob);
  * from the process-wide values; other threads see no change. A second begin replaces the first
  * (there is no nesting). A list with an unknown knob or an invalid value is rejected as a whole
  * (HFK_ERR_BAD_KNOB) and leaves the thread's overrides as they were. hfk_get_tuning shows the
- * calling thread's view.
+ * calling thread's view. No counterpart in the reference, whose only tunable is the aivNum argument
+ * of its ops (pcieThrough/csrc/host/gather_torch.cpp:32-36), passed per call.
  */
 typedef struct hfk_knob_value {
     int knob;       /* enum hfk_knob */
