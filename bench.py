@@ -702,20 +702,34 @@ def section_repeat(b, w, steps, warmup, flags, first_value):
     log("swap-out repeated at the end: %s GB/s in three batches (first measurement %s), isolated launches %.2f / %.2f / %.2f "
         "(slowest / median / fastest)" % (" / ".join("%.2f" % x[0] for x in batches),
                                            "%.2f" % first_value if first_value else "-", iso["max_ms"], iso["median_ms"], iso["min_ms"]))
-    # a paced launch of the same swap and how it kept its schedule
+    # a paced launch of the same swap and how it kept its schedule: at a fixed pace, and with the pace that the
+    # launches before it set (the library's default for a paced throughput-mode swap)
     report = torch.zeros(64 * 8, dtype=torch.int64, device=b.dev)
     paced = {}
     for permille in (890, 900):
-        with capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: permille, capi.KNOB_PACE_REPORT: report.data_ptr()}):
+        with capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: permille, capi.KNOB_ADAPTIVE_PACE: 0,
+                                 capi.KNOB_PACE_REPORT: report.data_ptr()}):
             _, pms = b.timed(lambda: w.swap_out(capi.SWAP_DST_HOST), max(4, steps // 2), 1)
             grid = capi.get_tuning(capi.KNOB_PACED_WORKGROUPS)
         rows = report.cpu().view(64, 8)[:grid]
         ran, allotted, turns, late, worst = (rows[:, i].double() for i in range(5))
-        paced["at_0.%d_of_link" % (permille // 10)] = {
+        paced["fixed_at_0.%d_of_link" % (permille // 10)] = {
             "GBps": round(w.payload / (pms * 1e6), 2), "workgroups": grid,
             "ran_over_allotted": round(float((ran / allotted.clamp(min=1)).max()), 4),
             "late_turns_pct": round(100 * float(late.sum() / turns.sum().clamp(min=1)), 2),
             "largest_delay_us": round(float(worst.max()) / 100.0, 1)}
+    for permille in (870, 910):          # wherever it starts, the pace set between launches ends up in the same place
+        with capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: permille}):
+            b.timed(lambda: w.swap_out(capi.SWAP_DST_HOST), 40, 0)
+            _, pms = b.timed(lambda: w.swap_out(capi.SWAP_DST_HOST), max(4, steps // 2), 0)
+        st = capi.pace_state()
+        paced["set_between_launches_from_0.%d" % (permille // 10)] = {
+            "GBps": round(w.payload / (pms * 1e6), 2), "factor": round(st[0] / 65536.0, 4),
+            "offered_share_of_link": round(permille / 1000.0 / (st[0] / 65536.0), 4),
+            "late_turns_pct_of_last_launch": round(100 * st[6] / 65536.0, 2), "launches_settled": st[5]}
+    for p in (0, cfg.planes - 1):
+        want = w.dev_bytes[p].index_select(0, w.ids_dev).cpu()
+        assert torch.equal(w.host_planes[p].index_select(0, w.dst_ids), want), "paced swap-out mismatch in plane %d" % p
     out["paced_launch_of_the_same_swap"] = paced
     log("paced launches of the same swap: %s" % json.dumps(paced))
     return out

@@ -30,6 +30,7 @@ KNOB_TRANSFER_PACE_PERMILLE = 15
 KNOB_TRANSFER_UNROLL = 16
 KNOB_CHECK_HOST_COLUMN = 17
 KNOB_TRANSFER_TILED = 18
+KNOB_ADAPTIVE_PACE = 19
 SWAP_DST_HOST = 1
 SWAP_SRC_HOST = 2
 SWAP_BESIDE_COMPUTE = 4
@@ -68,6 +69,7 @@ ENTRY_POINTS = (
     "hfk_gather_blocks",
     "hfk_set_tuning",
     "hfk_get_tuning",
+    "hfk_pace_state",
     "hfk_thread_tuning_begin",
     "hfk_thread_tuning_end",
 )
@@ -131,6 +133,8 @@ def load():
     L.hfk_set_tuning.restype = ci
     L.hfk_get_tuning.argtypes = [ci]
     L.hfk_get_tuning.restype = i64
+    L.hfk_pace_state.argtypes = [ctypes.POINTER(ctypes.c_uint32)]
+    L.hfk_pace_state.restype = ci
     L.hfk_thread_tuning_begin.argtypes = [ctypes.POINTER(KnobValue), u32]
     L.hfk_thread_tuning_begin.restype = ci
     L.hfk_thread_tuning_end.argtypes = []
@@ -222,6 +226,13 @@ def set_tuning(knob, value):
 
 def get_tuning(knob):
     return load().hfk_get_tuning(knob)
+
+
+def pace_state():
+    """The eight words of hfk_pace_state for the current device (waits for the device)."""
+    out = (ctypes.c_uint32 * 8)()
+    check(load().hfk_pace_state(out), "hfk_pace_state")
+    return list(out)
 
 
 class thread_tuning:

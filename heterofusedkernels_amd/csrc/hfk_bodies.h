@@ -56,6 +56,44 @@ typedef uint32_t vec16 __attribute__((ext_vector_type(4)));
 // throughput. Workgroup `bid` of `nb` starts its k-th work item no earlier than
 // (k + bid / nb) * pace_q8 / 256 ticks of the 100 MHz counter after it began, so the launch as a
 // whole offers one item per pace_q8 / 256 / nb ticks. pace_q8 == 0: no pacing.
+// A pace that is set between launches. What the link takes, and what a tick of the counter is worth,
+// differ by a percent from machine to machine and from moment to moment, and the room between a pace that
+// keeps the queues empty and one the link cannot hold is smaller than that. A launch cannot find the
+// right interval while it runs (its wavefronts hand their stores to the memory pipeline and notice an
+// overloaded link only when the queues behind them are full), but all of a launch's workgroups together
+// know afterwards how it went: how many of their turns began late (2 % at 0.89 of what the link takes,
+// 4 % at 0.895, 7 % at 0.90, 14 % at 0.905, its knee), and whether any of them ended behind its schedule.
+// The last workgroup to finish turns that into a factor for the next launch's interval, kept in eight
+// words of device memory that belong to the library: [0] the factor in 1/65536 (0 = 1.0), [1] turns and
+// [2] late turns of the launch in progress, [3] workgroups finished, [4] workgroups that ended behind
+// schedule, [5] launches settled, [6] late turns per 65536 turns of the last launch, [7] unused.
+// Launches on one stream see each other's result in order; launches that overlap on two streams may
+// read a factor one launch old, which is harmless.
+constexpr uint32_t kPaceFactorOne = 65536;
+constexpr uint32_t kPaceFactorMin = 61000;        // the interval may shrink by 7 % ...
+constexpr uint32_t kPaceFactorMax = 68157;        // ... and grow by 4 % from the nominal one: what slows a launch down
+                                                  // may be a neighbour and not the link, and must not cost it much
+
+HFK_HD uint32_t pace_factor(const uint32_t* state) {
+    if (state == nullptr) return kPaceFactorOne;
+    const uint32_t f = *reinterpret_cast<const HFK_GLOBAL uint32_t*>(reinterpret_cast<uint64_t>(state));
+    return f == 0 ? kPaceFactorOne : f;
+}
+
+// The factor for the next launch from this one's account: late turns per 65536 turns, and whether any
+// workgroup ended behind its schedule.
+HFK_HD uint32_t next_pace_factor(uint32_t factor, uint32_t late_per_65536, bool behind) {
+    uint64_t f = factor;
+    if (behind) f += f >> 6;                                   // could not hold it: 1.6 % slower
+    else if (late_per_65536 > 5243) f += f >> 8;               // more than 8 % late: 0.4 % slower
+    else if (late_per_65536 > 3604) f += f >> 9;               // more than 5.5 %: 0.2 % slower
+    else if (late_per_65536 < 1638) f -= f >> 8;               // fewer than 2.5 %: 0.4 % faster
+    else if (late_per_65536 < 2621) f -= f >> 10;              // fewer than 4 %: 0.1 % faster
+    if (f < kPaceFactorMin) f = kPaceFactorMin;
+    if (f > kPaceFactorMax) f = kPaceFactorMax;
+    return (uint32_t)f;
+}
+
 struct Pacer {
     uint64_t t0;
     uint64_t due_q8;
@@ -105,6 +143,34 @@ struct Pacer {
         row[5] = pace_q8;
         row[6] = 0;
         row[7] = 0;
+    }
+
+    // End of a workgroup of a launch whose pace is set between launches (see pace_factor): adds its
+    // account to the launch's, and the last workgroup settles the factor for the next launch.
+    HFK_HD void settle(uint32_t* state, uint32_t factor, uint32_t nb, uint32_t tid) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        if (state == nullptr || pace_q8 == 0 || tid != 0) return;
+        atomicAdd(&state[1], turns);
+        atomicAdd(&state[2], late_turns);
+        if (((HFK_TICKS_100MHZ() - t0) << 8) > due_q8 + 2ull * pace_q8) atomicAdd(&state[4], 1u);
+        __threadfence();
+        if (atomicAdd(&state[3], 1u) + 1u == nb) {
+            __threadfence();
+            const uint32_t all_turns = atomicAdd(&state[1], 0u), all_late = atomicAdd(&state[2], 0u);
+            const uint32_t behind = atomicAdd(&state[4], 0u);
+            const uint32_t late_per_65536 = all_turns != 0 ? (uint32_t)(((uint64_t)all_late << 16) / all_turns) : 0u;
+            HFK_GLOBAL uint32_t* g = reinterpret_cast<HFK_GLOBAL uint32_t*>(reinterpret_cast<uint64_t>(state));
+            g[0] = next_pace_factor(factor, late_per_65536, behind != 0);
+            g[1] = 0;
+            g[2] = 0;
+            g[3] = 0;
+            g[4] = 0;
+            g[5] = g[5] + 1;
+            g[6] = late_per_65536;
+        }
+#else
+        (void)state; (void)factor; (void)nb; (void)tid;
+#endif
     }
 };
 
@@ -198,6 +264,7 @@ struct BlockCopyArgs {
     uint32_t run_min;            // a run is "long" from this many consecutive ids on
     const int64_t* run_ids;      // entry j at run_ids[j * id_stride]
     uint64_t* pace_report;       // null, or where each workgroup of a paced launch leaves Pacer::report
+    uint32_t* pace_state;        // null, or the library's eight words for a pace set between launches (pace_factor)
 };
 
 // Which pairs of a block table a launch moves, when the table is split by run length: pair j belongs to
@@ -381,7 +448,8 @@ HFK_HD void zero_chunk(uint64_t d_addr, uint64_t block_bytes, uint32_t chunk, ui
 // instruction of its prologue.
 template <typename IdT, int UNROLL, int NT, bool SPLIT = false, bool PACED = true>
 HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
-    Pacer pacer(PACED ? a.pace_q8 : 0u, bid, nb);
+    const uint32_t factor = PACED ? pace_factor(a.pace_state) : kPaceFactorOne;
+    Pacer pacer(PACED ? (uint32_t)(((uint64_t)a.pace_q8 * factor) >> 16) : 0u, bid, nb);
     uint64_t id = bid;                  // 64-bit so that id + nb cannot wrap
     uint32_t judged_pair = 0xffffffffu; // SPLIT: the pair the filter was last evaluated for, and its verdict
     bool judged_selected = false;       // (a workgroup's consecutive items mostly belong to one pair)
@@ -413,7 +481,10 @@ HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t 
         }
         id += nb;
     }
-    if constexpr (PACED) pacer.report(a.pace_report, bid, tid);
+    if constexpr (PACED) {
+        pacer.report(a.pace_report, bid, tid);
+        pacer.settle(a.pace_state, factor, nb, tid);
+    }
 }
 
 // ---------------------------------------------------------------------------

@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256) void stage_slots_kernel(const int64_t* ids, ui
 // Every knob has a process-wide value (hfk_set_tuning) and, per thread, an optional override that
 // lasts from hfk_thread_tuning_begin to hfk_thread_tuning_end: a caller that wants a launch shape
 // of its own for a few calls changes nothing another thread can see.
-constexpr int kKnobCount = 19;
+constexpr int kKnobCount = 20;
 std::atomic<int64_t> g_knob[kKnobCount] = {
     1,       // HFK_KNOB_UNROLL
     3,       // HFK_KNOB_NONTEMPORAL
@@ -211,6 +211,7 @@ std::atomic<int64_t> g_knob[kKnobCount] = {
     8,       // HFK_KNOB_TRANSFER_UNROLL
     0,       // HFK_KNOB_CHECK_HOST_COLUMN
     1,       // HFK_KNOB_TRANSFER_TILED
+    1,       // HFK_KNOB_ADAPTIVE_PACE
 };
 
 struct ThreadTuning {
@@ -245,7 +246,8 @@ bool knob_value_valid(int k, int64_t v) {
         case HFK_KNOB_TRANSFER_PACE_PERMILLE: return v >= 0 && v <= 2000;
         case HFK_KNOB_TRANSFER_UNROLL: return v == 2 || v == 8;
         case HFK_KNOB_CHECK_HOST_COLUMN:
-        case HFK_KNOB_TRANSFER_TILED: return v == 0 || v == 1;
+        case HFK_KNOB_TRANSFER_TILED:
+        case HFK_KNOB_ADAPTIVE_PACE: return v == 0 || v == 1;
         default: return false;
     }
 }
@@ -432,6 +434,27 @@ int current_link_mbps() {
     return v > 0 ? v : 0;
 }
 
+// The eight words behind a pace that is set between launches (hfk::pace_factor): one set per device, in the
+// library's device image like the staging array below, zero until the first paced launch has settled.
+static __device__ __align__(32) uint32_t pace_state_words[8];
+std::atomic<void*> g_pace_state_ptr[kMaxDevices];
+
+int pace_state(uint32_t** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return HFK_ERR_TOO_LARGE;
+    void* ptr = g_pace_state_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(pace_state_words));   // `dev` is current: its copy of the words
+        if (e != hipSuccess) return (int)e;
+        if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+        g_pace_state_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = static_cast<uint32_t*>(ptr);
+    return HFK_OK;
+}
+
 // ---- block copy -----------------------------------------------------------
 template <Role ROLE, typename IdT, int UNROLL, int NT>
 void launch_block_copy_one(const BlockCopyArgs<IdT>& a, uint32_t grid, uint32_t lds, hipStream_t s) {
@@ -471,7 +494,7 @@ void launch_block_copy_nt(const BlockCopyArgs<IdT>& a, uint32_t grid, int nt, ui
 
 template <Role ROLE, typename IdT>
 int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, int preferred_unroll = 0,
-                      uint32_t pace_mbps = 0, bool plain_stores = false) {
+                      uint32_t pace_mbps = 0, bool plain_stores = false, bool pace_between_launches = false) {
     int unroll = 1;
     if (preferred_unroll == 0) preferred_unroll = (int)knob_value(HFK_KNOB_UNROLL);
     // Everything but the swap runs one workgroup per chunk and wants whole chunks.
@@ -484,6 +507,10 @@ int launch_block_copy(BlockCopyArgs<IdT> a, uint32_t workgroups, hipStream_t s, 
         // bytes per work item (average over a block) * workgroups / rate
         a.pace_q8 = pace_interval_q8((double)a.block_bytes / a.chunks_per_block, grid, pace_mbps);
         a.pace_report = reinterpret_cast<uint64_t*>((uintptr_t)knob_value(HFK_KNOB_PACE_REPORT));
+        if (pace_between_launches) {
+            rc = pace_state(&a.pace_state);
+            if (rc != 0) return rc;
+        }
     }
     const int nt = (int)knob_value(HFK_KNOB_NONTEMPORAL) & (plain_stores ? 1 : 3);
     // HBM-bound launches may ask for LDS they never touch: it bounds how many workgroups a compute
@@ -704,8 +731,12 @@ int launch_swap(const BlockCopyArgs<int64_t>& a, uint32_t flags, uint32_t workgr
                                  (uint32_t)knob_value(HFK_KNOB_SWAP_PACE_MBPS)};
     const hfk::SwapShape shape =
         hfk::choose_swap_shape(flags, bytes, a.block_bytes, wants_pace ? (uint32_t)current_link_mbps() : 0u, workgroups, tuning);
+    // A paced throughput-mode swap lets the launches before it set its pace (hfk::pace_factor); the beside-compute
+    // pace is meant to stay well under the link's limit and stays fixed.
+    const bool between = shape.pace_mbps != 0 && (flags & HFK_SWAP_BESIDE_COMPUTE) == 0 &&
+                         knob_value(HFK_KNOB_ADAPTIVE_PACE) != 0;
     return launch_block_copy<Role::kSwapBlocks, int64_t>(a, shape.workgroups, s, shape.unroll, shape.pace_mbps,
-                                                         shape.plain_stores);
+                                                         shape.plain_stores, between);
 }
 
 // ---- staged swap: HBM-only kernel + DMA copies ----------------------------
@@ -1245,6 +1276,15 @@ int hfk_gather_blocks(const void* dst_plane_ptrs, const void* src_plane_ptrs, co
         return launch_swap(a, flags, workgroups, (uint64_t)n_planes * n_ids * block_bytes, s);
     }
     return launch_block_copy<Role::kGatherBlocks, int64_t>(a, workgroups, s);
+}
+
+int hfk_pace_state(uint32_t* out8) {
+    if (out8 == nullptr) return HFK_ERR_NULL_POINTER;
+    uint32_t* words = nullptr;
+    int rc = pace_state(&words);
+    if (rc != 0) return rc;
+    hipError_t e = hipMemcpy(out8, words, 8 * sizeof(uint32_t), hipMemcpyDeviceToHost);   // waits for the device
+    return e == hipSuccess ? HFK_OK : (int)e;
 }
 
 int hfk_set_tuning(int knob, int64_t value) {

@@ -109,8 +109,11 @@ inline SwapShape choose_swap_shape(uint32_t flags, uint64_t bytes, uint64_t bloc
         if (beside) pace = t.beside_pace_mbps != 0 ? t.beside_pace_mbps : (uint32_t)(kBesidePaceShareOfLink * link_mbps);
         else pace = (uint32_t)(t.throughput_pace_permille / 1000.0 * link_mbps);
         if (pace != 0) {
-            const uint32_t grid = beside ? kBesidePacedWorkgroups : t.paced_workgroups;
-            return SwapShape{workgroups ? workgroups : grid, beside ? kFineUnroll : t.paced_unroll, pace, false};
+            // the paced throughput shape keeps paced_workgroups x paced_unroll vectors per lane in flight:
+            // blocks too small for that many vectors per lane get more workgroups instead
+            const int fitted = beside ? kFineUnroll : fit_unroll(block_bytes, t.paced_unroll);
+            const uint32_t grid = beside ? kBesidePacedWorkgroups : t.paced_workgroups * (uint32_t)(t.paced_unroll / fitted);
+            return SwapShape{workgroups ? workgroups : grid, fitted, pace, false};
         }
         if (!beside) {
             SwapShape shape = to_host_shape(block_bytes);

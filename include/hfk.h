@@ -8,8 +8,9 @@
  *   - returns 0 on success, a negative hfk_status for a rejected argument, or a
  *     positive hipError_t reported by the HIP runtime,
  *   - never throws, owns no memory and keeps no state between calls apart from
- *     cached device properties and the values set through hfk_set_tuning() (process-wide)
- *     or hfk_thread_tuning_begin() (calling thread only).
+ *     cached device properties, the values set through hfk_set_tuning() (process-wide)
+ *     or hfk_thread_tuning_begin() (calling thread only), one event per device for
+ *     hfk_swap_blocks_staged_static, and, on the device, the eight words of hfk_pace_state().
  *
  * "Device-visible" below means an address a kernel may dereference: device
  * memory, or pinned host memory in its mapped (hipHostGetDevicePointer) form.
@@ -446,8 +447,10 @@ enum hfk_knob {
                                        HFK_SWAP_BESIDE_COMPUTE. Default 0 = unpaced: 12 workgroups x 8 vectors
                                        per lane with plain stores, the fastest shape and the one whose rate does
                                        not depend on a clock; paced, HFK_KNOB_PACED_WORKGROUPS x
-                                       HFK_KNOB_PACED_UNROLL with non-temporal stores, gentler on kernels that
-                                       run beside it                                                       */
+                                       HFK_KNOB_PACED_UNROLL vectors per lane in flight with non-temporal stores,
+                                       gentler on kernels that run beside it (a device copy 1.3x slower instead of
+                                       5.5x), at 98.5-99.5 % of the unpaced rate once HFK_KNOB_ADAPTIVE_PACE has
+                                       had ten or so launches to settle the pace                            */
     HFK_KNOB_HBM_LDS_BYTES = 10,    /* dynamic LDS, 0..65536 bytes, that the HBM-bound launches (gathers, the
                                        staged swap's kernel) request without using it: with 160 KiB of LDS
                                        per compute unit it bounds the workgroups a unit holds at a time   */
@@ -469,10 +472,25 @@ enum hfk_knob {
     HFK_KNOB_TRANSFER_TILED = 18,   /* 1 (default): a block-table transfer into a packed pool in host memory goes through
                                        LDS tiles where its geometry allows (1 KiB runs on both sides); 0: always
                                        row by row                                                               */
+    HFK_KNOB_ADAPTIVE_PACE = 19,    /* 1 (default): a paced throughput-mode swap-out (HFK_KNOB_THROUGHPUT_PACE_PERMILLE != 0)
+                                       takes its interval times a factor that the paced launches before it on this
+                                       device have settled (see hfk_pace_state); 0: the interval as computed        */
     HFK_KNOB_CHECK_HOST_COLUMN = 17 /* debugging aid, default 0: hfk_swap_blocks_auto first waits for its stream,
                                        reads block_pairs back and compares its host column with host_block_ids;
                                        a difference rejects the call with HFK_ERR_TABLE_MISMATCH                */
 };
+/*
+ * The state behind a pace that is set between launches, for the current device: eight words,
+ * [0] the factor applied to the interval of the next paced throughput-mode swap-out, in 1/65536
+ * (0 = none settled yet, i.e. 1.0; kept within 0.93 .. 1.12), [1]-[4] the account of a launch in
+ * progress, [5] launches settled, [6] late turns per 65536 turns of the last one, [7] unused.
+ * Every such launch ends by settling the factor for the next one from how many of its turns began
+ * late and whether a workgroup ended behind its schedule: the pace follows what this machine's link
+ * takes instead of what its nominal rate and a nominal 100 MHz say. Diagnostic: waits for the device.
+ * No counterpart in the reference.
+ */
+HFK_API int hfk_pace_state(uint32_t* out8);
+
 HFK_API int hfk_set_tuning(int knob, int64_t value);
 HFK_API int64_t hfk_get_tuning(int knob);
 

@@ -709,6 +709,32 @@ void case_swap_shape() {
                         got.workgroups, got.unroll, r.wg, r.unroll);
         }
     }
+    // the paced throughput shape keeps 6 x 4 vectors per lane in flight whatever the block size
+    struct { uint64_t block; uint32_t wg; int unroll; } paced_by_block[] = {{4096, 24, 1}, {8192, 12, 2}, {16384, 6, 4}, {73728, 6, 4}};
+    for (const auto& r : paced_by_block) {
+        const SwapShape got = choose_swap_shape(out, big, r.block, link, 0, paced);
+        ++g_cases;
+        if (got.workgroups != r.wg || got.unroll != r.unroll || got.pace_mbps != 56083 || got.plain_stores) {
+            ++g_failures;
+            std::printf("paced swap shape for %llu-byte blocks: got %u x %d\n", (unsigned long long)r.block, got.workgroups, got.unroll);
+        }
+    }
+    // the factor a paced launch leaves for the next one: slower when it fell behind or many turns began late,
+    // faster when few did, unchanged in between, and never outside its bounds
+    struct { uint32_t factor; uint32_t late_per_65536; bool behind; int direction; } settle[] = {
+        {65536, 0, true, +1}, {65536, 6554, false, +1}, {65536, 3932, false, +1}, {65536, 3000, false, 0},
+        {65536, 2300, false, -1}, {65536, 655, false, -1}, {kPaceFactorMax, 65535, true, 0}, {kPaceFactorMin, 0, false, 0}};
+    for (const auto& r : settle) {
+        const uint32_t next = next_pace_factor(r.factor, r.late_per_65536, r.behind);
+        const int direction = next > r.factor ? +1 : next < r.factor ? -1 : 0;
+        ++g_cases;
+        if (direction != r.direction || next < kPaceFactorMin || next > kPaceFactorMax) {
+            ++g_failures;
+            std::printf("next_pace_factor(%u, %u, %d) = %u\n", r.factor, r.late_per_65536, (int)r.behind, next);
+        }
+    }
+    ++g_cases;
+    if (pace_factor(nullptr) != kPaceFactorOne) { ++g_failures; std::printf("pace_factor(nullptr)\n"); }
     SwapTuning forced = t;
     forced.beside_pace_mbps = 1;      // an explicit pace (the test of the bounded wait uses 1 MB/s)
     const SwapShape s1 = choose_swap_shape(out | beside, small, bb, 0, 0, forced);

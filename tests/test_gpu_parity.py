@@ -532,6 +532,51 @@ def test_pace_report_accounts_for_every_turn(memory):
     assert capi.get_tuning(capi.KNOB_PACE_REPORT) == 0             # the override ended with the block
 
 
+def test_pace_set_between_launches_keeps_its_account(memory):
+    """A paced throughput-mode swap-out (HFK_KNOB_THROUGHPUT_PACE_PERMILLE != 0) ends by settling, in eight words the
+    library keeps on the device, the factor the next such launch applies to its interval. Every launch is counted,
+    the account of a finished launch is cleared, the factor stays within its bounds and moves the way the late turns
+    say; with HFK_KNOB_ADAPTIVE_PACE off, and for a swap marked HFK_SWAP_BESIDE_COMPUTE, the words are left alone.
+    The bytes are right throughout."""
+    cfg = W.C2_LLAMA8B_SWAP_OUT.scaled(layers=8, dev_blocks=160, host_blocks=160, n_blocks=128)   # 64 MiB per launch
+    bb = cfg.block_bytes
+    cpu = [W.as_bytes(p).clone() for p in _cpu_planes(cfg, cfg.dev_blocks)]
+    dev = [p.to(DEV) for p in cpu]
+    src_ids, dst_ids = W.block_table(cfg, src_blocks=cfg.dev_blocks, dst_blocks=cfg.host_blocks)
+    pairs = W.pairs_tensor(src_ids, dst_ids).to(DEV)
+    dtab = ptr_table(dev)
+    pool, host = _host_pool(memory, cfg, cfg.host_blocks, fill=0x33)
+    htab = host_ptr_table(host)
+    assert cfg.planes * src_ids.numel() * bb >= 64 << 20
+    announce("pace set between launches: %d planes x %d blocks = %d MiB per launch" % (cfg.planes, src_ids.numel(),
+                                                                                      cfg.planes * src_ids.numel() * bb >> 20))
+
+    def launch(flags):
+        capi.check(capi.swap_blocks(htab.data_ptr(), dtab.data_ptr(), pairs.data_ptr(), cfg.planes, src_ids.numel(), bb, bb, bb,
+                                    cfg.dev_blocks, cfg.host_blocks, 0, stream_handle(), flags))
+
+    before = capi.pace_state()
+    with capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: 700}):      # far under the link's limit: no turn is late
+        for _ in range(6):
+            launch(capi.SWAP_DST_HOST)
+        after = capi.pace_state()
+        assert after[5] == before[5] + 6, (before, after)
+        assert after[1:5] == [0, 0, 0, 0], after
+        assert 61000 <= after[0] <= 68157, after
+        assert after[0] < (before[0] or 65536) or after[0] == 61000, (before, after)    # few late turns: the next interval is shorter
+        assert after[6] < 1638, after
+        launch(capi.SWAP_DST_HOST | capi.SWAP_BESIDE_COMPUTE)                # its pace is fixed: no account kept
+        with capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: 700, capi.KNOB_ADAPTIVE_PACE: 0}):
+            launch(capi.SWAP_DST_HOST)
+        assert capi.pace_state() == after
+    launch(capi.SWAP_DST_HOST)                                                # the default is unpaced: nothing to settle
+    assert capi.pace_state() == after
+    for p in range(cfg.planes):
+        want = torch.full((cfg.host_blocks, bb), 0x33, dtype=torch.uint8)
+        O.torch_swap_blocks(want, cpu[p], src_ids, dst_ids)
+        assert torch.equal(host[p], want), "plane %d" % p
+
+
 # ---------------------------------------------------------------------------
 # edge cases
 # ---------------------------------------------------------------------------
