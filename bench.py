@@ -714,7 +714,9 @@ def section_repeat(b, w, steps, warmup, flags, first_value):
         rows = report.cpu().view(64, 8)[:grid]
         ran, allotted, turns, late, worst = (rows[:, i].double() for i in range(5))
         paced["fixed_at_0.%d_of_link" % (permille // 10)] = {
-            "GBps": round(w.payload / (pms * 1e6), 2), "workgroups": grid,
+            "GBps": round(w.payload / (pms * 1e6), 2), "workgroups": grid, "launch_ms": round(pms, 4),
+            "slowest_workgroup_ran_ms": round(float(ran.max()) / 1e5, 4),
+            "allotted_ms": round(float(allotted.max()) / 1e5, 4),
             "ran_over_allotted": round(float((ran / allotted.clamp(min=1)).max()), 4),
             "late_turns_pct": round(100 * float(late.sum() / turns.sum().clamp(min=1)), 2),
             "largest_delay_us": round(float(worst.max()) / 100.0, 1)}

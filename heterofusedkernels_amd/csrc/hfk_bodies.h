@@ -68,7 +68,8 @@ typedef uint32_t vec16 __attribute__((ext_vector_type(4)));
 // [2] late turns of the launch in progress, [3] workgroups finished, [4] workgroups that ended behind
 // schedule, [5] launches settled, [6] late turns per 65536 turns of the last launch, [7] unused.
 // Launches on one stream see each other's result in order; launches that overlap on two streams may
-// read a factor one launch old, which is harmless.
+// read a factor one launch old and may settle on each other's counts, which costs the factor one
+// small step in a wrong direction and nothing else (it is bounded, and the data never depend on it).
 constexpr uint32_t kPaceFactorOne = 65536;
 constexpr uint32_t kPaceFactorMin = 61000;        // the interval may shrink by 7 % ...
 constexpr uint32_t kPaceFactorMax = 68157;        // ... and grow by 4 % from the nominal one: what slows a launch down
@@ -154,7 +155,7 @@ struct Pacer {
         atomicAdd(&state[2], late_turns);
         if (((HFK_TICKS_100MHZ() - t0) << 8) > due_q8 + 2ull * pace_q8) atomicAdd(&state[4], 1u);
         __threadfence();
-        if (atomicAdd(&state[3], 1u) + 1u == nb) {
+        if (atomicAdd(&state[3], 1u) + 1u >= nb) {   // >=: counts mixed up by overlapping launches still get cleared
             __threadfence();
             const uint32_t all_turns = atomicAdd(&state[1], 0u), all_late = atomicAdd(&state[2], 0u);
             const uint32_t behind = atomicAdd(&state[4], 0u);

@@ -286,8 +286,8 @@ constexpr uint64_t kAskTableSideBytes = 64ull << 10;
 //    costs it (one wavefront that only sleeps: 1.50x).
 // Toward the host, throughput mode: unpaced by default, 96 vectors per lane in flight over the grid
 // (12 workgroups x 8 for blocks of 32 KiB and more, see hfk::to_host_shape) with non-temporal loads
-// and PLAIN stores: 56.6-56.7 GB/s on every kind of block table, 0.899 of the link's raw rate and 99 %
-// of what hipMemcpy reaches, against 55.9-56.2 with non-temporal stores (which reach the link as
+// and PLAIN stores: 56.6-56.7 GB/s on every kind of block table (55.9 on a slower host), 0.899 of
+// the link's raw rate and 99 % of what hipMemcpy reaches, against 55.9-56.2 with non-temporal stores (which reach the link as
 // 1.4 % more write requests than the payload has lines; plain ones go through the L2, which hands the
 // link whole lines). It is the fast shape, not the gentle one: a device copy / SDPA / GEMM on another
 // stream runs 5.9x / 2.9x / 4.0x slower meanwhile.

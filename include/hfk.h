@@ -199,8 +199,8 @@ HFK_API int hfk_multi_layer_block_table_transfer(const void* dev_layer_ptrs, uin
  *                   every other kernel's traffic.
  *                 - HFK_SWAP_DST_HOST (swap-out): a swap of 64 MiB or more runs on 12 workgroups x 8
  *                   vectors per lane, unpaced, with non-temporal loads and plain stores (through the
- *                   L2, which hands the link whole lines): 56.6-56.7 GB/s on every block table, 99 % of
- *                   what hipMemcpy reaches toward the host / 5.9x / 4.0x. This is the fast shape, not
+ *                   L2, which hands the link whole lines): 56.6-56.7 GB/s on every block table (55.9
+ *                   on a slower host), 99 % of what hipMemcpy reaches toward the host / 5.9x / 4.0x. This is the fast shape, not
  *                   the gentle one; the gentle one is asked for with HFK_SWAP_BESIDE_COMPUTE. (Paced
  *                   through HFK_KNOB_THROUGHPUT_PACE_PERMILLE it runs on 6 x 4 with non-temporal stores:
  *                   at 890, 55.5-56.0 GB/s / 1.35x / 2.5x.) A shorter one runs as with no flags.
@@ -482,7 +482,7 @@ enum hfk_knob {
 /*
  * The state behind a pace that is set between launches, for the current device: eight words,
  * [0] the factor applied to the interval of the next paced throughput-mode swap-out, in 1/65536
- * (0 = none settled yet, i.e. 1.0; kept within 0.93 .. 1.12), [1]-[4] the account of a launch in
+ * (0 = none settled yet, i.e. 1.0; kept within 0.93 .. 1.04), [1]-[4] the account of a launch in
  * progress, [5] launches settled, [6] late turns per 65536 turns of the last one, [7] unused.
  * Every such launch ends by settling the factor for the next one from how many of its turns began
  * late and whether a workgroup ended behind its schedule: the pace follows what this machine's link

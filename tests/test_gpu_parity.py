@@ -571,6 +571,21 @@ def test_pace_set_between_launches_keeps_its_account(memory):
         assert capi.pace_state() == after
     launch(capi.SWAP_DST_HOST)                                                # the default is unpaced: nothing to settle
     assert capi.pace_state() == after
+    # Paced launches of different grids that overlap on two streams may settle on each other's counts: the account
+    # stays bounded and keeps being cleared, the factor stays within its bounds, and the bytes depend on none of it.
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    for _ in range(4):
+        with capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: 700}):
+            launch(capi.SWAP_DST_HOST)
+        with torch.cuda.stream(side), capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: 700,
+                                                          capi.KNOB_PACED_WORKGROUPS: 12}):
+            launch(capi.SWAP_DST_HOST)
+    torch.cuda.current_stream().wait_stream(side)
+    with capi.thread_tuning({capi.KNOB_THROUGHPUT_PACE_PERMILLE: 700}):
+        launch(capi.SWAP_DST_HOST)
+    mixed = capi.pace_state()
+    assert mixed[3] < 12 and mixed[5] > after[5] and 61000 <= mixed[0] <= 68157, (after, mixed)
     for p in range(cfg.planes):
         want = torch.full((cfg.host_blocks, bb), 0x33, dtype=torch.uint8)
         O.torch_swap_blocks(want, cpu[p], src_ids, dst_ids)
