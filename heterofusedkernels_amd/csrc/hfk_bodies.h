@@ -452,7 +452,7 @@ HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t 
     const uint32_t factor = PACED ? pace_factor(a.pace_state) : kPaceFactorOne;
     Pacer pacer(PACED ? (uint32_t)(((uint64_t)a.pace_q8 * factor) >> 16) : 0u, bid, nb);
     uint64_t id = bid;                  // 64-bit so that id + nb cannot wrap
-    uint32_t judged_pair = 0xffffffffu; // SPLIT: the pair the filter was last evaluated for, and its verdict
+    uint32_t judged_pair = 0xffffffffu; // SPLIT: the pair the filter was last evaluated for, and what it said
     bool judged_selected = false;       // (a workgroup's consecutive items mostly belong to one pair)
     while (id < a.n_work) {
         const uint64_t w = id;
