@@ -260,17 +260,22 @@ struct BlockCopyArgs {
                                  // valid gets zeros written instead of being left alone (a staging buffer
                                  // must never hand an earlier transfer's bytes on to the host)
     // Run filter (RunFilter below): lets one block table be split between two movers, by the length
-    // of the run of consecutive `run_ids` a pair belongs to. run_mode 0 = every pair.
+    // of the run of consecutive `run_ids` a pair belongs to. run_mode 0 = every pair. With
+    // kListedPairs the split has been made beforehand and run_ids is this launch's list of pairs.
     uint32_t run_mode;
-    uint32_t run_min;            // a run is "long" from this many consecutive ids on
-    const int64_t* run_ids;      // entry j at run_ids[j * id_stride]
+    uint32_t run_min;            // a run is "long" from this many consecutive ids on (listed: the table's length)
+    const int64_t* run_ids;      // entry j at run_ids[j * id_stride] (listed: entry i at run_ids[i])
     uint64_t* pace_report;       // null, or where each workgroup of a paced launch leaves Pacer::report
     uint32_t* pace_state;        // null, or the library's eight words for a pace set between launches (pace_factor)
 };
 
 // Which pairs of a block table a launch moves, when the table is split by run length: pair j belongs to
 // the maximal run of entries whose run_ids are consecutive (ids[i + 1] == ids[i] + 1) around it.
-enum RunFilter : uint32_t { kAllPairs = 0, kLongRunsOnly = 1, kShortRunsOnly = 2 };
+// kListedPairs: the launch moves the pairs a list names, in list order: run_ids[i] (stride 1) is the table
+// index of the launch's i-th pair, n_pairs the length of the list, run_min the table's length (an entry
+// that is not below it is skipped: a list is data, and its tail may be unfilled). A side without an id
+// column (a staging buffer) is indexed by the position in the list, not by the table index.
+enum RunFilter : uint32_t { kAllPairs = 0, kLongRunsOnly = 1, kShortRunsOnly = 2, kListedPairs = 3 };
 
 // Length of the maximal run of consecutive ids around entry j, counted no further than `cap`: the
 // result is min(cap, run length). The host uses the same function to decide which runs it copies,
@@ -297,7 +302,8 @@ enum ChunkAction : uint32_t { kSkip = 0, kCopy = 1, kZeroFill = 2 };
 
 // SPLIT selects, at compile time, the variant that honours the run filter; kernels that move whole
 // tables (the hot ones) are built without it and carry none of its code.
-template <typename IdT, bool SPLIT = false>
+// LISTED: the launch's pairs are named by a list (kListedPairs).
+template <typename IdT, bool SPLIT = false, bool LISTED = false>
 HFK_HD ChunkAction resolve_chunk(const BlockCopyArgs<IdT>& a, uint32_t w, uint64_t& s_addr, uint64_t& d_addr,
                                  uint32_t& chunk) {
     chunk = w % a.chunks_per_block;
@@ -315,8 +321,13 @@ HFK_HD ChunkAction resolve_chunk(const BlockCopyArgs<IdT>& a, uint32_t w, uint64
     // comparison, so a work item pays one scalar-load latency, not a chain of them. A workgroup that
     // keeps little in flight (the duplex swap: one vector per lane and direction) is as fast as its
     // iterations are short.
-    const uint64_t sb = a.src_ids ? (uint64_t)(int64_t)table_entry(a.src_ids, (uint64_t)pair * a.id_stride) : (uint64_t)pair;
-    const uint64_t db = a.dst_ids ? (uint64_t)(int64_t)table_entry(a.dst_ids, (uint64_t)pair * a.id_stride) : (uint64_t)pair;
+    uint64_t entry = pair;              // where the pair sits in the block table
+    if constexpr (LISTED) {
+        entry = (uint64_t)table_entry(a.run_ids, pair);
+        if (entry >= a.run_min) return kSkip;
+    }
+    const uint64_t sb = a.src_ids ? (uint64_t)(int64_t)table_entry(a.src_ids, entry * a.id_stride) : (uint64_t)pair;
+    const uint64_t db = a.dst_ids ? (uint64_t)(int64_t)table_entry(a.dst_ids, entry * a.id_stride) : (uint64_t)pair;
     const uint64_t s_plane = a.src_planes ? table_entry(a.src_planes, plane) : a.src_base + (uint64_t)plane * a.src_plane_stride;
     const uint64_t d_plane = a.dst_planes ? table_entry(a.dst_planes, plane) : a.dst_base + (uint64_t)plane * a.dst_plane_stride;
     s_addr = s_plane + sb * a.src_stride;
@@ -447,8 +458,10 @@ HFK_HD void zero_chunk(uint64_t d_addr, uint64_t block_bytes, uint32_t chunk, ui
 // PACED: the launch may be paced (a.pace_q8); kernels that never are (everything HBM-bound) are built
 // without it and carry none of the pacer's code: one workgroup per 4 KiB chunk pays for every
 // instruction of its prologue.
-template <typename IdT, int UNROLL, int NT, bool SPLIT = false, bool PACED = true>
+// LISTED: the launch's pairs come from a list (a.run_mode must be kListedPairs); not together with SPLIT.
+template <typename IdT, int UNROLL, int NT, bool SPLIT = false, bool PACED = true, bool LISTED = false>
 HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t nb, uint32_t tid) {
+    static_assert(!(SPLIT && LISTED), "a launch either filters the table's pairs or is handed a list of them");
     const uint32_t factor = PACED ? pace_factor(a.pace_state) : kPaceFactorOne;
     Pacer pacer(PACED ? (uint32_t)(((uint64_t)a.pace_q8 * factor) >> 16) : 0u, bid, nb);
     uint64_t id = bid;                  // 64-bit so that id + nb cannot wrap
@@ -469,7 +482,7 @@ HFK_HD void block_copy_body(const BlockCopyArgs<IdT>& a, uint32_t bid, uint32_t 
                 continue;
             }
         }
-        const ChunkAction what = resolve_chunk<IdT, SPLIT>(a, (uint32_t)w, s_addr, d_addr, chunk);
+        const ChunkAction what = resolve_chunk<IdT, SPLIT, LISTED>(a, (uint32_t)w, s_addr, d_addr, chunk);
         if (what == kSkip) {            // moves nothing, so it takes no turn on the link either
             id = SPLIT ? next_pair_item(a, w, bid, nb) : id + nb;
             continue;

@@ -59,6 +59,23 @@ __global__ __launch_bounds__(256) void scatter_long_runs_kernel(const BlockCopyA
     hfk::block_copy_body<int64_t, UNROLL, NT, true, false>(a, blockIdx.x, gridDim.x, threadIdx.x);
 }
 
+// The same three again, handed the list of their pairs (hfk::kListedPairs): what hfk_swap_blocks_auto launches
+// when it has room for the lists, so that no workgroup is started for a pair another mover takes.
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void swap_listed_pairs_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT, false, true, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void gather_listed_pairs_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT, false, false, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
+template <int UNROLL, int NT>
+__global__ __launch_bounds__(256) void scatter_listed_pairs_kernel(const BlockCopyArgs<int64_t> a) {
+    hfk::block_copy_body<int64_t, UNROLL, NT, false, false, true>(a, blockIdx.x, gridDim.x, threadIdx.x);
+}
+
 template <int UNROLL, int NT>
 __global__ __launch_bounds__(256) void swap_blocks_kernel(const BlockCopyArgs<int64_t> a) {
     hfk::block_copy_body<int64_t, UNROLL, NT>(a, blockIdx.x, gridDim.x, threadIdx.x);
@@ -141,13 +158,13 @@ __global__ __launch_bounds__(256) void transpose_to_packed_tiled_kernel(const Tr
     }
 }
 
-// Staging slots of a split table whose staging buffer holds only the long runs (see
-// hfk::fill_stage_slots, which states the result): one workgroup walks the table 256 pairs at a time,
-// marks the pairs in long runs, and numbers them with a running prefix sum.
-__global__ __launch_bounds__(256) void stage_slots_kernel(const int64_t* ids, uint32_t stride, uint32_t n, uint32_t min_run,
-                                                          int64_t* slots) {
+// The two lists of a split table (see hfk::fill_pair_lists, which states the result): one workgroup walks
+// the table 256 pairs at a time, marks the pairs in long runs, and numbers both kinds with a running
+// prefix sum; what is left of either list is set to -1.
+__global__ __launch_bounds__(256) void pair_lists_kernel(const int64_t* ids, uint32_t stride, uint32_t n, uint32_t min_run,
+                                                         int64_t* long_list, int64_t* short_list) {
     __shared__ uint32_t scan[256];
-    __shared__ uint32_t carried;
+    __shared__ uint32_t carried;        // pairs in long runs before this round
     const uint32_t tid = threadIdx.x;
     if (tid == 0) carried = 0;
     __syncthreads();
@@ -162,11 +179,18 @@ __global__ __launch_bounds__(256) void stage_slots_kernel(const int64_t* ids, ui
             scan[tid] += add;
             __syncthreads();
         }
-        if (j < n) slots[(uint64_t)j * stride] = is_long ? (int64_t)(carried + scan[tid] - 1u) : 0;
+        if (j < n) {
+            const uint32_t long_before = carried + scan[tid] - is_long;    // pairs in long runs among 0 .. j - 1
+            if (is_long) long_list[long_before] = (int64_t)j;
+            else short_list[j - long_before] = (int64_t)j;
+        }
         __syncthreads();
         if (tid == 255) carried += scan[255];
         __syncthreads();
     }
+    const uint32_t n_long = carried;
+    for (uint32_t i = n_long + tid; i < n; i += 256) long_list[i] = -1;
+    for (uint32_t i = n - n_long + tid; i < n; i += 256) short_list[i] = -1;
 }
 
 // ---- tuning state ---------------------------------------------------------
@@ -459,6 +483,16 @@ int pace_state(uint32_t** out) {
 template <Role ROLE, typename IdT, int UNROLL, int NT>
 void launch_block_copy_one(const BlockCopyArgs<IdT>& a, uint32_t grid, uint32_t lds, hipStream_t s) {
     if constexpr (std::is_same<IdT, int64_t>::value && ROLE != Role::kGatherRows) {
+        if (a.run_mode == hfk::kListedPairs) {
+            if constexpr (ROLE == Role::kSwapBlocks) {
+                hipLaunchKernelGGL((swap_listed_pairs_kernel<UNROLL, NT>), dim3(grid), dim3(256), lds, s, a);
+            } else if constexpr (ROLE == Role::kGatherBlocks) {
+                hipLaunchKernelGGL((gather_listed_pairs_kernel<UNROLL, NT != 0 ? 3 : 0>), dim3(grid), dim3(256), lds, s, a);
+            } else {
+                hipLaunchKernelGGL((scatter_listed_pairs_kernel<UNROLL, NT != 0 ? 3 : 0>), dim3(grid), dim3(256), lds, s, a);
+            }
+            return;
+        }
         if (a.run_mode != hfk::kAllPairs) {   // a split table: non-temporal or plain, nothing in between
             constexpr int SNT = NT != 0 ? 3 : 0;
             if constexpr (ROLE == Role::kSwapBlocks) {
@@ -1191,9 +1225,9 @@ int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs
     if (rc != 0) return rc;
     direct.zero_skipped = out ? 1u : 0u;   // one rule for the whole table, whichever mover takes a pair
     const uint64_t total_bytes = (uint64_t)n_planes * n_pairs * block_bytes;
-    // Staging the copy engines' share takes the host arrays and a buffer. One that holds the whole table
-    // ([n_planes][n_pairs] blocks) is used with pair j in slot j. A smaller one is used compactly if it
-    // holds the blocks of the long runs and, behind them, a table of their slots (16 bytes per pair).
+    // Staging the copy engines' share takes the host arrays and a buffer: one that holds the blocks of the
+    // long runs and, behind them, the two lists of pairs (16 bytes per pair), or one that holds the whole
+    // table ([n_planes][n_pairs] blocks).
     const bool have_arrays = staging != nullptr && host_plane_addrs != nullptr && host_block_ids != nullptr;
     const bool holds_table = have_arrays && staging_bytes / block_bytes / n_pairs >= n_planes;
     uint64_t min_run = min_run_blocks;
@@ -1215,37 +1249,41 @@ int hfk_swap_blocks_auto(const void* dev_plane_ptrs, const void* host_plane_ptrs
         }
         if (min_run <= kMaxRunFilter) long_blocks = hfk::blocks_in_long_runs(host_block_ids, n_pairs, min_run);
     }
-    bool compact = false;
-    uint64_t slots_offset = 0;
-    if (long_blocks != 0 && !holds_table) {
-        if (long_blocks < n_pairs && n_pairs <= 0x7fffffffu && long_blocks <= staging_bytes / block_bytes / n_planes) {
-            slots_offset = (n_planes * long_blocks * block_bytes + 255u) & ~(uint64_t)255u;
-            compact = slots_offset <= staging_bytes && n_pairs <= (staging_bytes - slots_offset) / (2 * sizeof(int64_t));
-        }
-        if (!compact) long_blocks = 0;   // the buffer is too small for this table's long runs: everything goes direct
+    // A table that is split is moved by two lists of pairs, which a one-workgroup kernel of this call writes
+    // behind the staged blocks; the staging buffer then holds the long runs only, in table order. Without room
+    // for the lists (tiny blocks) a buffer that holds the whole table is used with pair j in slot j and the
+    // kernels sort the pairs out themselves (the run filter); a buffer that holds neither is not used.
+    const bool split = long_blocks != 0 && long_blocks < n_pairs;
+    bool listed = false;
+    uint64_t lists_offset = 0;
+    if (split && n_pairs <= 0x7fffffffu && long_blocks <= staging_bytes / block_bytes / n_planes) {
+        lists_offset = (n_planes * long_blocks * block_bytes + 255u) & ~(uint64_t)255u;
+        listed = lists_offset <= staging_bytes && n_pairs <= (staging_bytes - lists_offset) / (2 * sizeof(int64_t));
     }
+    if (long_blocks != 0 && !listed && !holds_table) long_blocks = 0;   // everything goes direct
     if (long_blocks == 0) {   // nothing for the copy engines (or no staging to give them): one direct launch
         return launch_swap(direct, side_flags, 0, total_bytes, s);
     }
     HostLeg leg{host_plane_addrs, host_block_ids, n_planes, n_pairs, block_bytes, host_block_stride, staging, out};
-    leg.compact = compact;
+    leg.compact = listed;
     leg.stage_plane_blocks = long_blocks;
     const int64_t* host_column = block_pairs + (out ? 1 : 0);
     const int64_t* dev_column = block_pairs + (out ? 0 : 1);
-    int64_t* slots = compact ? reinterpret_cast<int64_t*>(static_cast<char*>(staging) + slots_offset) : nullptr;
     BlockCopyArgs<int64_t> hbm;   // long runs: device planes <-> staging, the copy engines do the rest
-    rc = hfk::plan_stage_blocks(hbm, dev_plane_ptrs, staging, dev_column, n_planes, n_pairs, block_bytes,
-                                dev_block_stride, dev_blocks, out, slots, long_blocks);
+    rc = hfk::plan_stage_blocks(hbm, dev_plane_ptrs, staging, dev_column, n_planes, listed ? long_blocks : n_pairs, block_bytes,
+                                dev_block_stride, dev_blocks, out);
     if (rc != 0) return rc;
     hbm.id_stride = 2;
-    if (compact) {   // the slot table, with the block table's stride, computed on the device from the device's table
-        hipLaunchKernelGGL(stage_slots_kernel, dim3(1), dim3(256), 0, s, host_column, 2u, (uint32_t)n_pairs, (uint32_t)min_run,
-                           slots);
+    if (listed) {   // both lists, computed on the device from the device's table
+        int64_t* long_list = reinterpret_cast<int64_t*>(static_cast<char*>(staging) + lists_offset);
+        int64_t* short_list = long_list + n_pairs;
+        hipLaunchKernelGGL(pair_lists_kernel, dim3(1), dim3(256), 0, s, host_column, 2u, (uint32_t)n_pairs, (uint32_t)min_run,
+                           long_list, short_list);
         rc = finish_launch();
         if (rc != 0) return rc;
-    }
-    const bool split = long_blocks < n_pairs;
-    if (split) {
+        hfk::list_pairs(hbm, long_list, (uint32_t)long_blocks, (uint32_t)n_pairs);
+        hfk::list_pairs(direct, short_list, (uint32_t)(n_pairs - long_blocks), (uint32_t)n_pairs);
+    } else if (split) {
         hfk::filter_runs(hbm, hfk::kLongRunsOnly, host_column, (uint32_t)min_run);
         hfk::filter_runs(direct, hfk::kShortRunsOnly, host_column, (uint32_t)min_run);
     }

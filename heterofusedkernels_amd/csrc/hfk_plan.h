@@ -342,14 +342,12 @@ inline int plan_gather_blocks(BlockCopyArgs<int64_t>& a, const void* dst_plane_p
 // The kernel half of a staged swap: blocks between the device planes and a
 // contiguous staging buffer [n_planes][n_blocks][block_bytes] in device memory.
 // to_staging: staging[p][i] = plane_p[ids[i]]  (gather);  else  plane_p[ids[i]] = staging[p][i]  (scatter).
-// `stage_slots` null: pair j's blocks live in staging slot j and a plane of the staging buffer holds
-// n_blocks slots. Otherwise pair j's slot is stage_slots[j * stride] (the caller sets a.id_stride: the
-// slot table is laid out with the stride of the block table it belongs to) and a plane holds
-// `stage_plane_blocks` slots: a staging buffer that holds only the share of the table that is staged.
+// Pair j's blocks live in staging slot j and a plane of the staging buffer holds n_blocks slots. (A launch
+// that is handed a list of pairs, list_pairs(), counts its slots by the position in the list, so a
+// staging buffer that holds only the listed share of a table is planned with n_blocks = that share.)
 inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_ptrs, void* staging,
                              const int64_t* dev_block_ids, uint32_t n_planes, uint64_t n_blocks, uint64_t block_bytes,
-                             uint64_t dev_block_stride, uint64_t dev_blocks, bool to_staging,
-                             const int64_t* stage_slots = nullptr, uint64_t stage_plane_blocks = 0) {
+                             uint64_t dev_block_stride, uint64_t dev_blocks, bool to_staging) {
     if (dev_plane_ptrs == nullptr || staging == nullptr || dev_block_ids == nullptr) return HFK_ERR_NULL_POINTER;
     if (block_bytes == 0 || dev_block_stride < block_bytes) return HFK_ERR_BAD_SIZE;
     if (n_blocks > kU32Max) return HFK_ERR_TOO_LARGE;
@@ -365,8 +363,8 @@ inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_pt
         a.src_stride = dev_block_stride;
         a.src_limit = limit;
         a.dst_base = (uint64_t)(uintptr_t)staging;
-        a.dst_ids = stage_slots;
-        a.dst_plane_stride = (stage_slots ? stage_plane_blocks : n_blocks) * block_bytes;
+        a.dst_ids = nullptr;
+        a.dst_plane_stride = n_blocks * block_bytes;
         a.dst_stride = block_bytes;
         a.dst_limit = kUnchecked;
         // The copies that follow move staging[p][i] to the host whatever ids[i] was (the ids live on the
@@ -379,8 +377,8 @@ inline int plan_stage_blocks(BlockCopyArgs<int64_t>& a, const void* dev_plane_pt
         a.dst_stride = dev_block_stride;
         a.dst_limit = limit;
         a.src_base = (uint64_t)(uintptr_t)staging;
-        a.src_ids = stage_slots;
-        a.src_plane_stride = (stage_slots ? stage_plane_blocks : n_blocks) * block_bytes;
+        a.src_ids = nullptr;
+        a.src_plane_stride = n_blocks * block_bytes;
         a.src_stride = block_bytes;
         a.src_limit = kUnchecked;
     }
@@ -412,20 +410,36 @@ inline uint64_t blocks_in_long_runs(const int64_t* ids, uint64_t n, uint64_t min
     return total;
 }
 
-// Staging slots of a split table whose staging buffer holds only the long runs: pair j of a long run
-// gets slot (number of pairs in long runs before j), written to slots[j * stride]; the entries of
-// other pairs are set to 0 and never used. The sequential statement of what stage_slots_kernel
-// computes in parallel; the copy engines' leg counts the same way as it walks the runs.
-inline void fill_stage_slots(const int64_t* ids, uint32_t stride, uint64_t n, uint64_t min_run, int64_t* slots) {
-    uint64_t next = 0;
+// The two lists a split table is moved by: long_list holds the table indices of the pairs in long runs
+// (runs of at least min_run consecutive ids), short_list those of all other pairs, both in table
+// order; what is left of either array (n entries each) is set to -1. The i-th pair of long_list has
+// staging slot i, which is how the copy engines' leg counts its slots as it walks the runs. The
+// sequential statement of what pair_lists_kernel computes in parallel.
+inline void fill_pair_lists(const int64_t* ids, uint32_t stride, uint64_t n, uint64_t min_run, int64_t* long_list,
+                            int64_t* short_list) {
+    uint64_t n_long = 0, n_short = 0;
     uint64_t first = 0;
     while (first < n) {
         uint64_t len = 1;
         while (first + len < n && ids[(first + len) * stride] == ids[(first + len - 1) * stride] + 1) ++len;
-        for (uint64_t i = 0; i < len; ++i) slots[(first + i) * stride] = len >= min_run ? (int64_t)(next + i) : 0;
-        if (len >= min_run) next += len;
+        for (uint64_t i = 0; i < len; ++i) {
+            if (len >= min_run) long_list[n_long++] = (int64_t)(first + i);
+            else short_list[n_short++] = (int64_t)(first + i);
+        }
         first += len;
     }
+    for (uint64_t i = n_long; i < n; ++i) long_list[i] = -1;
+    for (uint64_t i = n_short; i < n; ++i) short_list[i] = -1;
+}
+
+// Hands a planned block copy over a table of n_total pairs the list of the n_listed pairs it is to move
+// (BlockCopyArgs::run_mode kListedPairs).
+template <typename IdT>
+inline void list_pairs(BlockCopyArgs<IdT>& a, const int64_t* list, uint32_t n_listed, uint32_t n_total) {
+    a.run_mode = kListedPairs;
+    a.run_ids = list;
+    a.run_min = n_total;
+    a.n_pairs = n_listed;
 }
 
 // Restricts a planned block copy to the pairs in long (or short) runs of `run_ids`

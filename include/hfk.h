@@ -388,8 +388,10 @@ HFK_API int hfk_swap_blocks_staged_static(const void* dev_plane_ptrs, void* cons
  *   staging           device buffer (256-byte aligned), or NULL; staging_bytes its size.
  *                     n_planes * n_pairs * block_bytes always suffices. A smaller buffer is used when
  *                     it holds the staged share alone: n_planes * (blocks in runs of k or more) *
- *                     block_bytes, rounded up to 256, plus 16 bytes per pair for the table of staging
- *                     slots, which a one-workgroup kernel of the same call fills from block_pairs
+ *                     block_bytes, rounded up to 256, plus 16 bytes per pair for the two lists of pairs
+ *                     (those in long runs, and the others) that a one-workgroup kernel of the same call
+ *                     writes from block_pairs and the call's other launches are handed. A buffer with
+ *                     room for both is used that way even if it could hold the whole table
  *   flags             0 or HFK_SWAP_BESIDE_COMPUTE (shape of the direct launch, see hfk_swap_blocks;
  *                     the host side is named by to_host)
  * All work is enqueued on `stream` in order. Destination blocks must be distinct.

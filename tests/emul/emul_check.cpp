@@ -78,6 +78,16 @@ void run_block_copy(BlockCopyArgs<IdT> a, int preferred_unroll, uint32_t grid_ca
     int unroll = 1;   // whole_chunks: as the launcher plans every role but the swap
     if (plan_block_copy<IdT>(a, preferred_unroll, &unroll, whole_chunks) != HFK_OK) { std::printf("plan failed\n"); ++g_failures; return; }
     const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+    if (a.run_mode == kListedPairs) {   // a launch that is handed its pairs runs the bodies built for a list
+        switch (unroll) {
+            case 1: walk(a, grid, block_copy_body<IdT, 1, NT, false, true, true>); break;
+            case 2: walk(a, grid, block_copy_body<IdT, 2, NT, false, true, true>); break;
+            case 4: walk(a, grid, block_copy_body<IdT, 4, NT, false, true, true>); break;
+            case 8: walk(a, grid, block_copy_body<IdT, 8, NT, false, true, true>); break;
+            default: walk(a, grid, block_copy_body<IdT, 16, NT, false, true, true>); break;
+        }
+        return;
+    }
     if (a.run_mode != kAllPairs) {   // a split table runs the bodies built with the run filter, as the launcher does
         switch (unroll) {
             case 1: walk(a, grid, block_copy_body<IdT, 1, NT, true>); break;
@@ -347,16 +357,25 @@ void case_auto(uint32_t n_planes, uint32_t n_pairs, uint64_t block_bytes, uint32
         pairs[2 * j] = to_host ? dev_ids[j] : host_ids[j];
         pairs[2 * j + 1] = to_host ? host_ids[j] : dev_ids[j];
     }
-    // Every other case stages compactly: a buffer that holds exactly the long runs (a slot beyond it would be an
-    // access the sanitizer reports), slots from fill_stage_slots, which states what the slot kernel computes.
+    // Every other case is moved by lists of pairs: a buffer that holds exactly the long runs (a slot beyond it would
+    // be an access the sanitizer reports), lists from fill_pair_lists, which states what the list kernel computes.
+    // The others keep a buffer for the whole table and let the kernels filter the pairs.
     static unsigned auto_cases = 0;
     const uint64_t long_blocks = blocks_in_long_runs(host_ids.data(), n_pairs, min_run);
     const bool compact = (auto_cases++ % 2 == 1) && long_blocks != 0 && long_blocks < n_pairs;
     const uint64_t plane_slots = compact ? long_blocks : n_pairs;
     Buf staging((uint64_t)n_planes * plane_slots * block_bytes);
     staging.randomize();
-    std::vector<int64_t> slots(2 * (size_t)n_pairs, -1);
-    if (compact) fill_stage_slots(pairs.data() + (to_host ? 1 : 0), 2, n_pairs, min_run, slots.data());
+    std::vector<int64_t> long_list(n_pairs, 0), short_list(n_pairs, 0);
+    if (compact) {
+        fill_pair_lists(pairs.data() + (to_host ? 1 : 0), 2, n_pairs, min_run, long_list.data(), short_list.data());
+        uint64_t listed = 0;                     // every pair is in exactly one list, each list in table order
+        for (uint32_t i = 0; i < n_pairs; ++i) listed += (long_list[i] >= 0) + (short_list[i] >= 0);
+        if (listed != n_pairs || long_list[long_blocks - 1] < 0 || long_list[long_blocks] != -1) {
+            ++g_failures;
+            std::printf("case_auto: lists name %llu of %u pairs\n", (unsigned long long)listed, n_pairs);
+        }
+    }
     // expected
     for (uint32_t p = 0; p < n_planes; ++p)
         for (uint32_t j = 0; j < n_pairs; ++j) {
@@ -377,13 +396,18 @@ void case_auto(uint32_t n_planes, uint32_t n_pairs, uint64_t block_bytes, uint32
                                         block_bytes, dev_blocks, host_blocks)
                      : plan_swap_blocks(direct, dp.data(), hp.data(), pairs.data(), n_planes, n_pairs, block_bytes, block_bytes,
                                         block_bytes, host_blocks, dev_blocks);
-    if (rc == HFK_OK) rc = plan_stage_blocks(hbm, dp.data(), staging.p, dev_column, n_planes, n_pairs, block_bytes, block_bytes,
-                                             dev_blocks, to_host, compact ? slots.data() : nullptr, plane_slots);
+    if (rc == HFK_OK) rc = plan_stage_blocks(hbm, dp.data(), staging.p, dev_column, n_planes, plane_slots, block_bytes, block_bytes,
+                                             dev_blocks, to_host);
     if (rc != HFK_OK) { ++g_failures; std::printf("case_auto plan rc=%d\n", rc); return; }
     direct.zero_skipped = to_host ? 1u : 0u;
     hbm.id_stride = 2;
-    filter_runs(hbm, kLongRunsOnly, host_column, min_run);
-    filter_runs(direct, kShortRunsOnly, host_column, min_run);
+    if (compact) {
+        list_pairs(hbm, long_list.data(), (uint32_t)long_blocks, n_pairs);
+        list_pairs(direct, short_list.data(), (uint32_t)(n_pairs - long_blocks), n_pairs);
+    } else {
+        filter_runs(hbm, kLongRunsOnly, host_column, min_run);
+        filter_runs(direct, kShortRunsOnly, host_column, min_run);
+    }
     auto copies = [&]() {
         uint64_t staged_before = 0;      // as the copy engines' leg counts its slots
         for_each_host_run(host_ids.data(), n_pairs, [&](uint64_t first, uint64_t len) {
