@@ -476,6 +476,49 @@ void case_auto_with_disagreeing_columns() {
     expect_equal(host.p, want.p, host.n, "run-splitting swap with disagreeing host columns");
 }
 
+// The same disagreement when the call moves its pairs by lists (a table that is split, a buffer with room for the
+// lists). The array calls pairs 0-2 one long run and pair 3 a single slot, so three staging slots are copied to the
+// array's slots and the direct launch covers one position of the short list; the table has no long run at all, so
+// its long list is empty (every entry -1: the staging kernel moves nothing) and its short list starts with pair 0.
+// Pair 0 ends up right, pairs 1-3 are not moved, and the array's slots 11 and 12 hold what staging held before.
+void case_auto_listed_with_disagreeing_columns() {
+    const uint64_t bb = 4096;
+    const uint32_t n = 4, dev_blocks = 8, host_blocks = 40, min_run = 2;
+    Buf dev(dev_blocks * bb), host(host_blocks * bb), staging(3 * bb);
+    dev.randomize();
+    host.fill(0x11);
+    staging.fill(0xEE);
+    const int64_t array_ids[n] = {10, 11, 12, 20}, table_ids[n] = {10, 30, 12, 20}, dev_ids[n] = {3, 1, 7, 5};
+    std::vector<int64_t> pairs;
+    for (uint32_t j = 0; j < n; ++j) { pairs.push_back(dev_ids[j]); pairs.push_back(table_ids[j]); }
+    const uint64_t long_blocks = blocks_in_long_runs(array_ids, n, min_run);            // the host's count: 3
+    std::vector<int64_t> long_list(n), short_list(n);
+    fill_pair_lists(pairs.data() + 1, 2, n, min_run, long_list.data(), short_list.data());   // the device's lists
+    uint64_t dp[1] = {(uint64_t)(uintptr_t)dev.p}, hp[1] = {(uint64_t)(uintptr_t)host.p};
+    BlockCopyArgs<int64_t> direct, hbm;
+    int rc = plan_swap_blocks(direct, hp, dp, pairs.data(), 1, n, bb, bb, bb, dev_blocks, host_blocks);
+    if (rc == HFK_OK) rc = plan_stage_blocks(hbm, dp, staging.p, pairs.data(), 1, long_blocks, bb, bb, dev_blocks, true);
+    if (rc != HFK_OK || long_blocks != 3) { ++g_failures; std::printf("disagreeing columns, listed: plan rc=%d\n", rc); return; }
+    direct.zero_skipped = 1;
+    hbm.id_stride = 2;
+    list_pairs(hbm, long_list.data(), (uint32_t)long_blocks, n);
+    list_pairs(direct, short_list.data(), (uint32_t)(n - long_blocks), n);
+    run_block_copy<int64_t, 3>(hbm, 1, 4, true);
+    uint64_t staged_before = 0;
+    for_each_host_run(array_ids, n, [&](uint64_t first, uint64_t len) {
+        if (len < min_run) return;
+        std::memcpy(host.p + (uint64_t)array_ids[first] * bb, staging.p + staged_before * bb, len * bb);
+        staged_before += len;
+    });
+    run_block_copy<int64_t, 3>(direct, 1, 4);
+    Buf want(host_blocks * bb);
+    want.fill(0x11);
+    std::memset(want.p + 11 * bb, 0xEE, bb);
+    std::memset(want.p + 12 * bb, 0xEE, bb);
+    std::memcpy(want.p + 10 * bb, dev.p + 3 * bb, bb);    // staging's stale bytes first, then pair 0 by the direct launch
+    expect_equal(host.p, want.p, host.n, "run-splitting swap by lists with disagreeing host columns");
+}
+
 // ---- gather_blocks (multi-plane, shared ids) -------------------------------
 void case_gather_blocks(uint32_t n_planes, uint32_t n_ids, uint64_t block_bytes, uint64_t src_blocks, int unroll,
                         uint32_t grid_cap) {
@@ -889,6 +932,7 @@ int main() {
             }
 
     case_auto_with_disagreeing_columns();
+    case_auto_listed_with_disagreeing_columns();
 
     // block-table transfer, both directions
     for (bool to_packed : {false, true}) {
