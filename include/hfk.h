@@ -471,15 +471,15 @@ enum hfk_knob {
     HFK_KNOB_TRANSFER_PACE_PERMILLE = 15, /* the same for a block-table transfer into a packed pool in host
                                        memory; 0 (default) = unpaced                                            */
     HFK_KNOB_TRANSFER_UNROLL = 16,  /* 16-byte units per lane of that transfer, 2 or 8 (default 8)              */
+    HFK_KNOB_CHECK_HOST_COLUMN = 17, /* debugging aid, default 0: hfk_swap_blocks_auto first waits for its stream,
+                                       reads block_pairs back and compares its host column with host_block_ids;
+                                       a difference rejects the call with HFK_ERR_TABLE_MISMATCH                */
     HFK_KNOB_TRANSFER_TILED = 18,   /* 1 (default): a block-table transfer into a packed pool in host memory goes through
                                        LDS tiles where its geometry allows (1 KiB runs on both sides); 0: always
                                        row by row                                                               */
-    HFK_KNOB_ADAPTIVE_PACE = 19,    /* 1 (default): a paced throughput-mode swap-out (HFK_KNOB_THROUGHPUT_PACE_PERMILLE != 0)
+    HFK_KNOB_ADAPTIVE_PACE = 19     /* 1 (default): a paced throughput-mode swap-out (HFK_KNOB_THROUGHPUT_PACE_PERMILLE != 0)
                                        takes its interval times a factor that the paced launches before it on this
                                        device have settled (see hfk_pace_state); 0: the interval as computed        */
-    HFK_KNOB_CHECK_HOST_COLUMN = 17 /* debugging aid, default 0: hfk_swap_blocks_auto first waits for its stream,
-                                       reads block_pairs back and compares its host column with host_block_ids;
-                                       a difference rejects the call with HFK_ERR_TABLE_MISMATCH                */
 };
 /*
  * The state behind a pace that is set between launches, for the current device: eight words,
