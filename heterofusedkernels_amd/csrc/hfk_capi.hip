@@ -158,22 +158,72 @@ __global__ __launch_bounds__(256) void transpose_to_packed_tiled_kernel(const Tr
     }
 }
 
-// The two lists of a split table (see hfk::fill_pair_lists, which states the result): one workgroup walks
-// the table 256 pairs at a time, marks the pairs in long runs, and numbers both kinds with a running
-// prefix sum; what is left of either list is set to -1.
+// The two lists of a split table (see hfk::fill_pair_lists, which states the result), by one workgroup in three
+// passes over the table, 256 pairs at a time, each pass a scan with a value carried from round to round. No
+// pass looks further than a pair's neighbour, so the cost does not depend on how long the runs are or on the
+// threshold. short_list doubles as the scratch of the first two passes: the third reads an entry before any
+// lane of its round writes, and a pair's place in the short list is never behind the pair.
+//   1, forward:  where the run a pair belongs to starts (the last pair at or before it whose predecessor's id
+//                is not its own less one), into short_list[j];
+//   2, backward: where the next run starts (the first such pair after it, or n), hence the run's length, hence
+//                whether the pair is in a long run, into short_list[j];
+//   3, forward:  both lists by a running count of the pairs in long runs; what is left of either list is -1.
 __global__ __launch_bounds__(256) void pair_lists_kernel(const int64_t* ids, uint32_t stride, uint32_t n, uint32_t min_run,
                                                          int64_t* long_list, int64_t* short_list) {
     __shared__ uint32_t scan[256];
-    __shared__ uint32_t carried;        // pairs in long runs before this round
+    __shared__ uint32_t carried;
     const uint32_t tid = threadIdx.x;
-    if (tid == 0) carried = 0;
+    constexpr uint32_t kNone = 0xffffffffu;
+    if (tid == 0) carried = 0;           // pass 1: start of the run that reaches into this round
     __syncthreads();
     for (uint32_t base = 0; base < n; base += 256) {
         const uint32_t j = base + tid;
-        const uint32_t is_long = j < n && hfk::run_length_capped(ids, stride, n, j, min_run) >= min_run ? 1u : 0u;
+        const bool starts = j < n && (j == 0 || hfk::table_entry(ids, (uint64_t)(j - 1) * stride) + 1 !=
+                                                    hfk::table_entry(ids, (uint64_t)j * stride));
+        scan[tid] = starts ? j : 0u;
+        __syncthreads();
+        for (uint32_t step = 1; step < 256; step <<= 1) {     // inclusive maximum over the lanes up to this one
+            const uint32_t other = tid >= step ? scan[tid - step] : 0u;
+            __syncthreads();
+            if (other > scan[tid]) scan[tid] = other;
+            __syncthreads();
+        }
+        const uint32_t start = scan[tid] > carried ? scan[tid] : carried;
+        if (j < n) short_list[j] = (int64_t)start;
+        __syncthreads();
+        if (tid == 255) carried = start;
+        __syncthreads();
+    }
+    if (tid == 0) carried = n;           // pass 2: where the first run after this round starts
+    __syncthreads();
+    for (uint32_t base = ((n - 1) / 256) * 256;; base -= 256) {
+        const uint32_t j = base + tid;
+        const uint32_t start = j < n ? (uint32_t)short_list[j] : 0u;
+        scan[tid] = (j < n && start == j) ? j : kNone;
+        __syncthreads();
+        for (uint32_t step = 1; step < 256; step <<= 1) {     // inclusive minimum over the lanes from this one on
+            const uint32_t other = tid + step < 256 ? scan[tid + step] : kNone;
+            __syncthreads();
+            if (other < scan[tid]) scan[tid] = other;
+            __syncthreads();
+        }
+        uint32_t next = tid < 255 ? scan[tid + 1] : kNone;    // the first start after this pair
+        if (carried < next) next = carried;
+        const uint32_t first_start = scan[0] < carried ? scan[0] : carried;
+        __syncthreads();
+        if (j < n) short_list[j] = (next - start >= min_run) ? 1 : 0;
+        if (tid == 0) carried = first_start;
+        __syncthreads();
+        if (base == 0) break;
+    }
+    if (tid == 0) carried = 0;           // pass 3: pairs in long runs before this round
+    __syncthreads();
+    for (uint32_t base = 0; base < n; base += 256) {
+        const uint32_t j = base + tid;
+        const uint32_t is_long = j < n && short_list[j] != 0 ? 1u : 0u;
         scan[tid] = is_long;
         __syncthreads();
-        for (uint32_t step = 1; step < 256; step <<= 1) {     // inclusive scan over the workgroup
+        for (uint32_t step = 1; step < 256; step <<= 1) {     // inclusive sum over the lanes up to this one
             const uint32_t add = tid >= step ? scan[tid - step] : 0u;
             __syncthreads();
             scan[tid] += add;

@@ -413,6 +413,76 @@ def test_random_swap_blocks_auto(seed):
         assert np.array_equal(dev.now(), want_dev), "device side"
 
 
+def _pair_lists(host_ids, min_run):
+    """What hfk::fill_pair_lists states: table indices of the pairs in runs of at least min_run consecutive ids,
+    and of all others, each in table order and padded with -1 to the table's length."""
+    n = host_ids.shape[0]
+    starts = np.flatnonzero(np.r_[True, host_ids[1:] != host_ids[:-1] + 1])
+    run_len = np.ones(n, dtype=np.int64)
+    for first, last in zip(starts, np.r_[starts[1:], n]):
+        run_len[first:last] = last - first
+    is_long = run_len >= min_run
+    pad = lambda a: np.r_[a, np.full(n - a.shape[0], -1)].astype(np.int64)      # noqa: E731
+    return pad(np.flatnonzero(is_long)), pad(np.flatnonzero(~is_long))
+
+
+@pytest.mark.parametrize("min_run", [2, 7, 64, 300, 1024])
+def test_run_splitting_swap_on_a_long_table(min_run):
+    """A table of 1500 pairs (six rounds of the list kernel's 256) whose runs of host slots are 1 to 700 long, split
+    at thresholds from 2 to 1024, out and back: the bytes against the oracle, and the two lists the call leaves
+    behind its compact staging against their sequential statement."""
+    rng = np.random.default_rng(9100 + min_run + 17 * SEED_OFFSET)
+    n_planes, bb, dev_blocks, host_blocks = 2, 512, 2048, 6000
+    lengths = [700, 1, 1, 299, 300, 2, 63, 64, 65, 1, 3]
+    runs, at = [], 0
+    for length in lengths:
+        runs.append(np.arange(at, at + length, dtype=np.int64))
+        at += length + 1 + int(rng.integers(0, 3))
+    host_ids = np.concatenate([runs[i] for i in rng.permutation(len(runs))])
+    n = host_ids.shape[0]
+    assert n == sum(lengths) == 1499 and at <= host_blocks
+    dev_ids = rng.permutation(dev_blocks)[:n].astype(np.int64)
+    long_list, short_list = _pair_lists(host_ids, min_run)
+    long_blocks = int((long_list >= 0).sum())
+    lists_offset = (n_planes * long_blocks * bb + 255) // 256 * 256
+    staging_bytes = lists_offset + 16 * n
+    for to_host in (True, False):
+        announce("long table, min_run %d, to_host %s: %d pairs, %d in long runs" % (min_run, to_host, n, long_blocks))
+        dev = Arena(n_planes * dev_blocks * bb, False, rng)
+        host = Arena(n_planes * host_blocks * bb, True, rng)
+        dtab = _table(_planes(dev.addr, 0, n_planes, dev_blocks, bb))
+        htab = _table(_planes(host.addr, 0, n_planes, host_blocks, bb))
+        host_addrs = (ctypes.c_void_p * n_planes)(*_planes(host.host_addr, 0, n_planes, host_blocks, bb))
+        pairs = np.stack([dev_ids, host_ids] if to_host else [host_ids, dev_ids], 1).astype(np.int64)
+        pairs_d = torch.from_numpy(pairs).to(DEV)
+        staging = torch.full((staging_bytes + 4096,), 0xC3, dtype=torch.uint8, device=DEV)
+        capi.check(capi.swap_blocks_auto(dtab.data_ptr(), htab.data_ptr(), host_addrs, pairs_d.data_ptr(), host_ids.ctypes.data,
+                                         n_planes, n, bb, bb, bb, dev_blocks, host_blocks, staging.data_ptr(), staging_bytes,
+                                         int(to_host), min_run, capi.SWAP_BESIDE_COMPUTE, stream_handle()), "hfk_swap_blocks_auto")
+        torch.cuda.synchronize()
+        assert bool((staging[staging_bytes:] == 0xC3).all()), "staging was written beyond the size given"
+        if 0 < long_blocks < n:      # the table is split: the call wrote its lists
+            lists = staging[lists_offset:staging_bytes].cpu().numpy().view(np.int64)
+            assert np.array_equal(lists[:n], long_list), "list of the pairs in long runs"
+            assert np.array_equal(lists[n:], short_list), "list of the other pairs"
+        want_host, want_dev = host.before.copy(), dev.before.copy()
+        for p in range(n_planes):
+            d = _view(want_dev if not to_host else dev.before, 0, p, dev_blocks, bb, bb)
+            h = _view(want_host if to_host else host.before, 0, p, host_blocks, bb, bb)
+            if to_host:
+                h[host_ids] = d[dev_ids]
+            else:
+                d[dev_ids] = h[host_ids]
+        for p in range(n_planes):      # the same planes through the C oracle
+            src_buf, dst_buf = (dev.before, host.before) if to_host else (host.before, dev.before)
+            sb, db = (dev_blocks, host_blocks) if to_host else (host_blocks, dev_blocks)
+            chk = np.ascontiguousarray(_view(dst_buf, 0, p, db, bb, bb))
+            O.c_swap_blocks([chk], [np.ascontiguousarray(_view(src_buf, 0, p, sb, bb, bb))], pairs)
+            assert np.array_equal(chk, _view(want_host if to_host else want_dev, 0, p, db, bb, bb))
+        assert np.array_equal(host.now(), want_host), "host side"
+        assert np.array_equal(dev.now(), want_dev), "device side"
+
+
 @pytest.mark.parametrize("to_host", [True, False])
 def test_auto_swap_refuses_a_host_array_that_differs_from_the_table(to_host):
     """HFK_KNOB_CHECK_HOST_COLUMN: the host array of host slots and the device table's host column are two
