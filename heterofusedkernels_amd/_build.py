@@ -16,7 +16,6 @@ Run as ``python -m heterofusedkernels_amd._build`` or through ``build_all()``.
 import os
 import shutil
 import subprocess
-import sys
 import sysconfig
 import time
 

@@ -2,7 +2,6 @@
 the C-ABI. torch provides device memory and streams only."""
 import sys
 
-import numpy as np
 import torch
 
 from heterofusedkernels_amd import capi
