@@ -513,6 +513,9 @@ def section_staged(b, w, steps, warmup, out_flags):
             "auto_fragmented_beside_compute_in": lambda st: auto(False, beside, 0, st),
             "staged_fragmented_out": lambda st: staged(True, w.ids_dev, frag_host, st),
             "staged_fragmented_in": lambda st: staged(False, back_dev, frag_host, st)}
+    for k in (2, 8):      # the other ends of the trade-off: more of the table on the copy engines, or less
+        ways["auto_fragmented_beside_compute_out_min_run_%d" % k] = lambda st, k=k: auto(True, beside, k, st)
+        ways["auto_fragmented_beside_compute_in_min_run_%d" % k] = lambda st, k=k: auto(False, beside, k, st)
     # The floor: kernels that touch no memory at all and only stay resident (one sleeping wavefront; 16 workgroups)
     bench_lib = ctypes.CDLL(b.build.HFK_BENCH_SO)
     bench_lib.hfkb_idle_resident.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p]
