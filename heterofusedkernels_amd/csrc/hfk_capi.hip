@@ -159,10 +159,10 @@ __global__ __launch_bounds__(256) void transpose_to_packed_tiled_kernel(const Tr
 }
 
 // The two lists of a split table (see hfk::fill_pair_lists, which states the result), by one workgroup in three
-// passes over the table, 256 pairs at a time, each pass a scan with a value carried from round to round. No
+// passes over the table, 256 pairs at a time, each pass a scan with a value carried from batch to batch. No
 // pass looks further than a pair's neighbour, so the cost does not depend on how long the runs are or on the
 // threshold. short_list doubles as the scratch of the first two passes: the third reads an entry before any
-// lane of its round writes, and a pair's place in the short list is never behind the pair.
+// lane of its batch writes, and a pair's place in the short list is never behind the pair.
 //   1, forward:  where the run a pair belongs to starts (the last pair at or before it whose predecessor's id
 //                is not its own less one), into short_list[j];
 //   2, backward: where the next run starts (the first such pair after it, or n), hence the run's length, hence
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(256) void pair_lists_kernel(const int64_t* ids, uin
     __shared__ uint32_t carried;
     const uint32_t tid = threadIdx.x;
     constexpr uint32_t kNone = 0xffffffffu;
-    if (tid == 0) carried = 0;           // pass 1: start of the run that reaches into this round
+    if (tid == 0) carried = 0;           // pass 1: start of the run that reaches into this batch
     __syncthreads();
     for (uint32_t base = 0; base < n; base += 256) {
         const uint32_t j = base + tid;
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256) void pair_lists_kernel(const int64_t* ids, uin
         if (tid == 255) carried = start;
         __syncthreads();
     }
-    if (tid == 0) carried = n;           // pass 2: where the first run after this round starts
+    if (tid == 0) carried = n;           // pass 2: where the first run after this batch starts
     __syncthreads();
     for (uint32_t base = ((n - 1) / 256) * 256;; base -= 256) {
         const uint32_t j = base + tid;
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void pair_lists_kernel(const int64_t* ids, uin
         __syncthreads();
         if (base == 0) break;
     }
-    if (tid == 0) carried = 0;           // pass 3: pairs in long runs before this round
+    if (tid == 0) carried = 0;           // pass 3: pairs in long runs before this batch
     __syncthreads();
     for (uint32_t base = 0; base < n; base += 256) {
         const uint32_t j = base + tid;

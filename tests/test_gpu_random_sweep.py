@@ -428,7 +428,7 @@ def _pair_lists(host_ids, min_run):
 
 @pytest.mark.parametrize("min_run", [2, 7, 64, 300, 1024])
 def test_run_splitting_swap_on_a_long_table(min_run):
-    """A table of 1500 pairs (six rounds of the list kernel's 256) whose runs of host slots are 1 to 700 long, split
+    """A table of 1500 pairs (six batches of the list kernel's 256) whose runs of host slots are 1 to 700 long, split
     at thresholds from 2 to 1024, out and back: the bytes against the oracle, and the two lists the call leaves
     behind its compact staging against their sequential statement."""
     rng = np.random.default_rng(9100 + min_run + 17 * SEED_OFFSET)
