@@ -31,6 +31,7 @@ KNOB_TRANSFER_UNROLL = 16
 KNOB_CHECK_HOST_COLUMN = 17
 KNOB_TRANSFER_TILED = 18
 KNOB_ADAPTIVE_PACE = 19
+KNOB_FUSED_COPY_ENGINE = 20
 SWAP_DST_HOST = 1
 SWAP_SRC_HOST = 2
 SWAP_BESIDE_COMPUTE = 4

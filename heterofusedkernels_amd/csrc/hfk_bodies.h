@@ -654,6 +654,8 @@ struct TransposeArgs {
     uint32_t pace_q8;            // see Pacer; 0 = unpaced
     uint32_t tile_tokens;        // tiled form only (plan_transpose_tiles): tokens and packed rows per tile;
     uint32_t tile_rows;          // chunks_per_block is then the number of tiles per block
+    uint64_t mirror;             // 0, or (transfer out of the packed side only) the address of a second copy of the
+                                 // packed blocks, same strides: every unit read is also written there as it is
 };
 
 // Where the body finds layer l's address. The layer differs from lane to lane (a 128-byte row is 8
@@ -755,12 +757,17 @@ HFK_HD void transpose_store(const TransposeArgs& a, const TransposeItem& it, con
         if (g64 < a.total_units) {
             if constexpr (TO_PACKED) {
                 store_unit<NT>(global_out<V>(it.packed_addr) + g64, v[u]);
-            } else if ((layered_addr[u] & (sizeof(V) - 1)) == 0) {
-                store_unit<NT>(global_out<V>(layered_addr[u]), v[u]);
-            } else {  // byte stores for a misaligned layer cache
-                HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(layered_addr[u]);
-                for (uint32_t k = 0; k < sizeof(V); ++k) {
-                    d1[k] = unit_byte(v[u], k);
+            } else {
+                if ((layered_addr[u] & (sizeof(V) - 1)) == 0) {
+                    store_unit<NT>(global_out<V>(layered_addr[u]), v[u]);
+                } else {  // byte stores for a misaligned layer cache
+                    HFK_GLOBAL uint8_t* d1 = global_out<uint8_t>(layered_addr[u]);
+                    for (uint32_t k = 0; k < sizeof(V); ++k) {
+                        d1[k] = unit_byte(v[u], k);
+                    }
+                }
+                if (a.mirror != 0) {   // the packed block as it is, for the caller's staging buffer
+                    store_unit<NT>(global_out<V>(a.mirror + (it.packed_addr - a.packed)) + g64, v[u]);
                 }
             }
         }

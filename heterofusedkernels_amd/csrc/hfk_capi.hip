@@ -264,7 +264,7 @@ __global__ __launch_bounds__(256) void pair_lists_kernel(const int64_t* ids, uin
 // Every knob has a process-wide value (hfk_set_tuning) and, per thread, an optional override that
 // lasts from hfk_thread_tuning_begin to hfk_thread_tuning_end: a caller that wants a launch shape
 // of its own for a few calls changes nothing another thread can see.
-constexpr int kKnobCount = 20;
+constexpr int kKnobCount = 21;
 std::atomic<int64_t> g_knob[kKnobCount] = {
     1,       // HFK_KNOB_UNROLL
     3,       // HFK_KNOB_NONTEMPORAL
@@ -286,6 +286,7 @@ std::atomic<int64_t> g_knob[kKnobCount] = {
     0,       // HFK_KNOB_CHECK_HOST_COLUMN
     1,       // HFK_KNOB_TRANSFER_TILED
     1,       // HFK_KNOB_ADAPTIVE_PACE
+    0,       // HFK_KNOB_FUSED_COPY_ENGINE
 };
 
 struct ThreadTuning {
@@ -321,7 +322,8 @@ bool knob_value_valid(int k, int64_t v) {
         case HFK_KNOB_TRANSFER_UNROLL: return v == 2 || v == 8;
         case HFK_KNOB_CHECK_HOST_COLUMN:
         case HFK_KNOB_TRANSFER_TILED:
-        case HFK_KNOB_ADAPTIVE_PACE: return v == 0 || v == 1;
+        case HFK_KNOB_ADAPTIVE_PACE:
+        case HFK_KNOB_FUSED_COPY_ENGINE: return v == 0 || v == 1;
         default: return false;
     }
 }
@@ -738,8 +740,9 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
                      uint64_t packed_stride, uint64_t layered_stride, uint64_t packed_blocks,
                      uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t elem_bytes,
                      bool to_packed, int packed_side, uint32_t workgroups, hipStream_t s,
-                     bool beside_compute = false) {
+                     bool beside_compute = false, void* mirror = nullptr) {
     if (dev_layer_ptrs == nullptr || packed == nullptr) return HFK_ERR_NULL_POINTER;
+    if (mirror != nullptr && to_packed) return HFK_ERR_BAD_FLAGS;
     // With the packed side in host memory the PCIe link is the bound and a small grid does; an
     // unknown pointer gets the small grid too. Measured on the reference's four shapes, 8 blocks per
     // launch: host -> device (two units per lane) 56.0-57.0 GB/s on 16 workgroups, 57.1-57.6 on 24-36,
@@ -759,7 +762,7 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     TransposeArgs a;
     uint32_t unit = 16;
     int rc = hfk::plan_transpose(a, &unit, dev_layer_ptrs, packed, pairs, n_pairs, packed_stride, layered_stride,
-                                 packed_blocks, layered_blocks, T, L, H, D, elem_bytes, unroll);
+                                 packed_blocks, layered_blocks, T, L, H, D, elem_bytes, unroll, mirror);
     if (rc != 0) return rc;
     if (a.n_work == 0) return HFK_OK;  // nothing to move
     int tiled_unroll = 0;
@@ -1118,6 +1121,20 @@ int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs, cons
     const uint64_t bytes = (uint64_t)T * L * H * D * elem_bytes;
     if (bytes == 0) return HFK_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // A block in pinned, device-mapped host memory is read over the link once, by the kernel of the direct
+    // transfer, which writes every unit to its layer and to the staging buffer as well: the staging copy costs
+    // HBM writes the link-bound kernel has room for, and the call takes what the direct transfer takes (4 MiB:
+    // 80 us) instead of a copy and then a kernel (93 us: a block this short costs the copy engines 10 us before
+    // its first byte). A block the device cannot address (pageable memory), or HFK_KNOB_FUSED_COPY_ENGINE, takes
+    // the copy and the kernel.
+    if (knob_value(HFK_KNOB_FUSED_COPY_ENGINE) == 0) {
+        void* mapped = nullptr;
+        if (hipHostGetDevicePointer(&mapped, const_cast<void*>(host_block), 0) == hipSuccess && mapped != nullptr) {
+            return launch_transpose(dev_layer_ptrs, mapped, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, 1,
+                                    workgroups, s, false, staging);
+        }
+        (void)hipGetLastError();
+    }
     hipError_t e = hipMemcpyAsync(staging, host_block, bytes, hipMemcpyHostToDevice, s);
     if (e != hipSuccess) return (int)e;
     return launch_transpose(dev_layer_ptrs, staging, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem_bytes, false, 0,

@@ -199,11 +199,12 @@ inline int plan_flat_gather(FlatGatherArgs<IdT>& a, FlatGatherPlan& p, uint64_t 
 
 // Geometry of the layout-converting transfer over a block table (pairs == nullptr:
 // the single block at the two base addresses). Returns HFK_OK with n_work == 0
-// when there is nothing to move.
+// when there is nothing to move. `mirror`: a second place that receives the packed blocks as they
+// are while a transfer out of the packed side reads them (TransposeArgs::mirror), or null.
 inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_layer_ptrs, const void* packed,
                           const int64_t* pairs, uint64_t n_pairs, uint64_t packed_stride, uint64_t layered_stride,
                           uint64_t packed_blocks, uint64_t layered_blocks, uint32_t T, uint32_t L, uint32_t H,
-                          uint32_t D, uint32_t elem_bytes, int unroll = kTransposeUnroll) {
+                          uint32_t D, uint32_t elem_bytes, int unroll = kTransposeUnroll, const void* mirror = nullptr) {
     a = TransposeArgs{};
     if (dev_layer_ptrs == nullptr || packed == nullptr) return HFK_ERR_NULL_POINTER;
     if (elem_bytes == 0) return HFK_ERR_BAD_SIZE;
@@ -217,7 +218,7 @@ inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_
     if (pairs != nullptr && (packed_stride < block_bytes || layered_stride < layer_block_bytes)) {
         return HFK_ERR_BAD_SIZE;
     }
-    uint64_t align = (uint64_t)(uintptr_t)packed | row_bytes;
+    uint64_t align = (uint64_t)(uintptr_t)packed | (uint64_t)(uintptr_t)mirror | row_bytes;
     if (pairs != nullptr) align |= packed_stride | layered_stride;
     const uint32_t unit = pick_unit(align);
     const uint64_t row_units = row_bytes / unit;
@@ -240,6 +241,7 @@ inline int plan_transpose(TransposeArgs& a, uint32_t* unit_out, const void* dev_
     a.row_units = (uint32_t)row_units;
     a.total_units = (uint32_t)total;
     a.n_work = (uint32_t)(chunks * n_pairs);
+    a.mirror = (uint64_t)(uintptr_t)mirror;
     *unit_out = unit;
     return HFK_OK;
 }

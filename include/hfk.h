@@ -113,13 +113,18 @@ HFK_API int hfk_multi_layer_block_transfer(const void* dev_layer_ptrs, const voi
                                    hfk_stream_t stream);
 
 /*
- * Staged variant: hipMemcpyAsync(staging <- host_block, whole block) on `stream`,
- * then the transfer above reading `staging`. Afterwards staging == host_block.
+ * Staged variant: afterwards staging == host_block and the layers hold what the transfer above gives.
+ * The reference copies the block into staging (a whole-block asynchronous copy) and runs its kernel on
+ * staging. Here a block in pinned, device-mapped host memory is read over the link once, by the kernel,
+ * which writes every unit to its layer and to staging (as fast as the direct transfer: a block of
+ * 4 MiB in 80 us, where a copy followed by a kernel takes 93); a block the device cannot address
+ * (pageable memory), or HFK_KNOB_FUSED_COPY_ENGINE, goes the reference's way, hipMemcpyAsync on `stream`
+ * and then the kernel. The bytes are the same either way.
  *
  * Replaces pcieThrough/csrc/host/multi_layer_block_transfer_torch.cpp:82-106
  * (`pciethrough::fused_memcpy_multi_layer_block_transfer`).
  *
- *   host_block  the host address of the pinned [T,L,H,D] block (not its mapped form)
+ *   host_block  the host address of the [T,L,H,D] block (not its mapped form)
  *   staging     device buffer of T*L*H*D*elem_bytes bytes
  */
 HFK_API int hfk_fused_memcpy_multi_layer_block_transfer(const void* dev_layer_ptrs,
@@ -477,9 +482,12 @@ enum hfk_knob {
     HFK_KNOB_TRANSFER_TILED = 18,   /* 1 (default): a block-table transfer into a packed pool in host memory goes through
                                        LDS tiles where its geometry allows (1 KiB runs on both sides); 0: always
                                        row by row                                                               */
-    HFK_KNOB_ADAPTIVE_PACE = 19     /* 1 (default): a paced throughput-mode swap-out (HFK_KNOB_THROUGHPUT_PACE_PERMILLE != 0)
+    HFK_KNOB_ADAPTIVE_PACE = 19,    /* 1 (default): a paced throughput-mode swap-out (HFK_KNOB_THROUGHPUT_PACE_PERMILLE != 0)
                                        takes its interval times a factor that the paced launches before it on this
                                        device have settled (see hfk_pace_state); 0: the interval as computed        */
+    HFK_KNOB_FUSED_COPY_ENGINE = 20 /* 0 (default): hfk_fused_memcpy_multi_layer_block_transfer reads a block in pinned
+                                       host memory once, by the kernel, which fills the staging buffer as well;
+                                       1: hipMemcpyAsync into staging, then the kernel, as for pageable memory     */
 };
 /*
  * The state behind a pace that is set between launches, for the current device: eight words,

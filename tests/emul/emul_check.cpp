@@ -638,16 +638,30 @@ void case_transpose(uint32_t T, uint32_t L, uint32_t H, uint32_t D, uint32_t ele
         lp.push_back((uint64_t)(uintptr_t)dst.back()->p);
         ep.push_back(exp.back()->p);
     }
+    // every other case also fills a second copy of the packed block while it reads it (the staged op's single
+    // kernel); its alignment alternates with the case, so that it takes part in the choice of the unit
+    static unsigned cases = 0;
+    const bool mirrored = cases++ % 2 == 1;
+    Buf mirror(block, mirrored && cases % 4 == 0 ? 4 : 0);
+    mirror.fill(0x5A);
     TransposeArgs a;
     uint32_t unit = 0;
-    int rc = plan_transpose(a, &unit, lp.data(), src.p, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem);
+    int rc = plan_transpose(a, &unit, lp.data(), src.p, nullptr, 1, 0, 0, 0, 0, T, L, H, D, elem, kTransposeUnroll,
+                            mirrored ? mirror.p : nullptr);
     if (rc != HFK_OK) { ++g_failures; std::printf("plan_transpose rc=%d\n", rc); }
     else walk_transpose<false>(a, unit, grid_cap);
     oracle_multi_layer_block_transfer(ep.data(), src.p, T, L, H, D, elem, 3);
     char what[128];
-    std::snprintf(what, sizeof what, "transpose T=%u L=%u H=%u D=%u elem=%u mis=%zu/%zu grid=%u unit=%u", T, L, H, D, elem,
-                  s_mis, l_mis, grid_cap, unit);
+    std::snprintf(what, sizeof what, "transpose T=%u L=%u H=%u D=%u elem=%u mis=%zu/%zu grid=%u unit=%u mirror=%d", T, L, H, D,
+                  elem, s_mis, l_mis, grid_cap, unit, (int)mirrored);
     for (uint32_t l = 0; l < L; ++l) expect_equal(dst[l]->p, exp[l]->p, layer, what);
+    if (mirrored) {
+        expect_equal(mirror.p, src.p, block, what);
+    } else {
+        Buf untouched(block);
+        untouched.fill(0x5A);
+        expect_equal(mirror.p, untouched.p, block, what);
+    }
     for (auto* b : dst) delete b;
     for (auto* b : exp) delete b;
 }

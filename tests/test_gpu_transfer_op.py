@@ -84,6 +84,38 @@ def test_multi_layer_block_kv_transfer(memory, block_size, layers, heads, head_d
             assert torch.equal(staging[slot].cpu(), host_blocks_cache[i])
 
 
+@pytest.mark.parametrize("how", ["one_kernel", "copy_engine", "pageable"])
+def test_fused_transfer_gives_the_same_bytes_either_way(memory, how):
+    """fused_memcpy_multi_layer_block_transfer reads a pinned block once, by the kernel, which fills the staging
+    buffer too; with HFK_KNOB_FUSED_COPY_ENGINE, and for a block in pageable memory, it copies into staging first
+    and runs the kernel on staging, as the reference does (multi_layer_block_transfer_torch.cpp:82-106). Layers and
+    staging hold the same bytes in all three cases, on a geometry with 16-byte units and on one with 4-byte units
+    and a staging buffer off the 16-byte grid."""
+    from heterofusedkernels_amd import capi
+    for (T, L, H, D, e, stage_off) in ((64, 6, 2, 128, 1, 0), (40, 3, 2, 10, 2, 0), (16, 2, 3, 64, 2, 4)):
+        announce("fused transfer %s: T=%d L=%d H=%d D=%d elem=%d staging offset %d" % (how, T, L, H, D, e, stage_off))
+        nbytes = T * L * H * D * e
+        data = torch.randint(-128, 128, (nbytes,), dtype=torch.int8, generator=torch.Generator().manual_seed(T + L + D))
+        if how == "pageable":
+            host = data.clone().view(T, L, H, D * e)
+            assert not host.is_pinned()
+        else:
+            pool = memory.alloc_numa_pinned_tensor(nbytes)
+            pool.copy_(data)
+            host = pool.view(torch.int8).view(T, L, H, D * e)
+        layers = torch.full((L, H, T, D * e), 0x55, dtype=torch.int8, device="cuda")
+        ptrs = torch.tensor([layers[l].data_ptr() for l in range(L)], dtype=torch.int64).cuda()
+        backing = torch.full((nbytes + 16,), 0x66, dtype=torch.int8, device="cuda")
+        staging = backing[stage_off:stage_off + nbytes].view(T, L, H, D * e)
+        with capi.thread_tuning({capi.KNOB_FUSED_COPY_ENGINE: 1 if how == "copy_engine" else 0}):
+            torch.ops.pcie_through.fused_memcpy_multi_layer_block_transfer(ptrs, host, staging, 4)
+        torch.cuda.synchronize()
+        assert torch.equal(staging.cpu(), host), "staging"
+        assert bool((backing[:stage_off] == 0x66).all()) and bool((backing[stage_off + nbytes:] == 0x66).all())
+        want = O.c_multi_layer_block_transfer(data.view(torch.uint8).numpy(), T, L, H, D, e, cores=3)
+        assert np.array_equal(layers.cpu().view(torch.uint8).numpy().reshape(L, -1), want), "layers"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.int8, torch.uint8,
                                    torch.float8_e4m3fn])
 def test_transfer_dtypes(memory, dtype):
