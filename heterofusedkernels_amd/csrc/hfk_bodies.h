@@ -654,8 +654,8 @@ struct TransposeArgs {
     uint32_t pace_q8;            // see Pacer; 0 = unpaced
     uint32_t tile_tokens;        // tiled form only (plan_transpose_tiles): tokens and packed rows per tile;
     uint32_t tile_rows;          // chunks_per_block is then the number of tiles per block
-    uint64_t mirror;             // 0, or (transfer out of the packed side only) the address of a second copy of the
-                                 // packed blocks, same strides: every unit read is also written there as it is
+    uint64_t mirror;             // 0, or (transfer out of the packed side, bodies built with MIRROR) the address of a
+                                 // second copy of the packed blocks, same strides: every unit read is also written there
 };
 
 // Where the body finds layer l's address. The layer differs from lane to lane (a 128-byte row is 8
@@ -749,8 +749,11 @@ HFK_HD void transpose_load(const TransposeArgs& a, const TransposeItem& it, cons
     }
 }
 
-template <typename V, int UNROLL, int NT, bool TO_PACKED>
+// MIRROR: every unit is also written, as it is, to the second copy of the packed blocks at a.mirror (a variant of
+// its own, so that the ordinary transfer carries none of it: a branch per unit cost its 24 x 2 launch 2 %).
+template <typename V, int UNROLL, int NT, bool TO_PACKED, bool MIRROR = false>
 HFK_HD void transpose_store(const TransposeArgs& a, const TransposeItem& it, const uint64_t (&layered_addr)[UNROLL], const V (&v)[UNROLL]) {
+    static_assert(!(MIRROR && TO_PACKED), "only a transfer out of the packed side can mirror what it reads");
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
         const uint64_t g64 = it.g0 + (uint64_t)u * kWorkgroupLanes;
@@ -766,7 +769,7 @@ HFK_HD void transpose_store(const TransposeArgs& a, const TransposeItem& it, con
                         d1[k] = unit_byte(v[u], k);
                     }
                 }
-                if (a.mirror != 0) {   // the packed block as it is, for the caller's staging buffer
+                if constexpr (MIRROR) {   // the packed block as it is, for the caller's staging buffer
                     store_unit<NT>(global_out<V>(a.mirror + (it.packed_addr - a.packed)) + g64, v[u]);
                 }
             }
@@ -774,7 +777,7 @@ HFK_HD void transpose_store(const TransposeArgs& a, const TransposeItem& it, con
     }
 }
 
-template <typename V, int UNROLL, int NT, bool TO_PACKED, typename LayerTable>
+template <typename V, int UNROLL, int NT, bool TO_PACKED, bool MIRROR = false, typename LayerTable>
 HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid, const LayerTable& layer_address) {
     constexpr uint32_t kChunkUnits = kWorkgroupLanes * UNROLL;
     Pacer pacer(a.pace_q8, bid, nb);
@@ -788,13 +791,13 @@ HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, ui
         uint64_t layered_addr[UNROLL];
         transpose_addresses<V, UNROLL>(a, it, layer_address, layered_addr);
         transpose_load<V, UNROLL, NT, TO_PACKED>(a, it, layered_addr, v);
-        transpose_store<V, UNROLL, NT, TO_PACKED>(a, it, layered_addr, v);
+        transpose_store<V, UNROLL, NT, TO_PACKED, MIRROR>(a, it, layered_addr, v);
     }
 }
 
-template <typename V, int UNROLL, int NT, bool TO_PACKED>
+template <typename V, int UNROLL, int NT, bool TO_PACKED, bool MIRROR = false>
 HFK_HD void transpose_body(const TransposeArgs& a, uint32_t bid, uint32_t nb, uint32_t tid) {
-    transpose_body<V, UNROLL, NT, TO_PACKED>(a, bid, nb, tid, LayerTableInMemory{a.layer_ptrs});
+    transpose_body<V, UNROLL, NT, TO_PACKED, MIRROR>(a, bid, nb, tid, LayerTableInMemory{a.layer_ptrs});
 }
 
 // ---------------------------------------------------------------------------

@@ -114,15 +114,16 @@ struct LayerTableInLds {
     __device__ uint64_t operator()(uint32_t l) const { return table[l]; }
 };
 
-template <typename V, int UNROLL, int NT, bool TO_PACKED>
+template <typename V, int UNROLL, int NT, bool TO_PACKED, bool MIRROR = false>
 __device__ void transpose_with_layer_table(const TransposeArgs& a) {
     __shared__ uint64_t layer_table[kLayerTableLdsEntries];
     if (a.L <= kLayerTableLdsEntries) {   // uniform over the grid
         for (uint32_t l = threadIdx.x; l < a.L; l += 256) layer_table[l] = hfk::table_entry(a.layer_ptrs, l);
         __syncthreads();
-        hfk::transpose_body<V, UNROLL, NT, TO_PACKED>(a, blockIdx.x, gridDim.x, threadIdx.x, LayerTableInLds{layer_table});
+        hfk::transpose_body<V, UNROLL, NT, TO_PACKED, MIRROR>(a, blockIdx.x, gridDim.x, threadIdx.x,
+                                                              LayerTableInLds{layer_table});
     } else {
-        hfk::transpose_body<V, UNROLL, NT, TO_PACKED>(a, blockIdx.x, gridDim.x, threadIdx.x);
+        hfk::transpose_body<V, UNROLL, NT, TO_PACKED, MIRROR>(a, blockIdx.x, gridDim.x, threadIdx.x);
     }
 }
 
@@ -130,6 +131,13 @@ __device__ void transpose_with_layer_table(const TransposeArgs& a) {
 template <typename V, int UNROLL, int NT>
 __global__ __launch_bounds__(256) void transpose_kernel(const TransposeArgs a) {
     transpose_with_layer_table<V, UNROLL, NT, false>(a);
+}
+
+// The same, also writing every unit it reads to a second copy of the packed blocks (a.mirror): the staged
+// single-block transfer in one kernel.
+template <typename V, int UNROLL, int NT>
+__global__ __launch_bounds__(256) void transpose_and_stage_kernel(const TransposeArgs a) {
+    transpose_with_layer_table<V, UNROLL, NT, false, true>(a);
 }
 
 // ... and back: per-layer caches -> packed blocks.
@@ -337,7 +345,12 @@ constexpr uint64_t kShortTransferBytes = 128ull << 20;
 constexpr uint32_t kShorterTransferToHostWorkgroups = 128;  // under 64 MiB
 constexpr uint64_t kShorterTransferBytes = 64ull << 20;
 constexpr uint32_t kTransferFromHostWorkgroups = 24;
+// One block out of host memory, 4 / 8 / 32 / 64 MiB. The rate over the grid is not smooth: the direct transfer gives
+// 53.2 / 55.3 / 57.0 / 57.3 GB/s on 32 workgroups (24: 0.3 below) and 50.2 / 52.2 / 53.8 / 54.2 on 48-56; the
+// variant that fills the staging buffer as well gives 52.9 / 55.0 / 56.9 / 57.2 on 64 (48-72 within 0.3) and
+// 49.1 / 52.1 / 54.4 / 55.0 on 24. Each sits in the middle of its plateau.
 constexpr uint32_t kSingleBlockTransferWorkgroups = 32;
+constexpr uint32_t kSingleBlockStagedTransferWorkgroups = 64;
 constexpr uint32_t kHostGatherWorkgroups = 64;
 constexpr uint64_t kLongHostGatherBytes = 4ull << 20;
 constexpr uint64_t kAskTableSideBytes = 64ull << 10;
@@ -676,8 +689,15 @@ int gather_rows_typed(const void* table, void* dst, const IdT* ids, uint64_t n_i
 // ---- transpose ------------------------------------------------------------
 template <typename V, int U, int NT>
 void launch_transpose_nt(const TransposeArgs& a, uint32_t grid, bool to_packed, hipStream_t s) {
-    if (to_packed) hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, NT>), dim3(grid), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((transpose_kernel<V, U, NT>), dim3(grid), dim3(256), 0, s, a);
+    if (to_packed) {
+        hipLaunchKernelGGL((transpose_to_packed_kernel<V, U, NT>), dim3(grid), dim3(256), 0, s, a);
+    } else if (a.mirror != 0) {
+        if constexpr (U == hfk::kTransposeUnroll) {   // the one shape the staged op launches
+            hipLaunchKernelGGL((transpose_and_stage_kernel<V, U, NT>), dim3(grid), dim3(256), 0, s, a);
+        }
+    } else {
+        hipLaunchKernelGGL((transpose_kernel<V, U, NT>), dim3(grid), dim3(256), 0, s, a);
+    }
 }
 
 template <typename V, int U>
@@ -772,7 +792,7 @@ int launch_transpose(const void* dev_layer_ptrs, const void* packed, const int64
     if (workgroups == 0 && side != 0) {
         // One block (the reference's op: 4-64 MiB, over in 0.1-1.2 ms) is sized for speed alone; a
         // block table may run for many milliseconds beside other kernels and gets the smaller grid.
-        workgroups = pairs == nullptr ? kSingleBlockTransferWorkgroups
+        workgroups = pairs == nullptr ? (mirror != nullptr ? kSingleBlockStagedTransferWorkgroups : kSingleBlockTransferWorkgroups)
                      : beside_compute ? kBesideTransferWorkgroups
                      : to_packed      ? transfer_to_host_workgroups((uint64_t)a.total_units * unit * n_pairs)
                                       : kTransferFromHostWorkgroups;

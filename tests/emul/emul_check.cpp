@@ -588,6 +588,14 @@ template <bool TO_PACKED, int UNROLL = kTransposeUnroll>
 void walk_transpose(const TransposeArgs& a, uint32_t unit, uint32_t grid_cap) {
     if (a.n_work == 0) return;
     const uint32_t grid = a.n_work < grid_cap ? a.n_work : grid_cap;
+    if constexpr (!TO_PACKED) {
+        if (a.mirror != 0) {   // the bodies the staged op's single kernel is built from
+            if (unit == 16u) walk(a, grid, transpose_body<vec16, UNROLL, 3, false, true>);
+            else if (unit == 4u) walk(a, grid, transpose_body<uint32_t, UNROLL, 0, false, true>);
+            else walk(a, grid, transpose_body<uint8_t, UNROLL, 0, false, true>);
+            return;
+        }
+    }
     if (unit == 16u) walk(a, grid, transpose_body<vec16, UNROLL, 3, TO_PACKED>);
     else if (unit == 4u) walk(a, grid, transpose_body<uint32_t, UNROLL, 0, TO_PACKED>);
     else walk(a, grid, transpose_body<uint8_t, UNROLL, 0, TO_PACKED>);
